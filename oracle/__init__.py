@@ -1,0 +1,180 @@
+"""ctypes front end of the CPU oracle (TEST INFRASTRUCTURE, not product code).
+
+Only tests, the smoke check and the CPU-baseline leg of the benchmark may import
+this package; the shipped library never does.  The arithmetic lives in
+``attention_ref.cc`` (a restatement of the reference's CPU attention,
+src/models/gpt.rs:139-144 and its autograd backward); this module only moves
+numpy arrays across the C boundary.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile liboracle.so with the Makefile next to this file."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.oracle_max_threads.restype = ctypes.c_int
+    return _lib
+
+
+def max_threads() -> int:
+    return int(lib().oracle_max_threads())
+
+
+_I64 = ctypes.c_int64
+
+
+def _suffix(dtype) -> str:
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return "f32"
+    if dtype == np.float64:
+        return "f64"
+    raise TypeError(f"oracle supports float32/float64 arrays, got {dtype}")
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def causal_mask(batch: int, tgt_len: int, seqlen_offset: int, dtype=np.float32) -> np.ndarray:
+    """Additive mask [batch,1,tgt,tgt+offset] (src/nn/functional.rs:12-55)."""
+    out = np.empty((batch, 1, tgt_len, tgt_len + seqlen_offset), dtype=dtype)
+    getattr(lib(), f"oracle_causal_mask_{_suffix(dtype)}")(
+        _I64(batch), _I64(tgt_len), _I64(seqlen_offset), _ptr(out))
+    return out
+
+
+def matmul(a: np.ndarray, b: np.ndarray, nthreads: int = 1) -> np.ndarray:
+    """Batched matmul of two equal-rank arrays; views (transposes) are passed by stride,
+    the way the reference's CPU backend consumes them (src/storage/cpu.rs:688-753)."""
+    assert a.dtype == b.dtype and a.ndim == b.ndim >= 2
+    suf = _suffix(a.dtype)
+    m, k = a.shape[-2:]
+    k2, n = b.shape[-2:]
+    assert k == k2 and a.shape[:-2] == b.shape[:-2]
+    batch_shape = a.shape[:-2]
+    batch = int(np.prod(batch_shape)) if batch_shape else 1
+    # Flatten the batch dims.  numpy keeps the last-two-dims strides when the batch
+    # dims collapse without a copy; otherwise it copies (same values, compact strides).
+    def prep(x):
+        if x.ndim == 2:
+            return x, 0
+        x3 = x.reshape((batch,) + x.shape[-2:])
+        return x3, x3.strides[0] // x3.itemsize
+    a3, a_bs = prep(a)
+    b3, b_bs = prep(b)
+    isz = a.itemsize
+    out = np.empty(batch_shape + (m, n), dtype=a.dtype)
+    getattr(lib(), f"oracle_matmul_{suf}")(
+        _ptr(a3), _I64(a_bs), _I64(a3.strides[-2] // isz), _I64(a3.strides[-1] // isz),
+        _ptr(b3), _I64(b_bs), _I64(b3.strides[-2] // isz), _I64(b3.strides[-1] // isz),
+        _ptr(out), _I64(batch), _I64(m), _I64(n), _I64(k), ctypes.c_int(nthreads))
+    return out
+
+
+def scalar_mul(x: np.ndarray, s: float) -> np.ndarray:
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    getattr(lib(), f"oracle_scalar_mul_{_suffix(x.dtype)}")(
+        _ptr(x), _I64(x.size), ctypes.c_double(s), _ptr(out))
+    return out
+
+
+def log_sum_exp(x: np.ndarray) -> np.ndarray:
+    """Row-wise log-sum-exp over the last axis (src/storage/cpu.rs:755-771)."""
+    x = np.ascontiguousarray(x)
+    cols = x.shape[-1]
+    rows = x.size // cols
+    out = np.empty(x.shape[:-1], dtype=x.dtype)
+    getattr(lib(), f"oracle_log_sum_exp_{_suffix(x.dtype)}")(
+        _ptr(x), _I64(rows), _I64(cols), _ptr(out))
+    return out
+
+
+def softmax(x: np.ndarray) -> np.ndarray:
+    """exp(x - lse(x)) over the last axis (src/tensor.rs:408-425, 456-458)."""
+    x = np.ascontiguousarray(x)
+    cols = x.shape[-1]
+    out = np.empty_like(x)
+    getattr(lib(), f"oracle_softmax_{_suffix(x.dtype)}")(
+        _ptr(x), _I64(x.size // cols), _I64(cols), _ptr(out))
+    return out
+
+
+def attn_fwd(q, k, v, scale: float | None = None, dtype=np.float32, nthreads: int = 0,
+             return_lse: bool = False, return_attn: bool = False, heads_per_call: int = 0):
+    """softmax(q k^T * scale + causal_mask) v for q [B,H,Tq,D], k,v [B,H,Tk,D].
+
+    Inputs are converted to ``dtype`` (float32 follows the reference's f32 path;
+    f16 configurations pass the f16-rounded values here).  ``scale`` defaults to
+    1/sqrt(D) computed in double (src/models/gpt.rs:139).  ``heads_per_call`` bounds
+    memory by evaluating that many batch entries at a time (0 = everything at
+    once, the way the reference materialises it).
+    """
+    q, k, v = _c(q, dtype), _c(k, dtype), _c(v, dtype)
+    B, H, tq, D = q.shape
+    tk = k.shape[2]
+    assert k.shape == (B, H, tk, D) and v.shape == (B, H, tk, D) and tk >= tq
+    if scale is None:
+        scale = 1.0 / np.sqrt(float(D))
+    y = np.empty((B, H, tq, D), dtype=dtype)
+    lse = np.empty((B, H, tq), dtype=dtype) if return_lse else None
+    attn = np.empty((B, H, tq, tk), dtype=dtype) if return_attn else None
+    fn = getattr(lib(), f"oracle_attn_fwd_{_suffix(dtype)}")
+    step = heads_per_call if heads_per_call > 0 else B
+    for b0 in range(0, B, step):
+        b1 = min(B, b0 + step)
+        fn(_ptr(q[b0:b1]), _ptr(k[b0:b1]), _ptr(v[b0:b1]), _I64(b1 - b0), _I64(H), _I64(tq),
+           _I64(tk), _I64(D), ctypes.c_double(scale), _ptr(y[b0:b1]),
+           _ptr(lse[b0:b1]) if lse is not None else None,
+           _ptr(attn[b0:b1]) if attn is not None else None, ctypes.c_int(nthreads))
+    res = (y,)
+    if return_lse:
+        res += (lse,)
+    if return_attn:
+        res += (attn,)
+    return res if len(res) > 1 else y
+
+
+def attn_bwd(q, k, v, dy, scale: float | None = None, dtype=np.float32, nthreads: int = 0,
+             heads_per_call: int = 0):
+    """Gradients (dq, dk, dv) of attn_fwd for upstream gradient dy [B,H,Tq,D]."""
+    q, k, v, dy = _c(q, dtype), _c(k, dtype), _c(v, dtype), _c(dy, dtype)
+    B, H, tq, D = q.shape
+    tk = k.shape[2]
+    if scale is None:
+        scale = 1.0 / np.sqrt(float(D))
+    dq, dk, dv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
+    fn = getattr(lib(), f"oracle_attn_bwd_{_suffix(dtype)}")
+    step = heads_per_call if heads_per_call > 0 else B
+    for b0 in range(0, B, step):
+        b1 = min(B, b0 + step)
+        fn(_ptr(q[b0:b1]), _ptr(k[b0:b1]), _ptr(v[b0:b1]), _ptr(dy[b0:b1]), _I64(b1 - b0),
+           _I64(H), _I64(tq), _I64(tk), _I64(D), ctypes.c_double(scale), _ptr(dq[b0:b1]),
+           _ptr(dk[b0:b1]), _ptr(dv[b0:b1]), ctypes.c_int(nthreads))
+    return dq, dk, dv

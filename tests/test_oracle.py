@@ -1,0 +1,220 @@
+"""Pins the CPU oracle (oracle/attention_ref.cc) before anything trusts it.
+
+Each check is chosen so a plausible slip (dropped term, wrong sign or index,
+transposed operand, off-by-one in the mask) fails at least one of them:
+literal vectors the reference's own tests hold, closed forms, brute force in
+float64, finite differences, structural invariants, and a library routine.
+"""
+import glob
+import math
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from deers_amd import synth
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+NINF = -np.inf
+
+
+# ---- literal vectors from the reference's tests ---------------------------------------------
+
+def test_causal_mask_literal():
+    # tests/nn.rs:193-219
+    m = oracle.causal_mask(2, 3, 0)
+    assert m.shape == (2, 1, 3, 3)
+    row = [0, NINF, NINF, 0, 0, NINF, 0, 0, 0]
+    assert m.ravel().tolist() == row + row
+
+
+def test_causal_mask_with_offset_literal():
+    # tests/nn.rs:221-232
+    m = oracle.causal_mask(1, 2, 3)
+    assert m.shape == (1, 1, 2, 5)
+    assert m.ravel().tolist() == [0, 0, 0, 0, NINF, 0, 0, 0, 0, 0]
+
+
+def test_decode_mask_row_is_all_zero():
+    assert not np.isinf(oracle.causal_mask(2, 1, 40)).any()
+
+
+def test_matmul_integer_products():
+    # tests/tensor.rs:83-110 inputs; the product of small integers is exact in f32.
+    a = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.float32)
+    b = np.array([[7, 8], [9, 10], [11, 12]], dtype=np.float32)
+    assert oracle.matmul(a, b).tolist() == [[58, 64], [139, 154]]
+
+
+def test_matmul_transposed_views_and_batches():
+    rng = np.random.default_rng(0)
+    a = rng.integers(-4, 5, size=(2, 3, 5, 7)).astype(np.float32)
+    b = rng.integers(-4, 5, size=(2, 3, 6, 7)).astype(np.float32)
+    got = oracle.matmul(a, b.transpose(0, 1, 3, 2), nthreads=3)      # rhs passed as a view
+    assert np.array_equal(got, np.einsum("bhik,bhjk->bhij", a, b))
+    got = oracle.matmul(a.transpose(0, 1, 3, 2), a)                   # lhs passed as a view
+    assert np.array_equal(got, np.einsum("bhki,bhkj->bhij", a, a))
+
+
+def test_scalar_mul_narrows_scalar_first():
+    # `v * self.0 as f32` (src/storage.rs:105-123): the f64 scale is rounded to f32 first.
+    x = np.array([3.0, -7.5, 1e-3], dtype=np.float32)
+    s = 1.0 / math.sqrt(32.0)
+    assert np.array_equal(oracle.scalar_mul(x, s), x * np.float32(s))
+
+
+def test_log_sum_exp_closed_form():
+    # input of tests/tensor.rs:1887
+    x = np.array([[1.0, 2.0, 3.0], [1.5, 0.5, -1.0]], dtype=np.float32)
+    want = [3 + math.log(1 + math.exp(-1) + math.exp(-2)),
+            1.5 + math.log(1 + math.exp(-1) + math.exp(-2.5))]
+    np.testing.assert_allclose(oracle.log_sum_exp(x), want, rtol=0, atol=2e-7)
+
+
+def test_softmax_closed_form_and_masked_row():
+    x = np.array([[1.0, 2.0, 3.0], [1.5, 0.5, -1.0], [0.25, NINF, NINF]], dtype=np.float32)
+    e = np.exp(x.astype(np.float64) - x.astype(np.float64).max(1, keepdims=True))
+    np.testing.assert_allclose(oracle.softmax(x), e / e.sum(1, keepdims=True), atol=1e-7)
+    assert oracle.softmax(x)[2].tolist() == [1.0, 0.0, 0.0]
+
+
+# ---- forward: brute force, invariants -----------------------------------------------------------
+
+def brute_force_fwd(q, k, v, scale):
+    """The definition, element by element in float64 (small shapes only)."""
+    B, H, tq, D = q.shape
+    tk = k.shape[2]
+    off = tk - tq
+    y = np.zeros((B, H, tq, D))
+    for b in range(B):
+        for h in range(H):
+            for i in range(tq):
+                w = [math.exp(scale * sum(float(q[b, h, i, d]) * float(k[b, h, j, d])
+                                          for d in range(D)))
+                     for j in range(i + off + 1)]
+                z = sum(w)
+                for d in range(D):
+                    y[b, h, i, d] = sum(w[j] * float(v[b, h, j, d]) for j in range(len(w))) / z
+    return y
+
+
+def rand(shape, seed):
+    return synth.normal(shape, seed)
+
+
+@pytest.mark.parametrize("tq,tk", [(7, 7), (3, 9), (1, 6)])
+def test_fwd_matches_brute_force(tq, tk):
+    q, k, v = rand((2, 2, tq, 4), 1), rand((2, 2, tk, 4), 2), rand((2, 2, tk, 4), 3)
+    want = brute_force_fwd(q, k, v, 0.5)
+    np.testing.assert_allclose(oracle.attn_fwd(q, k, v, dtype=np.float64), want, atol=1e-12)
+    np.testing.assert_allclose(oracle.attn_fwd(q, k, v), want, atol=2e-6)
+
+
+def test_fwd_invariants():
+    B, H, T, D = 2, 3, 19, 8
+    q, k, v = rand((B, H, T, D), 4), rand((B, H, T, D), 5), rand((B, H, T, D), 6)
+    y, lse, p = oracle.attn_fwd(q, k, v, return_lse=True, return_attn=True)
+    np.testing.assert_allclose(p.sum(-1), 1.0, atol=1e-6)            # rows are distributions
+    assert np.all(np.triu(p, 1) == 0)                                 # strictly-future weights are 0
+    np.testing.assert_array_equal(y[:, :, 0], v[:, :, 0])             # first token sees only itself
+    # causality: perturbing K/V after position t leaves y[..t] unchanged
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, 10:] += 3.0
+    v2[:, :, 10:] -= 2.0
+    np.testing.assert_array_equal(oracle.attn_fwd(q, k2, v2)[:, :, :10], y[:, :, :10])
+    # q = 0 -> uniform weights -> running mean of v
+    ym = oracle.attn_fwd(np.zeros_like(q), k, v, dtype=np.float64)
+    want = np.cumsum(v.astype(np.float64), 2) / np.arange(1, T + 1)[None, None, :, None]
+    np.testing.assert_allclose(ym, want, atol=1e-12)
+    # lse really is the log of the softmax denominator
+    s = np.einsum("bhid,bhjd->bhij", q, k).astype(np.float64) / math.sqrt(D)
+    s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+    np.testing.assert_allclose(lse, np.log(np.exp(s).sum(-1)), atol=2e-6)
+
+
+def test_default_scale_is_inverse_sqrt_d():
+    q, k, v = rand((1, 1, 5, 16), 7), rand((1, 1, 5, 16), 8), rand((1, 1, 5, 16), 9)
+    np.testing.assert_array_equal(oracle.attn_fwd(q, k, v), oracle.attn_fwd(q, k, v, scale=0.25))
+
+
+# ---- backward: finite differences, invariants ----------------------------------------------------
+
+@pytest.mark.parametrize("tq,tk", [(6, 6), (2, 5)])
+def test_bwd_matches_central_differences(tq, tk):
+    q, k, v = (rand((1, 2, t, 4), s).astype(np.float64) for t, s in ((tq, 11), (tk, 12), (tk, 13)))
+    do = rand((1, 2, tq, 4), 14).astype(np.float64)
+    dq, dk, dv = oracle.attn_bwd(q, k, v, do, dtype=np.float64)
+
+    def loss(q_, k_, v_):
+        return float((oracle.attn_fwd(q_, k_, v_, dtype=np.float64) * do).sum())
+
+    eps = 1e-6
+    for name, x, g in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        num = np.zeros_like(x)
+        for idx in np.ndindex(*x.shape):
+            xp, xm = x.copy(), x.copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            args_p = {"q": q, "k": k, "v": v, name: xp}
+            args_m = {"q": q, "k": k, "v": v, name: xm}
+            num[idx] = (loss(args_p["q"], args_p["k"], args_p["v"])
+                        - loss(args_m["q"], args_m["k"], args_m["v"])) / (2 * eps)
+        np.testing.assert_allclose(g, num, atol=1e-8, err_msg=name)
+
+
+def test_bwd_invariants():
+    B, H, T, D = 1, 2, 17, 8
+    q, k, v, do = (rand((B, H, T, D), s) for s in (21, 22, 23, 24))
+    dq, dk, dv = oracle.attn_bwd(q, k, v, do)
+    p = oracle.attn_fwd(q, k, v, return_attn=True)[1].astype(np.float64)
+    np.testing.assert_allclose(dv, np.einsum("bhij,bhid->bhjd", p, do), atol=2e-6)   # dV = P^T dO
+    # the last key/value is seen only by the last query
+    do2 = do.copy()
+    do2[:, :, :-1] = 0
+    dq2, dk2, dv2 = oracle.attn_bwd(q, k, v, do2)
+    np.testing.assert_allclose(dk2[:, :, -1], dk[:, :, -1], atol=1e-7)
+    np.testing.assert_allclose(dv2[:, :, -1], dv[:, :, -1], atol=1e-7)
+    assert np.all(dq2[:, :, :-1] == 0)
+    # the backward map is linear in dO
+    dq3, dk3, dv3 = oracle.attn_bwd(q, k, v, 2 * do)
+    np.testing.assert_allclose(dq3, 2 * dq, atol=1e-6)
+    np.testing.assert_allclose(dk3, 2 * dk, atol=1e-6)
+    # first query attends only to key 0: its softmax is constant 1, so dq[0] = 0
+    np.testing.assert_allclose(dq[:, :, 0], 0, atol=1e-7)
+    assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
+
+
+# ---- a library routine: torch SDPA + autograd, and the fixtures made from it -----------------
+
+def test_against_torch_sdpa_live():
+    torch = pytest.importorskip("torch")
+    B, H, T, D = 2, 3, 40, 16
+    q, k, v, do = (rand((B, H, T, D), s) for s in (31, 32, 33, 34))
+    qt, kt, vt = (torch.tensor(a, requires_grad=True) for a in (q, k, v))
+    y = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, is_causal=True)
+    y.backward(torch.tensor(do))
+    np.testing.assert_allclose(oracle.attn_fwd(q, k, v), y.detach().numpy(), atol=2e-6)
+    for got, want in zip(oracle.attn_bwd(q, k, v, do), (qt.grad, kt.grad, vt.grad)):
+        np.testing.assert_allclose(got, want.numpy(), atol=1e-5)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))),
+                         ids=lambda p: os.path.basename(p)[:-4])
+def test_against_golden_fixtures(path):
+    f = np.load(path)
+    q, k, v, do = f["q"], f["k"], f["v"], f["do"]
+    y, lse = oracle.attn_fwd(q, k, v, return_lse=True)
+    np.testing.assert_allclose(y, f["y"], atol=5e-6)
+    np.testing.assert_allclose(lse, f["lse"], atol=5e-6)
+    for got, name in zip(oracle.attn_bwd(q, k, v, do), ("dq", "dk", "dv")):
+        np.testing.assert_allclose(got, f[name], atol=2e-5, err_msg=name)
+
+
+def test_fixture_inputs_regenerate_from_seed():
+    f = np.load(os.path.join(GOLDEN, "f16_b2h3t33d64.npz"))
+    B, H, T, D, L, seed, ver = f["header"].tolist()
+    assert ver == synth.GENERATOR_VERSION
+    x = synth.attention_inputs("f16_b2h3t33d64", B, H, T, D, np.float16, base_seed=seed)
+    for name in ("q", "k", "v", "do"):
+        np.testing.assert_array_equal(x[name], f[name])
