@@ -1,0 +1,159 @@
+// Decode attention: one query row per (b,h) against a KV cache of L rows, f16.
+//
+// Same math as the forward with tgt_len = 1 and seqlen_offset = L-1, where the
+// causal mask row is all zero (src/nn/functional.rs:26,42).  1 FLOP per byte:
+// the kernel is an HBM stream, so the design is about bytes in flight, not
+// matrix cores.
+//
+//   grid = (splits, B*H).  A workgroup streams `chunk` cache rows of one head.
+//   A row of D halfs is covered by LPR = D/8 lanes with one 16-byte load each,
+//   so a wave reads 1 KiB of K and 1 KiB of V per load instruction, fully
+//   coalesced.  ROWS_PER_IT rows are in flight per lane group (K and V loads
+//   are issued together: V does not wait for the scores).
+//   Each lane group keeps a private online softmax (m, l, o[8] per lane) over
+//   the rows it visits; groups are merged once at the end through LDS in a
+//   fixed order, and the split partial (m, l, o[D]) goes to the workspace.
+//   A second tiny kernel merges the splits and writes f16 output.
+#include "common.h"
+
+namespace deers {
+
+constexpr int kDecRowsPerIt = 4;
+
+int decode_pick_splits(int64_t BH, int64_t L, int* chunk) {
+  int splits = 1;
+  while (BH * splits < 2048 && L / (splits * 2) >= 256) splits *= 2;
+  int64_t c = (L + splits - 1) / splits;
+  c = (c + 63) / 64 * 64;
+  *chunk = (int)c;
+  return splits;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
+  constexpr int LPR = D / 8;        // lanes per cache row
+  constexpr int GROUPS = 256 / LPR; // row groups per workgroup
+  __shared__ float red_m[GROUPS];
+  __shared__ float red_l[GROUPS];
+  __shared__ float red_o[GROUPS * D];
+
+  const int tid = threadIdx.x;
+  const int part = tid % LPR;
+  const int grp = tid / LPR;
+  const int split = blockIdx.x;
+  const int bh = blockIdx.y;
+  const int b = bh / p.H, h = bh % p.H;
+
+  const half_t* K = (const half_t*)p.k + b * p.skb + h * p.skh + 8 * part;
+  const half_t* V = (const half_t*)p.v + b * p.skb + h * p.skh + 8 * part;
+  const half8 qh = *(const half8*)((const half_t*)p.q + (int64_t)bh * D + 8 * part);
+  float qf[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) qf[e] = (float)qh[e] * p.scale_log2;
+
+  const int row_begin = split * p.chunk;
+  int row_end = row_begin + p.chunk;
+  if (row_end > p.L) row_end = p.L;
+
+  float m = -INFINITY, l = 0.f;
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = 0.f;
+
+  for (int r0 = row_begin + grp; r0 < row_end; r0 += GROUPS * kDecRowsPerIt) {
+    half8 kk[kDecRowsPerIt], vv[kDecRowsPerIt];
+#pragma unroll
+    for (int u = 0; u < kDecRowsPerIt; ++u) {
+      const int row = r0 + u * GROUPS;
+      if (row < row_end) {
+        kk[u] = *(const half8*)(K + (int64_t)row * p.skl);
+        vv[u] = *(const half8*)(V + (int64_t)row * p.skl);
+      } else {
+        kk[u] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        vv[u] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+    float s[kDecRowsPerIt];
+#pragma unroll
+    for (int u = 0; u < kDecRowsPerIt; ++u) {
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += qf[e] * (float)kk[u][e];
+#pragma unroll
+      for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+      s[u] = (r0 + u * GROUPS < row_end) ? acc : -INFINITY;
+    }
+    float mloc = s[0];
+#pragma unroll
+    for (int u = 1; u < kDecRowsPerIt; ++u) mloc = fmaxf(mloc, s[u]);
+    const float m_new = fmaxf(m, mloc);  // finite: row r0 itself is always valid
+    const float alpha = fast_exp2(m - m_new);
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] *= alpha;
+#pragma unroll
+    for (int u = 0; u < kDecRowsPerIt; ++u) {
+      const float pu = fast_exp2(s[u] - m_new);
+      l += pu;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] += pu * (float)vv[u][e];
+    }
+    m = m_new;
+  }
+
+  // ---- merge the row groups of this workgroup (fixed order) ----
+  if (part == 0) {
+    red_m[grp] = m;
+    red_l[grp] = l;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red_o[grp * D + 8 * part + e] = o[e];
+  __syncthreads();
+  if (tid < D) {
+    float M = -INFINITY;
+    for (int gi = 0; gi < GROUPS; ++gi) M = fmaxf(M, red_m[gi]);
+    float lsum = 0.f, osum = 0.f;
+    for (int gi = 0; gi < GROUPS; ++gi) {
+      const float mg = red_m[gi];
+      const float w = (mg == -INFINITY) ? 0.f : fast_exp2(mg - M);
+      lsum += w * red_l[gi];
+      osum += w * red_o[gi * D + tid];
+    }
+    const int64_t slot = (int64_t)bh * p.splits + split;
+    p.part_o[slot * D + tid] = osum;
+    if (tid == 0) {
+      p.part_ml[slot * 2 + 0] = M;
+      p.part_ml[slot * 2 + 1] = lsum;
+    }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(D) void attn_decode_merge_kernel(DecodeParams p) {
+  const int bh = blockIdx.x;
+  const int d = threadIdx.x;
+  float M = -INFINITY;
+  for (int s = 0; s < p.splits; ++s) M = fmaxf(M, p.part_ml[((int64_t)bh * p.splits + s) * 2]);
+  float lsum = 0.f, osum = 0.f;
+  for (int s = 0; s < p.splits; ++s) {
+    const int64_t slot = (int64_t)bh * p.splits + s;
+    const float ms = p.part_ml[slot * 2];
+    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);
+    lsum += w * p.part_ml[slot * 2 + 1];
+    osum += w * p.part_o[slot * D + d];
+  }
+  ((half_t*)p.o)[(int64_t)bh * D + d] = (half_t)(osum / lsum);
+}
+
+void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream) {
+  dim3 grid(p.splits, B * p.H);
+  if (D == 64) {
+    hipLaunchKernelGGL(attn_decode_f16_kernel<64>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(B * p.H), dim3(64), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL(attn_decode_f16_kernel<128>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(B * p.H), dim3(128), 0, stream, p);
+  }
+}
+
+}  // namespace deers

@@ -1,0 +1,381 @@
+// Host side of the C ABI declared in include/deers_rocm.h: the process-global
+// runtime (device, stream, workspace), memory and timer calls, and the argument
+// checks in front of every kernel launch.  The shape of the runtime follows what
+// the reference's CUDA backend keeps in its OnceLock (one context, one stream,
+// device ordinal fixed at init: src/storage/cuda.rs:462-528).
+#include "../../include/deers_rocm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+#include <string>
+
+#include "common.h"
+
+namespace deers {
+void launch_attn_fwd_f16(const FwdParams& p, int B, int D, hipStream_t stream);
+void launch_attn_fwd_f32(const FwdParams& p, int B, int D, hipStream_t stream);
+void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream);
+void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream);
+void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream);
+int decode_pick_splits(int64_t BH, int64_t L, int* chunk);
+}  // namespace deers
+
+namespace {
+
+struct Runtime {
+  bool ready = false;
+  int ordinal = -1;
+  hipStream_t stream = nullptr;
+  void* workspace = nullptr;  // grows on demand, freed never (process lifetime)
+  size_t workspace_bytes = 0;
+};
+
+Runtime g_rt;
+std::mutex g_mu;
+thread_local std::string t_err;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  t_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess)                                                               \
+      return fail(DEERS_ROCM_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));   \
+  } while (0)
+
+#define NEED_INIT()                                                                     \
+  do {                                                                                  \
+    if (!g_rt.ready)                                                                    \
+      return fail(DEERS_ROCM_ERR_NOT_INIT, "deers_rocm_init has not been called");      \
+  } while (0)
+
+bool device_is_gfx950(int ordinal) {
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, ordinal) != hipSuccess) return false;
+  return std::string(prop.gcnArchName).rfind("gfx950", 0) == 0;
+}
+
+// Workspace that only grows; callers hold g_mu.
+int workspace(size_t bytes, void** out) {
+  if (bytes > g_rt.workspace_bytes) {
+    if (g_rt.workspace) {
+      HIP_TRY(hipStreamSynchronize(g_rt.stream));
+      HIP_TRY(hipFree(g_rt.workspace));
+      g_rt.workspace = nullptr;
+      g_rt.workspace_bytes = 0;
+    }
+    const size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    HIP_TRY(hipMalloc(&g_rt.workspace, want));
+    g_rt.workspace_bytes = want;
+  }
+  *out = g_rt.workspace;
+  return DEERS_ROCM_OK;
+}
+
+// Resolves a [B,H,T,D] stride argument (NULL = compact) and checks what the
+// kernels assume: unit D stride and 16-byte aligned rows.
+int resolve_strides(const char* name, const void* ptr, const int64_t* strides, int64_t H,
+                    int64_t T, int64_t D, size_t elem, deers::Strides3* out) {
+  if (!ptr) return fail(DEERS_ROCM_ERR_ARG, "%s: null pointer", name);
+  int64_t sb = H * T * D, sh = T * D, st = D, sd = 1;
+  if (strides) {
+    sb = strides[0];
+    sh = strides[1];
+    st = strides[2];
+    sd = strides[3];
+  }
+  if (sd != 1)
+    return fail(DEERS_ROCM_ERR_LAYOUT,
+                "%s: innermost stride is %lld, the kernels need 1 (compact the tensor first)",
+                name, (long long)sd);
+  const int64_t per16 = 16 / (int64_t)elem;
+  if (sb % per16 || sh % per16 || st % per16 || (reinterpret_cast<uintptr_t>(ptr) & 15))
+    return fail(DEERS_ROCM_ERR_LAYOUT,
+                "%s: rows must be 16-byte aligned (ptr %p, strides %lld,%lld,%lld)", name, ptr,
+                (long long)sb, (long long)sh, (long long)st);
+  out->b = sb;
+  out->h = sh;
+  out->t = st;
+  return DEERS_ROCM_OK;
+}
+
+int check_problem(int dtype, int64_t B, int64_t H, int64_t T, int64_t D) {
+  if (dtype != DEERS_ROCM_F16 && dtype != DEERS_ROCM_F32)
+    return fail(DEERS_ROCM_ERR_ARG, "dtype %d is neither DEERS_ROCM_F16 nor DEERS_ROCM_F32", dtype);
+  if (B < 1 || H < 1 || T < 1)
+    return fail(DEERS_ROCM_ERR_ARG, "B, H, T must be >= 1 (got %lld, %lld, %lld)", (long long)B,
+                (long long)H, (long long)T);
+  if (D != 32 && D != 64 && D != 128)
+    return fail(DEERS_ROCM_ERR_ARG, "head dim %lld unsupported (32, 64 or 128)", (long long)D);
+  if (B * H > 65535 || T > (int64_t(1) << 24))
+    return fail(DEERS_ROCM_ERR_ARG, "B*H must be <= 65535 and T <= 2^24");
+  return DEERS_ROCM_OK;
+}
+
+struct Timer {
+  hipEvent_t start, stop;
+};
+
+}  // namespace
+
+extern "C" {
+
+int deers_rocm_available(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (g_rt.ready) return 1;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n < 1) return 0;
+  return device_is_gfx950(0) ? 1 : 0;
+}
+
+int deers_rocm_init(int ordinal) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (g_rt.ready) {
+    if (g_rt.ordinal == ordinal) return DEERS_ROCM_OK;
+    return fail(DEERS_ROCM_ERR_ARG, "runtime already initialised on device %d", g_rt.ordinal);
+  }
+  int n = 0;
+  HIP_TRY(hipGetDeviceCount(&n));
+  if (ordinal < 0 || ordinal >= n)
+    return fail(DEERS_ROCM_ERR_ARG, "device ordinal %d out of range (%d devices)", ordinal, n);
+  if (!device_is_gfx950(ordinal))
+    return fail(DEERS_ROCM_ERR_ARG, "device %d is not gfx950; this library targets MI355X only",
+                ordinal);
+  HIP_TRY(hipSetDevice(ordinal));
+  HIP_TRY(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
+  g_rt.ordinal = ordinal;
+  g_rt.ready = true;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_sync(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+const char* deers_rocm_last_error(void) { return t_err.c_str(); }
+
+void* deers_rocm_stream(void) { return g_rt.ready ? (void*)g_rt.stream : nullptr; }
+
+int deers_rocm_alloc(size_t bytes, void** out_ptr) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!out_ptr) return fail(DEERS_ROCM_ERR_ARG, "alloc: null out_ptr");
+  *out_ptr = nullptr;
+  if (bytes == 0) return DEERS_ROCM_OK;
+  HIP_TRY(hipSetDevice(g_rt.ordinal));
+  HIP_TRY(hipMalloc(out_ptr, bytes));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_alloc_zeros(size_t bytes, void** out_ptr) {
+  int rc = deers_rocm_alloc(bytes, out_ptr);
+  if (rc != DEERS_ROCM_OK || bytes == 0) return rc;
+  std::lock_guard<std::mutex> lock(g_mu);
+  HIP_TRY(hipMemsetAsync(*out_ptr, 0, bytes, g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_free(void* ptr) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!ptr) return DEERS_ROCM_OK;
+  // Work already enqueued may still read the buffer.
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  HIP_TRY(hipFree(ptr));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_htod(void* dst_device, const void* src_host, size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (bytes == 0) return DEERS_ROCM_OK;
+  if (!dst_device || !src_host) return fail(DEERS_ROCM_ERR_ARG, "htod: null pointer");
+  HIP_TRY(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));  // pageable source: safe to reuse on return
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_dtoh(void* dst_host, const void* src_device, size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (bytes == 0) return DEERS_ROCM_OK;
+  if (!dst_host || !src_device) return fail(DEERS_ROCM_ERR_ARG, "dtoh: null pointer");
+  HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_dtod(void* dst_device, const void* src_device, size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (bytes == 0) return DEERS_ROCM_OK;
+  if (!dst_device || !src_device) return fail(DEERS_ROCM_ERR_ARG, "dtod: null pointer");
+  HIP_TRY(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_timer_create(void** out_timer) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!out_timer) return fail(DEERS_ROCM_ERR_ARG, "timer_create: null out_timer");
+  Timer* t = new Timer;
+  hipError_t e = hipEventCreate(&t->start);
+  if (e == hipSuccess) e = hipEventCreate(&t->stop);
+  if (e != hipSuccess) {
+    delete t;
+    return fail(DEERS_ROCM_ERR_HIP, "hipEventCreate failed: %s", hipGetErrorString(e));
+  }
+  *out_timer = t;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_timer_start(void* timer) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!timer) return fail(DEERS_ROCM_ERR_ARG, "timer_start: null timer");
+  HIP_TRY(hipEventRecord(static_cast<Timer*>(timer)->start, g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_timer_stop(void* timer) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!timer) return fail(DEERS_ROCM_ERR_ARG, "timer_stop: null timer");
+  HIP_TRY(hipEventRecord(static_cast<Timer*>(timer)->stop, g_rt.stream));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_timer_elapsed_ms(void* timer, float* out_ms) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!timer || !out_ms) return fail(DEERS_ROCM_ERR_ARG, "timer_elapsed_ms: null argument");
+  Timer* t = static_cast<Timer*>(timer);
+  HIP_TRY(hipEventSynchronize(t->stop));
+  HIP_TRY(hipEventElapsedTime(out_ms, t->start, t->stop));
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_timer_destroy(void* timer) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!timer) return DEERS_ROCM_OK;
+  Timer* t = static_cast<Timer*>(timer);
+  hipEventDestroy(t->start);
+  hipEventDestroy(t->stop);
+  delete t;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_attn_fwd(int dtype, const void* q, const int64_t* q_strides, const void* k,
+                        const int64_t* k_strides, const void* v, const int64_t* v_strides,
+                        void* o, const int64_t* o_strides, float* lse, int64_t B, int64_t H,
+                        int64_t T, int64_t D, float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_problem(dtype, B, H, T, D)) return rc;
+  if (!lse) return fail(DEERS_ROCM_ERR_ARG, "attn_fwd: null lse");
+  const size_t elem = dtype == DEERS_ROCM_F16 ? 2 : 4;
+  deers::FwdParams p{};
+  if (int rc = resolve_strides("q", q, q_strides, H, T, D, elem, &p.sq)) return rc;
+  if (int rc = resolve_strides("k", k, k_strides, H, T, D, elem, &p.sk)) return rc;
+  if (int rc = resolve_strides("v", v, v_strides, H, T, D, elem, &p.sv)) return rc;
+  if (int rc = resolve_strides("o", o, o_strides, H, T, D, elem, &p.so)) return rc;
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
+  p.H = (int)H; p.T = (int)T;
+  p.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  if (dtype == DEERS_ROCM_F16)
+    deers::launch_attn_fwd_f16(p, (int)B, (int)D, g_rt.stream);
+  else
+    deers::launch_attn_fwd_f32(p, (int)B, (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, const void* k,
+                        const int64_t* k_strides, const void* v, const int64_t* v_strides,
+                        const void* o, const int64_t* o_strides, const float* lse,
+                        const void* d_o, const int64_t* do_strides, void* dq,
+                        const int64_t* dq_strides, void* dk, const int64_t* dk_strides, void* dv,
+                        const int64_t* dv_strides, int64_t B, int64_t H, int64_t T, int64_t D,
+                        float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_problem(dtype, B, H, T, D)) return rc;
+  if (!lse) return fail(DEERS_ROCM_ERR_ARG, "attn_bwd: null lse");
+  const size_t elem = dtype == DEERS_ROCM_F16 ? 2 : 4;
+  deers::BwdParams p{};
+  if (int rc = resolve_strides("q", q, q_strides, H, T, D, elem, &p.sq)) return rc;
+  if (int rc = resolve_strides("k", k, k_strides, H, T, D, elem, &p.sk)) return rc;
+  if (int rc = resolve_strides("v", v, v_strides, H, T, D, elem, &p.sv)) return rc;
+  if (int rc = resolve_strides("o", o, o_strides, H, T, D, elem, &p.so)) return rc;
+  if (int rc = resolve_strides("d_o", d_o, do_strides, H, T, D, elem, &p.sdo)) return rc;
+  if (int rc = resolve_strides("dq", dq, dq_strides, H, T, D, elem, &p.sdq)) return rc;
+  if (int rc = resolve_strides("dk", dk, dk_strides, H, T, D, elem, &p.sdk)) return rc;
+  if (int rc = resolve_strides("dv", dv, dv_strides, H, T, D, elem, &p.sdv)) return rc;
+  void* ws = nullptr;
+  if (int rc = workspace((size_t)(B * H * T) * sizeof(float), &ws)) return rc;
+  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
+  p.delta = static_cast<float*>(ws);
+  p.dq = dq; p.dk = dk; p.dv = dv;
+  p.H = (int)H; p.T = (int)T;
+  p.scale = scale;
+  p.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  if (dtype == DEERS_ROCM_F16)
+    deers::launch_attn_bwd_f16(p, (int)B, (int)D, g_rt.stream);
+  else
+    deers::launch_attn_bwd_f32(p, (int)B, (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                           const int64_t* kv_strides, void* o, int64_t B, int64_t H, int64_t L,
+                           int64_t D, float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (dtype != DEERS_ROCM_F16)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: only DEERS_ROCM_F16 caches are supported");
+  if (B < 1 || H < 1 || L < 1 || B * H > 65535 || L > (int64_t(1) << 30))
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: need B,H,L >= 1, B*H <= 65535, L <= 2^30");
+  if (D != 64 && D != 128)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: head dim %lld unsupported (64 or 128)",
+                (long long)D);
+  if (!q || !k_cache || !v_cache || !o) return fail(DEERS_ROCM_ERR_ARG, "attn_decode: null pointer");
+  deers::DecodeParams p{};
+  p.skb = H * L * D; p.skh = L * D; p.skl = D;
+  if (kv_strides) { p.skb = kv_strides[0]; p.skh = kv_strides[1]; p.skl = kv_strides[2]; }
+  if (p.skb % 8 || p.skh % 8 || p.skl % 8 || (reinterpret_cast<uintptr_t>(k_cache) & 15) ||
+      (reinterpret_cast<uintptr_t>(v_cache) & 15) || (reinterpret_cast<uintptr_t>(q) & 15) ||
+      (reinterpret_cast<uintptr_t>(o) & 15))
+    return fail(DEERS_ROCM_ERR_LAYOUT, "attn_decode: cache rows, q and o must be 16-byte aligned");
+  int chunk = 0;
+  const int splits = deers::decode_pick_splits(B * H, L, &chunk);
+  void* ws = nullptr;
+  const size_t part_o = (size_t)(B * H) * splits * D * sizeof(float);
+  const size_t part_ml = (size_t)(B * H) * splits * 2 * sizeof(float);
+  if (int rc = workspace(part_o + part_ml, &ws)) return rc;
+  p.q = q; p.k = k_cache; p.v = v_cache; p.o = o;
+  p.part_o = static_cast<float*>(ws);
+  p.part_ml = reinterpret_cast<float*>(static_cast<char*>(ws) + part_o);
+  p.H = (int)H; p.L = (int)L; p.splits = splits; p.chunk = chunk;
+  p.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  deers::launch_attn_decode_f16(p, (int)B, (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,212 @@
+"""Python binding of the C ABI in include/deers_rocm.h (ctypes, no torch).
+
+This is host-side plumbing for tests and the benchmark: device buffers, copies,
+timers and the three attention entry points, called exactly the way a
+`Device::Rocm` storage backend in deers would call them over `extern "C"`.
+There is no CPU fallback: if the HIP library is missing or no gfx950 device is
+present, every call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+F16, F32 = 0, 1
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdeers_rocm.so")
+
+_lib = None
+_inited = False
+
+
+class RocmError(RuntimeError):
+    """A non-zero return code from the library (the role of deers' backend error variant)."""
+
+
+def load() -> ctypes.CDLL:
+    """Loads libdeers_rocm.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RocmError(
+                f"{LIB_PATH} is missing: build it with `make -C deers_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback path")
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.deers_rocm_last_error.restype = ctypes.c_char_p
+        lib.deers_rocm_stream.restype = ctypes.c_void_p
+        _lib = lib
+    return _lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise RocmError(f"deers_rocm error {rc}: {load().deers_rocm_last_error().decode()}")
+
+
+def available() -> bool:
+    return bool(load().deers_rocm_available())
+
+
+def init(ordinal: int = 0):
+    global _inited
+    if not _inited:
+        _check(load().deers_rocm_init(ctypes.c_int(ordinal)))
+        _inited = True
+
+
+def sync():
+    _check(load().deers_rocm_sync())
+
+
+def dtype_code(dtype) -> int:
+    dtype = np.dtype(dtype)
+    if dtype == np.float16:
+        return F16
+    if dtype == np.float32:
+        return F32
+    raise TypeError(f"unsupported dtype {dtype}")
+
+
+class DeviceBuffer:
+    """An owned device allocation with a shape and dtype (compact row-major)."""
+
+    def __init__(self, shape, dtype, zeros: bool = False):
+        init()
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        ptr = ctypes.c_void_p()
+        fn = load().deers_rocm_alloc_zeros if zeros else load().deers_rocm_alloc
+        _check(fn(ctypes.c_size_t(self.nbytes), ctypes.byref(ptr)))
+        self.ptr = ptr
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        buf = cls(a.shape, a.dtype)
+        _check(load().deers_rocm_htod(buf.ptr, a.ctypes.data_as(ctypes.c_void_p),
+                                      ctypes.c_size_t(buf.nbytes)))
+        return buf
+
+    def numpy(self) -> np.ndarray:
+        out = np.empty(self.shape, dtype=self.dtype)
+        _check(load().deers_rocm_dtoh(out.ctypes.data_as(ctypes.c_void_p), self.ptr,
+                                      ctypes.c_size_t(self.nbytes)))
+        return out
+
+    def free(self):
+        if self.ptr is not None and self.ptr.value:
+            _check(load().deers_rocm_free(self.ptr))
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Timer:
+    """hipEvent pair on the library stream."""
+
+    def __init__(self):
+        init()
+        self.h = ctypes.c_void_p()
+        _check(load().deers_rocm_timer_create(ctypes.byref(self.h)))
+
+    def start(self):
+        _check(load().deers_rocm_timer_start(self.h))
+
+    def stop(self):
+        _check(load().deers_rocm_timer_stop(self.h))
+
+    def elapsed_ms(self) -> float:
+        ms = ctypes.c_float()
+        _check(load().deers_rocm_timer_elapsed_ms(self.h, ctypes.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            load().deers_rocm_timer_destroy(self.h)
+        except Exception:
+            pass
+
+
+def _strides(s):
+    if s is None:
+        return None
+    return (ctypes.c_int64 * 4)(*[int(x) for x in s])
+
+
+def attn_fwd_raw(dtype, q, k, v, o, lse, B, H, T, D, scale, q_strides=None, k_strides=None,
+                 v_strides=None, o_strides=None):
+    """deers_rocm_attn_fwd on raw device pointers (DeviceBuffer.ptr)."""
+    _check(load().deers_rocm_attn_fwd(
+        ctypes.c_int(dtype_code(dtype)), q, _strides(q_strides), k, _strides(k_strides), v,
+        _strides(v_strides), o, _strides(o_strides), lse, ctypes.c_int64(B), ctypes.c_int64(H),
+        ctypes.c_int64(T), ctypes.c_int64(D), ctypes.c_float(scale)))
+
+
+def attn_bwd_raw(dtype, q, k, v, o, lse, do, dq, dk, dv, B, H, T, D, scale, strides=None):
+    """deers_rocm_attn_bwd on raw device pointers; `strides` maps tensor name -> 4 strides."""
+    s = strides or {}
+    g = lambda n: _strides(s.get(n))  # noqa: E731
+    _check(load().deers_rocm_attn_bwd(
+        ctypes.c_int(dtype_code(dtype)), q, g("q"), k, g("k"), v, g("v"), o, g("o"), lse, do,
+        g("do"), dq, g("dq"), dk, g("dk"), dv, g("dv"), ctypes.c_int64(B), ctypes.c_int64(H),
+        ctypes.c_int64(T), ctypes.c_int64(D), ctypes.c_float(scale)))
+
+
+def attn_decode_raw(dtype, q, k_cache, v_cache, o, B, H, L, D, scale, kv_strides=None):
+    ks = None if kv_strides is None else (ctypes.c_int64 * 3)(*[int(x) for x in kv_strides])
+    _check(load().deers_rocm_attn_decode(
+        ctypes.c_int(dtype_code(dtype)), q, k_cache, v_cache, ks, o, ctypes.c_int64(B),
+        ctypes.c_int64(H), ctypes.c_int64(L), ctypes.c_int64(D), ctypes.c_float(scale)))
+
+
+def default_scale(D: int) -> float:
+    """1/sqrt(D) in double, narrowed to f32 (src/models/gpt.rs:139, src/storage.rs:115-117)."""
+    return float(np.float32(1.0 / np.sqrt(float(D))))
+
+
+# ---- numpy-in / numpy-out conveniences (copy to the device, run, copy back) ----
+
+def attn_fwd(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float | None = None):
+    """Returns (o, lse) for compact [B,H,T,D] numpy inputs of one dtype (f16 or f32)."""
+    B, H, T, D = q.shape
+    scale = default_scale(D) if scale is None else scale
+    dq_, dk_, dv_ = (DeviceBuffer.from_numpy(a) for a in (q, k, v))
+    o = DeviceBuffer(q.shape, q.dtype)
+    lse = DeviceBuffer((B, H, T), np.float32)
+    attn_fwd_raw(q.dtype, dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, B, H, T, D, scale)
+    return o.numpy(), lse.numpy()
+
+
+def attn_fwd_bwd(q, k, v, do, scale: float | None = None):
+    """Returns (o, lse, dq, dk, dv): forward then backward through the C ABI."""
+    B, H, T, D = q.shape
+    scale = default_scale(D) if scale is None else scale
+    bq, bk, bv, bdo = (DeviceBuffer.from_numpy(a) for a in (q, k, v, do))
+    o = DeviceBuffer(q.shape, q.dtype)
+    lse = DeviceBuffer((B, H, T), np.float32)
+    gq, gk, gv = (DeviceBuffer(q.shape, q.dtype) for _ in range(3))
+    attn_fwd_raw(q.dtype, bq.ptr, bk.ptr, bv.ptr, o.ptr, lse.ptr, B, H, T, D, scale)
+    attn_bwd_raw(q.dtype, bq.ptr, bk.ptr, bv.ptr, o.ptr, lse.ptr, bdo.ptr, gq.ptr, gk.ptr, gv.ptr,
+                 B, H, T, D, scale)
+    return o.numpy(), lse.numpy(), gq.numpy(), gk.numpy(), gv.numpy()
+
+
+def attn_decode(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray,
+                scale: float | None = None, length: int | None = None):
+    """q [B,H,D], caches [B,H,Lcap,D] (f16); attends to the first `length` cache rows."""
+    B, H, D = q.shape
+    Lcap = k_cache.shape[2]
+    L = Lcap if length is None else length
+    scale = default_scale(D) if scale is None else scale
+    bq, bk, bv = (DeviceBuffer.from_numpy(a) for a in (q, k_cache, v_cache))
+    o = DeviceBuffer((B, H, D), q.dtype)
+    attn_decode_raw(q.dtype, bq.ptr, bk.ptr, bv.ptr, o.ptr, B, H, L, D, scale,
+                    kv_strides=(H * Lcap * D, Lcap * D, D))
+    return o.numpy()

@@ -1,0 +1,161 @@
+/*
+ * deers_rocm.h — C ABI of the MI355X (gfx950) causal self-attention path for deers.
+ *
+ * This is the boundary a `Device::Rocm` storage backend in deers
+ * (a `src/storage/rocm.rs` next to src/storage/cuda.rs) binds with `extern "C"`.
+ * Plain pointers and sizes only.  Every function returns 0 on success and a
+ * non-zero DEERS_ROCM_ERR_* code on failure; the message for the calling
+ * thread's last failure is available from deers_rocm_last_error(), which is
+ * what the Rust side wraps into its backend error variant (the role
+ * `Error::Cuda(String)` plays at src/error.rs:40-41).
+ *
+ * Conventions shared by all entry points
+ *  - One process-global runtime, one device ordinal, one in-order stream; every
+ *    launch and copy below is enqueued on that stream and returns without
+ *    waiting, except deers_rocm_dtoh and deers_rocm_sync (the reference's CUDA
+ *    backend behaves the same way: src/storage/cuda.rs:462-521, 1541-1555,
+ *    1598-1602).
+ *  - The caller owns every buffer it passes.  The library keeps no pointer past
+ *    the call and never frees caller memory.  Internal workspace (softmax
+ *    statistics of the backward pass, split partial results of decode) is owned
+ *    and cached by the library.
+ *  - Entry points may be called from any thread; they serialise on an internal
+ *    mutex.
+ *  - dtype: DEERS_ROCM_F16 (IEEE half storage, f32 accumulate) or
+ *    DEERS_ROCM_F32.
+ *  - Tensors are logical [B,H,T,D].  A `strides` argument gives the four
+ *    element strides in that order (the reference's Layout strides,
+ *    src/layout.rs:151-155); NULL means compact row-major.  The innermost (D)
+ *    stride must be 1 and rows must be 16-byte aligned; other layouts are
+ *    rejected with DEERS_ROCM_ERR_LAYOUT and the caller compacts first, as
+ *    FusedLogSoftmax::forward does for its argument (src/ops.rs:1205).
+ */
+#ifndef DEERS_ROCM_H
+#define DEERS_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DEERS_ROCM_F16 0
+#define DEERS_ROCM_F32 1
+
+#define DEERS_ROCM_OK 0
+#define DEERS_ROCM_ERR_HIP 1         /* a HIP runtime call failed */
+#define DEERS_ROCM_ERR_ARG 2         /* null pointer, bad dtype, unsupported size */
+#define DEERS_ROCM_ERR_LAYOUT 3      /* strides the kernels cannot consume */
+#define DEERS_ROCM_ERR_NOT_INIT 4    /* deers_rocm_init has not succeeded */
+
+/* ---- runtime ------------------------------------------------------------ */
+
+/* Creates the process-global runtime on device `ordinal` (idempotent for the
+ * same ordinal).  Replaces the lazily-built CUDA runtime: context, default
+ * stream, module load (src/storage/cuda.rs:492-528). */
+int deers_rocm_init(int ordinal);
+
+/* 1 if a gfx950 device is present and the runtime can be (or was) created,
+ * else 0.  Replaces `is_available()` (src/storage/cuda.rs:647-649,
+ * src/device.rs:36-46). */
+int deers_rocm_available(void);
+
+/* Blocks until all work enqueued so far has finished.  Replaces
+ * `synchronize()` (src/storage/cuda.rs:1598-1602, src/device.rs:65-75). */
+int deers_rocm_sync(void);
+
+/* Message of the calling thread's most recent failure ("" if none).  The
+ * pointer stays valid until the same thread's next failing call. */
+const char* deers_rocm_last_error(void);
+
+/* The HIP stream all work is enqueued on (a hipStream_t), for callers that
+ * want to order their own work after it. */
+void* deers_rocm_stream(void);
+
+/* ---- device memory (the storage backend's alloc / to-device / to_vec) ---- */
+
+/* Replaces stream.alloc / alloc_zeros (src/storage/cuda.rs, `zeros` at
+ * src/device.rs:77-90).  `bytes` may be 0 (returns a NULL pointer). */
+int deers_rocm_alloc(size_t bytes, void** out_ptr);
+int deers_rocm_alloc_zeros(size_t bytes, void** out_ptr);
+int deers_rocm_free(void* ptr);
+
+/* Host->device copy, replaces CpuStorage::to(device) (src/storage/cpu.rs:26-32).
+ * Returns after the host buffer may be reused. */
+int deers_rocm_htod(void* dst_device, const void* src_host, size_t bytes);
+/* Device->host copy; waits for prior work, replaces to_vec
+ * (src/storage/cuda.rs:1541-1555). */
+int deers_rocm_dtoh(void* dst_host, const void* src_device, size_t bytes);
+/* Device->device copy on the stream (storage clone). */
+int deers_rocm_dtod(void* dst_device, const void* src_device, size_t bytes);
+
+/* ---- device timers (hipEvent pairs on the library stream) ---------------- */
+/* Replaces the per-launch start/end events the CUDA backend feeds its profiler
+ * with (src/storage/cuda.rs:530-561). */
+int deers_rocm_timer_create(void** out_timer);
+int deers_rocm_timer_start(void* timer);
+int deers_rocm_timer_stop(void* timer);
+/* Waits for the stop event and returns the elapsed milliseconds. */
+int deers_rocm_timer_elapsed_ms(void* timer, float* out_ms);
+int deers_rocm_timer_destroy(void* timer);
+
+/* ---- the attention path --------------------------------------------------- */
+
+/* Fused forward of the attention core of CausalSelfAttention::forward
+ * (src/models/gpt.rs:139-144):
+ *     O = softmax(Q K^T * scale + causal_mask) V
+ * which the reference evaluates as matmul -> scalar_mul -> causal_mask
+ * (src/nn/functional.rs:12-55) -> add -> log_sum_exp -> sub -> exp -> matmul,
+ * materialising [B,H,T,T] at each step.  Also writes LSE[B,H,T] (float32,
+ * compact), the natural-log row sums of the masked scaled scores, which is what
+ * the backward pass consumes instead of a saved probability tensor.
+ * q,k,v,o: [B,H,T,D] of `dtype`; D in {32,64,128}; T >= 1. */
+int deers_rocm_attn_fwd(int dtype,
+                        const void* q, const int64_t* q_strides,
+                        const void* k, const int64_t* k_strides,
+                        const void* v, const int64_t* v_strides,
+                        void* o, const int64_t* o_strides,
+                        float* lse,
+                        int64_t B, int64_t H, int64_t T, int64_t D, float scale);
+
+/* Fused backward: given dO, returns dQ, dK, dV equal to what the reference's
+ * autograd sweep (src/backprop.rs:52-66) produces through MatMul, Exp, Sub,
+ * Broadcast, LogSumExp, Add, ScalarMul and MatMul backward
+ * (src/ops.rs:1089-1101, 422-425, 210-214, 777-799, 1162-1175, 638-643):
+ *     P = exp(S*scale + mask - LSE);  dV = P^T dO;  dP = dO V^T;
+ *     dS = P o (dP - rowsum(dO o O));  dQ = scale dS K;  dK = scale dS^T Q.
+ * o and lse are the forward outputs.  dq,dk,dv are overwritten (not
+ * accumulated into); the caller's GradientStore::accumulate
+ * (src/backprop.rs:101-112) adds them to existing gradients. */
+int deers_rocm_attn_bwd(int dtype,
+                        const void* q, const int64_t* q_strides,
+                        const void* k, const int64_t* k_strides,
+                        const void* v, const int64_t* v_strides,
+                        const void* o, const int64_t* o_strides,
+                        const float* lse,
+                        const void* d_o, const int64_t* do_strides,
+                        void* dq, const int64_t* dq_strides,
+                        void* dk, const int64_t* dk_strides,
+                        void* dv, const int64_t* dv_strides,
+                        int64_t B, int64_t H, int64_t T, int64_t D, float scale);
+
+/* Decode: one query token per (b,h) against a KV cache of length L.  Same math
+ * as the forward with tgt_len = 1 and seqlen_offset = L-1, where the mask row
+ * is all zero (src/nn/functional.rs:26,42; tests/nn.rs:221-232); the reference
+ * has no KV cache and re-runs the whole window per token
+ * (examples/tinystories_train.rs:250-276).
+ * q,o: [B,H,D] compact.  k_cache,v_cache: [B,H,L_cap,D] with element strides
+ * `kv_strides` = {b,h,l} (NULL: compact with L_cap = L); only rows [0,L) are
+ * read.  D in {64,128}. */
+int deers_rocm_attn_decode(int dtype,
+                           const void* q,
+                           const void* k_cache, const void* v_cache,
+                           const int64_t* kv_strides,
+                           void* o,
+                           int64_t B, int64_t H, int64_t L, int64_t D, float scale);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEERS_ROCM_H */

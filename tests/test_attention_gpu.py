@@ -1,0 +1,221 @@
+"""Parity of the HIP attention path (through the C ABI) against the CPU oracle.
+
+Tolerances are the contract's: max abs error <= 1e-4 for f32, <= 5e-3 for f16
+against the f32 oracle evaluated on the same f16-rounded inputs.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from deers_amd import rocm, synth
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float16): 5e-3}
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def max_err(a, b):
+    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))))
+
+
+def check_case(x, tol, label, heads=None):
+    """Runs fwd+bwd on the GPU for inputs dict x and compares with the oracle."""
+    q, k, v, do = x["q"], x["k"], x["v"], x["do"]
+    o, lse, dq, dk, dv = rocm.attn_fwd_bwd(q, k, v, do)
+    sl = slice(None) if heads is None else heads
+    ro, rlse = oracle.attn_fwd(q[sl], k[sl], v[sl], return_lse=True, heads_per_call=1)
+    rdq, rdk, rdv = oracle.attn_bwd(q[sl], k[sl], v[sl], do[sl], heads_per_call=1)
+    errs = {"o": max_err(o[sl], ro), "lse": max_err(lse[sl], rlse), "dq": max_err(dq[sl], rdq),
+            "dk": max_err(dk[sl], rdk), "dv": max_err(dv[sl], rdv)}
+    say(f"{label}: " + " ".join(f"{n}={e:.2e}" for n, e in errs.items()))
+    for n, e in errs.items():
+        assert e <= tol, f"{label}: {n} max abs err {e:.3e} > {tol}"
+    return o, lse, dq, dk, dv
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))),
+                         ids=lambda p: os.path.basename(p)[:-4])
+def test_golden_fixtures(path):
+    f = np.load(path)
+    q, k, v, do = f["q"], f["k"], f["v"], f["do"]
+    tol = TOL[q.dtype]
+    say(f"fixture {os.path.basename(path)} dtype={q.dtype} q{q.shape} k{k.shape}")
+    if q.shape[2] == 1 and k.shape[2] > 1:  # decode fixture
+        o = rocm.attn_decode(q[:, :, 0], k, v)
+        assert max_err(o, f["y"][:, :, 0]) <= tol
+        return
+    o, lse, dq, dk, dv = rocm.attn_fwd_bwd(q, k, v, do)
+    for got, name in ((o, "y"), (lse, "lse"), (dq, "dq"), (dk, "dk"), (dv, "dv")):
+        e = max_err(got, f[name])
+        say(f"  {name}: {e:.2e}")
+        assert e <= tol, f"{name}: {e:.3e} > {tol}"
+
+
+SHAPES = [
+    # dtype, B, H, T, D
+    (np.float32, 1, 1, 1, 32), (np.float32, 2, 2, 31, 32), (np.float32, 1, 3, 64, 32),
+    (np.float32, 1, 2, 129, 64), (np.float32, 2, 1, 257, 64), (np.float32, 1, 1, 300, 128),
+    (np.float16, 1, 1, 1, 64), (np.float16, 2, 2, 5, 64), (np.float16, 1, 2, 63, 64),
+    (np.float16, 1, 2, 64, 64), (np.float16, 1, 2, 65, 64), (np.float16, 2, 3, 127, 64),
+    (np.float16, 1, 2, 128, 64), (np.float16, 1, 2, 129, 64), (np.float16, 1, 2, 300, 64),
+    (np.float16, 1, 2, 513, 64), (np.float16, 2, 2, 100, 32), (np.float16, 1, 2, 257, 128),
+    (np.float16, 1, 1, 1024, 128),
+]
+
+
+@pytest.mark.parametrize("dtype,B,H,T,D", SHAPES,
+                         ids=[f"{np.dtype(s[0]).name}-b{s[1]}h{s[2]}t{s[3]}d{s[4]}" for s in SHAPES])
+def test_ragged_shapes_match_oracle(dtype, B, H, T, D):
+    name = f"shape-{np.dtype(dtype).name}-{B}-{H}-{T}-{D}"
+    x = synth.attention_inputs(name, B, H, T, D, dtype, base_seed=7)
+    check_case(x, TOL[np.dtype(dtype)], name)
+
+
+def test_config1_f32_full():
+    """B=4 H=6 T=256 D=32 f32: the reference's own CPU-runnable case."""
+    x = synth.attention_inputs("c1", 4, 6, 256, 32, np.float32, base_seed=0)
+    check_case(x, 1e-4, "C1")
+
+
+def test_config2_f16_full_size():
+    """B=8 H=12 T=1024 D=64 f16: GPU on the whole problem, oracle on batches 0 and 7."""
+    x = synth.attention_inputs("c2", 8, 12, 1024, 64, np.float16, base_seed=0)
+    o, lse, dq, dk, dv = check_case(x, 5e-3, "C2", heads=[0, 7])
+    for a in (o, lse, dq, dk, dv):
+        assert np.isfinite(a.astype(np.float32)).all()
+    # size-independent properties on the full problem
+    np.testing.assert_array_equal(o[:, :, 0], x["v"][:, :, 0])        # first row attends to itself
+    o2, lse2, dq2, dk2, dv2 = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])
+    for a, b in ((o, o2), (lse, lse2), (dq, dq2), (dk, dk2), (dv, dv2)):
+        np.testing.assert_array_equal(a, b)                           # no atomics: bit-reproducible
+
+
+def test_config3_long_context_f16():
+    """B=1 H=16 T=8192 D=128 f16, sigma 0.5: GPU on all heads, oracle on heads 0 and 15."""
+    x = synth.attention_inputs("c3", 1, 16, 8192, 128, np.float16, base_seed=0, sigma=0.5)
+    q, k, v, do = x["q"], x["k"], x["v"], x["do"]
+    o, lse, dq, dk, dv = rocm.attn_fwd_bwd(q, k, v, do)
+    for hsel in (0, 15):
+        sl = (slice(None), slice(hsel, hsel + 1))
+        ro, rlse = oracle.attn_fwd(q[sl], k[sl], v[sl], return_lse=True)
+        rdq, rdk, rdv = oracle.attn_bwd(q[sl], k[sl], v[sl], do[sl])
+        errs = {"o": max_err(o[sl], ro), "lse": max_err(lse[sl], rlse),
+                "dq": max_err(dq[sl], rdq), "dk": max_err(dk[sl], rdk), "dv": max_err(dv[sl], rdv)}
+        say(f"C3 head {hsel}: " + " ".join(f"{n}={e:.2e}" for n, e in errs.items()))
+        for n, e in errs.items():
+            assert e <= 5e-3, f"C3 head {hsel} {n}: {e:.3e}"
+
+
+def test_causality_and_linearity_properties():
+    x = synth.attention_inputs("prop", 2, 4, 384, 64, np.float16, base_seed=3)
+    q, k, v, do = x["q"], x["k"], x["v"], x["do"]
+    o, lse, dq, dk, dv = rocm.attn_fwd_bwd(q, k, v, do)
+    # perturbing keys/values at positions >= 200 cannot change outputs before 200 (bit-exact)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, 200:] = -k2[:, :, 200:]
+    v2[:, :, 200:] += np.float16(1.0)
+    o2, lse2 = rocm.attn_fwd(q, k2, v2)
+    np.testing.assert_array_equal(o2[:, :, :200], o[:, :, :200])
+    np.testing.assert_array_equal(lse2[:, :, :200], lse[:, :, :200])
+    # q = 0: uniform weights, output is the running mean of v
+    om, _ = rocm.attn_fwd(np.zeros_like(q), k, v)
+    want = np.cumsum(v.astype(np.float64), 2) / np.arange(1, 385)[None, None, :, None]
+    assert max_err(om, want) <= 2e-3
+    # the backward map is linear in dO: zero dO gives exactly zero gradients
+    _, _, z1, z2, z3 = rocm.attn_fwd_bwd(q, k, v, np.zeros_like(do))
+    assert not z1.any() and not z2.any() and not z3.any()
+    # the last key/value only receives gradient from the last query
+    do_last = np.zeros_like(do)
+    do_last[:, :, -1] = do[:, :, -1]
+    _, _, gq, gk, gv = rocm.attn_fwd_bwd(q, k, v, do_last)
+    assert not gq[:, :, :-1].any()
+    assert max_err(gk[:, :, -1], dk[:, :, -1]) <= 5e-3 and max_err(gv[:, :, -1], dv[:, :, -1]) <= 5e-3
+
+
+def test_strided_head_interleaved_layout():
+    """v reaches the reference's matmul as a [B,H,T,D] view of [B,T,H,D] memory
+    (strides [T*C, D, C, 1], src/models/gpt.rs:137); the ABI takes such views by stride."""
+    B, H, T, D = 2, 3, 150, 64
+    x = synth.attention_inputs("strided", B, H, T, D, np.float16, base_seed=5)
+    want_o, want_lse, want_dq, want_dk, want_dv = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])
+    C = H * D
+    st = (T * C, D, C, 1)
+    bufs = {n: rocm.DeviceBuffer.from_numpy(np.ascontiguousarray(x[n].transpose(0, 2, 1, 3)))
+            for n in ("q", "k", "v", "do")}
+    o = rocm.DeviceBuffer((B, T, H, D), np.float16)
+    gq, gk, gv = (rocm.DeviceBuffer((B, T, H, D), np.float16) for _ in range(3))
+    lse = rocm.DeviceBuffer((B, H, T), np.float32)
+    sc = rocm.default_scale(D)
+    rocm.attn_fwd_raw(np.float16, bufs["q"].ptr, bufs["k"].ptr, bufs["v"].ptr, o.ptr, lse.ptr,
+                      B, H, T, D, sc, st, st, st, st)
+    names = ("q", "k", "v", "o", "do", "dq", "dk", "dv")
+    rocm.attn_bwd_raw(np.float16, bufs["q"].ptr, bufs["k"].ptr, bufs["v"].ptr, o.ptr, lse.ptr,
+                      bufs["do"].ptr, gq.ptr, gk.ptr, gv.ptr, B, H, T, D, sc,
+                      strides={n: st for n in names})
+    np.testing.assert_array_equal(o.numpy().transpose(0, 2, 1, 3), want_o)
+    np.testing.assert_array_equal(lse.numpy(), want_lse)
+    for got, want in ((gq, want_dq), (gk, want_dk), (gv, want_dv)):
+        np.testing.assert_array_equal(got.numpy().transpose(0, 2, 1, 3), want)
+
+
+@pytest.mark.parametrize("B,H,L,D", [(1, 1, 1, 64), (2, 3, 77, 64), (3, 2, 1000, 64),
+                                     (2, 2, 4096, 128), (1, 5, 333, 128)])
+def test_decode_matches_oracle(B, H, L, D):
+    name = f"dec-{B}-{H}-{L}-{D}"
+    x = synth.attention_inputs(name, B, H, 1, D, np.float16, base_seed=9, kv_len=L,
+                               names=("q", "k", "v"))
+    o = rocm.attn_decode(x["q"][:, :, 0], x["k"], x["v"])
+    want = oracle.attn_fwd(x["q"], x["k"], x["v"])[:, :, 0]
+    e = max_err(o, want)
+    say(f"{name}: {e:.2e}")
+    assert e <= 5e-3
+
+
+def test_decode_config4_full_size_and_cache_capacity():
+    """B=32 H=12 L=4096 D=64 f16; also a cache with spare capacity past L."""
+    B, H, L, D = 32, 12, 4096, 64
+    x = synth.attention_inputs("c4", B, H, 1, D, np.float16, base_seed=0, kv_len=L,
+                               names=("q", "k", "v"))
+    o = rocm.attn_decode(x["q"][:, :, 0], x["k"], x["v"])
+    want = oracle.attn_fwd(x["q"], x["k"], x["v"])[:, :, 0]
+    e = max_err(o, want)
+    say(f"C4: {e:.2e}")
+    assert e <= 5e-3
+    # rows past `length` must not be read into the result
+    o_short = rocm.attn_decode(x["q"][:, :, 0], x["k"], x["v"], length=1000)
+    want_short = oracle.attn_fwd(x["q"], x["k"][:, :, :1000], x["v"][:, :, :1000])[:, :, 0]
+    assert max_err(o_short, want_short) <= 5e-3
+
+
+def test_decode_equals_last_row_of_prefill():
+    """Decode with offset L-1 is the last row of the causal forward (same math, no mask)."""
+    x = synth.attention_inputs("dec-vs-fwd", 2, 2, 200, 64, np.float16, base_seed=11)
+    o, _ = rocm.attn_fwd(x["q"], x["k"], x["v"])
+    od = rocm.attn_decode(x["q"][:, :, -1], x["k"], x["v"])
+    assert max_err(od, o[:, :, -1]) <= 2e-3
+
+
+def test_error_paths_report_messages():
+    B, H, T, D = 1, 1, 16, 64
+    buf = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    lse = rocm.DeviceBuffer((B, H, T), np.float32)
+    with pytest.raises(rocm.RocmError, match="head dim"):
+        rocm.attn_fwd_raw(np.float16, buf.ptr, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, T, 48, 0.1)
+    with pytest.raises(rocm.RocmError, match="innermost stride"):
+        rocm.attn_fwd_raw(np.float16, buf.ptr, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, T, D, 0.1,
+                          q_strides=(T * D, T * D, 1, T))
+    with pytest.raises(rocm.RocmError, match="16-byte"):
+        rocm.attn_fwd_raw(np.float16, buf.ptr, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, T, D, 0.1,
+                          q_strides=(T * D, T * D, D + 2, 1))
+    with pytest.raises(rocm.RocmError, match="null"):
+        rocm.attn_fwd_raw(np.float16, None, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, T, D, 0.1)
+    with pytest.raises(rocm.RocmError, match=">= 1"):
+        rocm.attn_fwd_raw(np.float16, buf.ptr, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, 0, D, 0.1)
