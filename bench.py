@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X causal-attention path (one GPU).
+
+A "step" is one fused forward + backward of causal self-attention over one batch
+of synthetic, seeded inputs that are already resident in HBM:
+f16, B=8 H=12 T=1024 D=64 (GPT-2-small geometry).  The headline value is
+TFLOP/s with the FlashAttention FLOP convention, fwd+bwd = 7*B*H*T^2*D
+(causal-halved; the backward counted as 2.5x the forward however many tile
+GEMMs the kernels really execute).  The decode kernel (B=32 H=12 L=4096 D=64,
+f16) is timed in the same run and reported as achieved HBM GB/s.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel of the step from
+per-kernel hipEvent times taken in a second pass of the same K steps (event
+pairs between kernels would perturb the headline timing, so that pass is
+separate); `cpu_baseline` is the CPU oracle (a restatement of the reference's
+materialised CPU path) timed on this box's host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from deers_amd import rocm, synth  # noqa: E402
+
+PEAK_F16_TFLOPS = 2500.0  # MI355X dense f16 MFMA, published
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+
+C2 = dict(B=8, H=12, T=1024, D=64)
+C4 = dict(B=32, H=12, L=4096, D=64)
+
+
+def attn_flops(B, H, T, D):
+    fwd = 4.0 * B * H * T * T * D / 2.0
+    return fwd, 2.5 * fwd
+
+
+def bench_train(steps: int, warmup: int):
+    B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
+    x = synth.attention_inputs("c2", B, H, T, D, np.float16, base_seed=0)
+    q, k, v, do = (rocm.DeviceBuffer.from_numpy(x[n]) for n in ("q", "k", "v", "do"))
+    o = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    lse = rocm.DeviceBuffer((B, H, T), np.float32)
+    dq, dk, dv = (rocm.DeviceBuffer((B, H, T, D), np.float16) for _ in range(3))
+    scale = rocm.default_scale(D)
+
+    def step():
+        rocm.attn_fwd_raw(np.float16, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, B, H, T, D, scale)
+        rocm.attn_bwd_raw(np.float16, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, do.ptr, dq.ptr, dk.ptr,
+                          dv.ptr, B, H, T, D, scale)
+
+    for _ in range(warmup):
+        step()
+    rocm.sync()
+    timer = rocm.Timer()
+    t0 = time.perf_counter()
+    timer.start()
+    for _ in range(steps):
+        step()
+    timer.stop()
+    rocm.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    dev_ms = timer.elapsed_ms()
+
+    # second pass: per-kernel device times
+    rocm.profile_enable(True)
+    for _ in range(steps):
+        step()
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    kernels = {n: {"calls": c, "avg_us": 1e3 * ms / c} for n, (c, ms) in prof.items()}
+    return dict(wall_ms=wall_ms, dev_ms=dev_ms, kernels=kernels)
+
+
+def bench_decode(steps: int, warmup: int, rotate: int = 4):
+    """Decode over `rotate` distinct KV caches in turn so the 256 MB last-level cache
+    cannot serve a 403 MB working set from one call to the next."""
+    B, H, L, D = C4["B"], C4["H"], C4["L"], C4["D"]
+    x = synth.attention_inputs("c4", B, H, 1, D, np.float16, base_seed=0, kv_len=L,
+                               names=("q", "k", "v"))
+    qb = rocm.DeviceBuffer.from_numpy(x["q"][:, :, 0])
+    caches = []
+    for r in range(rotate):
+        kk = np.roll(x["k"], r, axis=0)
+        vv = np.roll(x["v"], r, axis=0)
+        caches.append((rocm.DeviceBuffer.from_numpy(kk), rocm.DeviceBuffer.from_numpy(vv)))
+    ob = rocm.DeviceBuffer((B, H, D), np.float16)
+    scale = rocm.default_scale(D)
+
+    def call(i):
+        kb, vb = caches[i % rotate]
+        rocm.attn_decode_raw(np.float16, qb.ptr, kb.ptr, vb.ptr, ob.ptr, B, H, L, D, scale)
+
+    for i in range(warmup):
+        call(i)
+    rocm.sync()
+    rocm.profile_enable(True)
+    for i in range(steps):
+        call(i)
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    calls, ms = prof["attn_decode_f16"]
+    mcalls, mms = prof["attn_decode_merge"]
+    nbytes = 2.0 * B * H * L * D * 2 + 2 * B * H * D * 2
+    main_us = 1e3 * ms / calls
+    total_us = main_us + 1e3 * mms / mcalls
+    return dict(bytes=nbytes, kernel_us=main_us, call_us=total_us,
+                gbs_kernel=nbytes / (main_us * 1e-6) / 1e9,
+                gbs_call=nbytes / (total_us * 1e-6) / 1e9)
+
+
+def cpu_baseline():
+    """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
+    attention; the Rust reference itself cannot be built here) on the full B=8 H=12
+    T=1024 D=64 problem, 1 warm-up + 2 timed fwd+bwd passes, median.  GEMMs use all
+    host threads, element-wise passes one thread, mirroring the reference."""
+    import oracle  # the checker; only ever the thing measured in this baseline leg
+    B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
+    x = synth.attention_inputs("c2", B, H, T, D, np.float16, base_seed=0)
+    q, k, v, do = (x[n].astype(np.float32) for n in ("q", "k", "v", "do"))
+    threads = oracle.max_threads()
+    times = []
+    for it in range(3):
+        t0 = time.perf_counter()
+        oracle.attn_fwd(q, k, v, nthreads=threads)
+        oracle.attn_bwd(q, k, v, do, nthreads=threads)
+        if it > 0:
+            times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    fwd, bwd = attn_flops(B, H, T, D)
+    return {"value": (fwd + bwd) / sec / 1e12, "unit": "TFLOP/s", "cores": threads,
+            "kind": "port", "seconds_per_step": sec,
+            "sample": "full workload (B=8 H=12 T=1024 D=64, f32 on the f16-rounded inputs), "
+                      "1 warm-up + 2 timed fwd+bwd passes, median"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the attention path has no cross-GPU exchange "
+                 "(it shards over batch x heads with no communication); run with --gpus 1")
+    if not rocm.available():
+        sys.exit("no gfx950 device visible: the attention path has no CPU fallback")
+    rocm.init(0)
+
+    B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
+    fwd_f, bwd_f = attn_flops(B, H, T, D)
+    tr = bench_train(args.steps, args.warmup)
+    ms_per_step = tr["dev_ms"] / args.steps
+    tflops = (fwd_f + bwd_f) / (ms_per_step * 1e-3) / 1e12
+
+    # dominant kernel of the step and its roofline
+    kern = tr["kernels"]
+    dom = max(kern, key=lambda n: kern[n]["avg_us"] * kern[n]["calls"])
+    # tile GEMMs each kernel must execute (causal-halved, 2*B*H*T^2*D/2 FLOP each)
+    gemm = 2.0 * B * H * T * T * D / 2.0
+    kernel_flops = {"attn_fwd_f16": 2 * gemm, "attn_bwd_dkdv_f16": 4 * gemm,
+                    "attn_bwd_dq_f16": 3 * gemm}
+    for n, st in kern.items():
+        if n in kernel_flops:
+            st["tflops"] = kernel_flops[n] / (st["avg_us"] * 1e-6) / 1e12
+            st["frac_mfma_peak"] = st["tflops"] / PEAK_F16_TFLOPS
+    achieved = kern[dom].get("tflops")
+    roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
+                "unit": "TFLOP/s", "frac": (achieved / PEAK_F16_TFLOPS) if achieved else None,
+                "traffic": None, "avg_launch_us": kern[dom]["avg_us"],
+                "flops_per_launch": kernel_flops.get(dom)}
+
+    dec = bench_decode(args.steps, args.warmup)
+
+    out = {
+        "metric": "causal attn fwd+bwd TFLOP/s & %MFMA peak (T=1024,D=64,f16); decode HBM GB/s",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "causal self-attention fwd+bwd, f16 in / f32 accumulate, "
+                               "B=8 H=12 T=1024 D=64 (BASELINE configs[1])",
+                   "flops_per_step": fwd_f + bwd_f, "flop_convention": "7*B*H*T^2*D"},
+        "frac_mfma_peak": tflops / PEAK_F16_TFLOPS,
+        "peak_tflops_f16_dense": PEAK_F16_TFLOPS,
+        "wall_ms_per_step": tr["wall_ms"] / args.steps,
+        "kernels": kern,
+        "roofline": roofline,
+        "decode": {"workload": "decode f16 B=32 H=12 L=4096 D=64 (BASELINE configs[3]), "
+                               "4 KV caches in rotation",
+                   "bytes_per_call": dec["bytes"], "kernel_us": dec["kernel_us"],
+                   "call_us": dec["call_us"], "GB/s": dec["gbs_kernel"],
+                   "GB/s_incl_merge": dec["gbs_call"], "peak_GB/s": PEAK_HBM_GBS,
+                   "frac_hbm_peak": dec["gbs_kernel"] / PEAK_HBM_GBS},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -350,11 +350,20 @@ static void launch_bwd_f32_d(const BwdParams& p, int B, hipStream_t stream) {
   const int64_t rows = (int64_t)B * p.H * p.T;
   constexpr int LPR = D / 4;
   const int64_t threads = rows * LPR;
-  hipLaunchKernelGGL((attn_bwd_delta_kernel<float, D>), dim3((threads + 255) / 256), dim3(256), 0,
-                     stream, p, B);
+  {
+    LaunchScope scope("attn_bwd_delta", stream);
+    hipLaunchKernelGGL((attn_bwd_delta_kernel<float, D>), dim3((threads + 255) / 256), dim3(256),
+                       0, stream, p, B);
+  }
   dim3 grid((p.T + kBwd32Blk - 1) / kBwd32Blk, B * p.H);
-  hipLaunchKernelGGL((attn_bwd_dkdv_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
-  hipLaunchKernelGGL((attn_bwd_dq_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
+  {
+    LaunchScope scope("attn_bwd_dkdv_f32", stream);
+    hipLaunchKernelGGL((attn_bwd_dkdv_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
+  }
+  {
+    LaunchScope scope("attn_bwd_dq_f32", stream);
+    hipLaunchKernelGGL((attn_bwd_dq_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
+  }
 }
 
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream) {

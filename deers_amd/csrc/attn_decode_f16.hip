@@ -148,10 +148,18 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(DecodeParams p) {
 void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream) {
   dim3 grid(p.splits, B * p.H);
   if (D == 64) {
-    hipLaunchKernelGGL(attn_decode_f16_kernel<64>, grid, dim3(256), 0, stream, p);
+    {
+      LaunchScope scope("attn_decode_f16", stream);
+      hipLaunchKernelGGL(attn_decode_f16_kernel<64>, grid, dim3(256), 0, stream, p);
+    }
+    LaunchScope scope("attn_decode_merge", stream);
     hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(B * p.H), dim3(64), 0, stream, p);
   } else {
-    hipLaunchKernelGGL(attn_decode_f16_kernel<128>, grid, dim3(256), 0, stream, p);
+    {
+      LaunchScope scope("attn_decode_f16", stream);
+      hipLaunchKernelGGL(attn_decode_f16_kernel<128>, grid, dim3(256), 0, stream, p);
+    }
+    LaunchScope scope("attn_decode_merge", stream);
     hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(B * p.H), dim3(128), 0, stream, p);
   }
 }

@@ -193,6 +193,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f16_kernel(FwdParams p) {
 
 void launch_attn_fwd_f16(const FwdParams& p, int B, int D, hipStream_t stream) {
   dim3 grid((p.T + kFwdBM - 1) / kFwdBM, B * p.H);
+  LaunchScope scope("attn_fwd_f16", stream);
   switch (D) {
     case 32: hipLaunchKernelGGL(attn_fwd_f16_kernel<32>, grid, dim3(256), 0, stream, p); break;
     case 64: hipLaunchKernelGGL(attn_fwd_f16_kernel<64>, grid, dim3(256), 0, stream, p); break;

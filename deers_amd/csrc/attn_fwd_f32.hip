@@ -174,6 +174,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(FwdParams p) {
 
 void launch_attn_fwd_f32(const FwdParams& p, int B, int D, hipStream_t stream) {
   dim3 grid((p.T + kFwd32BM - 1) / kFwd32BM, B * p.H);
+  LaunchScope scope("attn_fwd_f32", stream);
   switch (D) {
     case 32:
       hipLaunchKernelGGL((attn_fwd_f32_kernel<32, 64>), grid, dim3(256), 0, stream, p);

@@ -104,4 +104,18 @@ struct DecodeParams {
   float scale_log2;
 };
 
+// Brackets one kernel launch with a hipEvent pair when per-kernel profiling is
+// switched on (deers_rocm_profile_enable); a no-op otherwise.  Defined in
+// runtime.hip.
+struct LaunchScope {
+  LaunchScope(const char* name, hipStream_t stream);
+  ~LaunchScope();
+  LaunchScope(const LaunchScope&) = delete;
+  LaunchScope& operator=(const LaunchScope&) = delete;
+
+ private:
+  void* rec_;
+  hipStream_t stream_;
+};
+
 }  // namespace deers

@@ -10,8 +10,10 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <map>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "common.h"
 
@@ -128,7 +130,53 @@ struct Timer {
   hipEvent_t start, stop;
 };
 
+// Per-kernel profiling records (guarded by g_mu: launches happen under it).
+struct LaunchRecord {
+  const char* name;
+  hipEvent_t start, stop;
+};
+bool g_prof_on = false;
+std::vector<LaunchRecord*> g_prof_records;
+struct ProfRow {
+  std::string name;
+  int64_t calls;
+  float total_ms;
+};
+std::vector<ProfRow> g_prof_rows;
+
+void prof_clear() {
+  for (LaunchRecord* r : g_prof_records) {
+    (void)hipEventDestroy(r->start);
+    (void)hipEventDestroy(r->stop);
+    delete r;
+  }
+  g_prof_records.clear();
+  g_prof_rows.clear();
+}
+
 }  // namespace
+
+namespace deers {
+
+LaunchScope::LaunchScope(const char* name, hipStream_t stream) : rec_(nullptr), stream_(stream) {
+  if (!g_prof_on) return;
+  LaunchRecord* r = new LaunchRecord{name, nullptr, nullptr};
+  if (hipEventCreate(&r->start) != hipSuccess || hipEventCreate(&r->stop) != hipSuccess ||
+      hipEventRecord(r->start, stream) != hipSuccess) {
+    delete r;
+    return;
+  }
+  rec_ = r;
+}
+
+LaunchScope::~LaunchScope() {
+  if (!rec_) return;
+  LaunchRecord* r = static_cast<LaunchRecord*>(rec_);
+  (void)hipEventRecord(r->stop, stream_);
+  g_prof_records.push_back(r);
+}
+
+}  // namespace deers
 
 extern "C" {
 
@@ -274,9 +322,49 @@ int deers_rocm_timer_destroy(void* timer) {
   std::lock_guard<std::mutex> lock(g_mu);
   if (!timer) return DEERS_ROCM_OK;
   Timer* t = static_cast<Timer*>(timer);
-  hipEventDestroy(t->start);
-  hipEventDestroy(t->stop);
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
   delete t;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  if (on) prof_clear();
+  g_prof_on = on != 0;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_profile_collect(int* out_rows) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (!out_rows) return fail(DEERS_ROCM_ERR_ARG, "profile_collect: null out_rows");
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  std::map<std::string, ProfRow> agg;
+  for (LaunchRecord* r : g_prof_records) {
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, r->start, r->stop));
+    ProfRow& row = agg[r->name];
+    row.name = r->name;
+    row.calls += 1;
+    row.total_ms += ms;
+  }
+  g_prof_rows.clear();
+  for (auto& kv : agg) g_prof_rows.push_back(kv.second);
+  *out_rows = (int)g_prof_rows.size();
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_profile_row(int index, const char** out_name, int64_t* out_calls,
+                           float* out_total_ms) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (index < 0 || index >= (int)g_prof_rows.size() || !out_name || !out_calls || !out_total_ms)
+    return fail(DEERS_ROCM_ERR_ARG, "profile_row: bad index or null argument");
+  *out_name = g_prof_rows[index].name.c_str();
+  *out_calls = g_prof_rows[index].calls;
+  *out_total_ms = g_prof_rows[index].total_ms;
   return DEERS_ROCM_OK;
 }
 

@@ -134,6 +134,25 @@ class Timer:
             pass
 
 
+def profile_enable(on: bool = True):
+    """Switch per-kernel event timing on (clears earlier records) or off."""
+    init()
+    _check(load().deers_rocm_profile_enable(ctypes.c_int(1 if on else 0)))
+
+
+def profile_collect() -> dict:
+    """{kernel name: (calls, total_ms)} for launches since profile_enable(True)."""
+    n = ctypes.c_int()
+    _check(load().deers_rocm_profile_collect(ctypes.byref(n)))
+    out = {}
+    for i in range(n.value):
+        name, calls, ms = ctypes.c_char_p(), ctypes.c_int64(), ctypes.c_float()
+        _check(load().deers_rocm_profile_row(ctypes.c_int(i), ctypes.byref(name),
+                                             ctypes.byref(calls), ctypes.byref(ms)))
+        out[name.value.decode()] = (int(calls.value), float(ms.value))
+    return out
+
+
 def _strides(s):
     if s is None:
         return None

@@ -100,6 +100,18 @@ int deers_rocm_timer_stop(void* timer);
 int deers_rocm_timer_elapsed_ms(void* timer, float* out_ms);
 int deers_rocm_timer_destroy(void* timer);
 
+/* ---- per-kernel device times ---------------------------------------------- */
+/* When enabled, every kernel the library launches is bracketed by a hipEvent
+ * pair, the way the reference's CUDA backend reports per-launch device time to
+ * its profiler (src/storage/cuda.rs:530-561, src/profiler.rs:361-367).
+ * enable(1) clears earlier records; collect() waits for the stream, aggregates
+ * by kernel name and returns the number of rows; row(i) reads one aggregate
+ * (name pointer valid until the next collect/enable). */
+int deers_rocm_profile_enable(int on);
+int deers_rocm_profile_collect(int* out_rows);
+int deers_rocm_profile_row(int index, const char** out_name, int64_t* out_calls,
+                           float* out_total_ms);
+
 /* ---- the attention path --------------------------------------------------- */
 
 /* Fused forward of the attention core of CausalSelfAttention::forward
