@@ -8,22 +8,32 @@
 //     dQ = scale dS K                       dK = scale dS^T Q
 //
 // Three launches, no atomics, bit-reproducible:
-//   1. delta   : delta[b,h,t] = sum_d dO*O (f32).
+//   1. prep    : negdelta[b,h,t] = -sum_d dO*O and lse2 = LSE*log2(e), both f32 in a
+//                workspace whose rows are padded to a multiple of 64 per head
+//                (lse2 = +inf, negdelta = 0 in the padding, so padded query rows
+//                get probability exactly 0).
 //   2. dK/dV   : a workgroup owns 128 key rows (32 per wave, K^T and V^T held in
-//                registers as B operands) and walks the query tiles at or below
-//                the diagonal.  Orientation S[q,kv] (one key column per lane) so P
-//                and dS leave the accumulators directly as B operands of
+//                registers as B operands) and walks the 64-row query tiles at or
+//                below the diagonal.  Orientation S[q,kv] (one key column per lane)
+//                so P and dS leave the accumulators directly as B operands of
 //                dV^T += dO^T P and dK^T += Q^T dS; dO^T / Q^T fragments come
 //                from the row-major LDS tiles via ds_read_b64_tr_b16.
 //   3. dQ      : a workgroup owns 128 query rows (32 per wave, Q and dO in
-//                registers) and walks key tiles up to the diagonal.  Orientation
-//                S^T[kv,q] (one query column per lane, LSE and delta are per-lane
-//                scalars); dS^T leaves the accumulators as the B operand of
+//                registers) and walks 64-row key tiles up to the diagonal.
+//                Orientation S^T[kv,q] (one query column per lane, LSE and delta are
+//                per-lane scalars); dS^T leaves the accumulators as the B operand of
 //                dQ^T += K^T dS^T with K^T fragments read transposed from LDS.
 // Recomputing S and dP in both 2 and 3 costs 7 tile GEMMs instead of 5 but
 // keeps every product in registers and needs no dQ accumulation buffer.
+//
+// The "- delta" of dS is folded into the dP accumulator's initial value, so the
+// vector pipe spends per score one fma + one exp2 (P), one multiply (dS) and the
+// f16 packing.  Streamed tiles go global -> LDS asynchronously
+// (global_load_lds_dwordx4), unpadded and XOR-swizzled, into a ring of P+1 slots
+// requested P iterations ahead; one barrier per iteration.
+#include <type_traits>
+
 #include "common.h"
-#include "bwd_delta.h"
 
 namespace deers {
 
@@ -33,29 +43,96 @@ constexpr int kBwdStep = 64;  // rows of the streamed operand per iteration
 #define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
 
+template <int D>
+struct BwdCfg {
+  static constexpr int P = (D == 128) ? 1 : 2;   // prefetch distance in iterations
+  static constexpr int NS = P + 1;               // ring slots
+  static constexpr int RB = D * 2;               // row bytes
+  static constexpr int TILE_B = kBwdStep * RB;   // bytes of one streamed tile
+  static constexpr int VEC_B = kBwdStep * 4;     // bytes of one per-row f32 vector
+  static constexpr int SLOT_B = 2 * TILE_B + 2 * VEC_B;  // dK/dV: Q, dO, lse2, negdelta
+  static constexpr size_t kLdsDkdv = NS * SLOT_B;
+  static constexpr size_t kLdsDq = NS * 2 * TILE_B;      // dQ: K, V
+};
+
+// Maps blockIdx.x to (head, block rank) so that a head stays on one XCD and the
+// workgroups an XCD's CUs receive in turn (items i, i+32, i+64, ...) have even
+// total length: the XCD's list is sorted longest first and every second group of
+// 32 is reversed.  rank 0 is the longest block.  Returns false for padding ids.
+__device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int BH, int* bh,
+                                          int* rank) {
+  const int xcd = blockIdx.x & 7;
+  int idx = blockIdx.x >> 3;
+  const int per_xcd = n_blocks * heads_per_xcd;
+  const int grp = idx >> 5, pos = idx & 31;
+  const int grp_len = min(32, per_xcd - 32 * grp);
+  if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
+  *bh = (idx % heads_per_xcd) * 8 + xcd;
+  *rank = idx / heads_per_xcd;
+  return *bh < BH;
+}
+
+// ---------------------------------------------------------------------------
+// prep: negdelta and lse2, LPR lanes share one row.
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_prep_f16_kernel(BwdParams p, int B) {
+  constexpr int LPR = D / 8;  // lanes per row
+  const int64_t rows = (int64_t)B * p.H * p.t_pad;
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+  const int part = threadIdx.x % LPR;
+  float acc = 0.f;
+  const int t = row < rows ? (int)(row % p.t_pad) : 0;
+  const int bh = row < rows ? (int)(row / p.t_pad) : 0;
+  const bool live = row < rows && t < p.T;
+  if (live) {
+    const int b = bh / p.H, h = bh % p.H;
+    const half_t* o = (const half_t*)p.o + b * p.so.b + h * p.so.h + (int64_t)t * p.so.t + 8 * part;
+    const half_t* d =
+        (const half_t*)p.d_o + b * p.sdo.b + h * p.sdo.h + (int64_t)t * p.sdo.t + 8 * part;
+    const half8 ov = *(const half8*)o;
+    const half8 dv = *(const half8*)d;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
+  }
+#pragma unroll
+  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (row < rows && part == 0) {
+    p.negdelta[row] = live ? -acc : 0.f;
+    p.lse2[row] = live ? p.lse[(int64_t)bh * p.T + t] * kLog2e : INFINITY;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // dK / dV
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_f16_kernel(BwdParams p) {
-  constexpr int LD = D + 8;
+__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_kernel(BwdParams p, int BH,
+                                                                   int n_blocks,
+                                                                   int heads_per_xcd) {
+  using Cfg = BwdCfg<D>;
+  constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
+  constexpr int VEC_B = Cfg::VEC_B, SLOT_B = Cfg::SLOT_B;
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
   constexpr int CH = D / 8;
-  constexpr int NLOAD = kBwdStep * CH / 256;
+  constexpr int RPW = 1024 / RB;       // tile rows covered by one wave-wide 1 KiB load
+  constexpr int NWLW = TILE_B / 4096;  // 1 KiB loads per wave per tile
+  // every wave issues the same number of loads per iteration (vmcnt bookkeeping):
+  // Q and dO slabs plus one 256-byte vector (even waves: lse2, odd waves: negdelta)
+  constexpr int LPI = 2 * NWLW + 1;
 
-  __shared__ __attribute__((aligned(16))) half_t Qs[kBwdStep * LD];
-  __shared__ __attribute__((aligned(16))) half_t dOs[kBwdStep * LD];
-  __shared__ __attribute__((aligned(16))) float lse2s[kBwdStep];
-  __shared__ __attribute__((aligned(16))) float deltas[kBwdStep];
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  const int kvblk = blockIdx.x;  // block 0 walks the most query tiles: it goes first
-  const int bh = blockIdx.y;
+
+  int bh, rank;
+  if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  const int kvblk = rank;  // key block 0 walks the most query tiles
   const int b = bh / p.H, h = bh % p.H;
 
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
@@ -64,12 +141,49 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f16_kernel(BwdParams p) {
   const half_t* dO = (const half_t*)p.d_o + b * p.sdo.b + h * p.sdo.h;
   half_t* dK = (half_t*)p.dk + b * p.sdk.b + h * p.sdk.h;
   half_t* dV = (half_t*)p.dv + b * p.sdv.b + h * p.sdv.h;
-  const float* lse = p.lse + (int64_t)bh * T;
-  const float* delta = p.delta + (int64_t)bh * T;
+  const float* lse2 = p.lse2 + (int64_t)bh * p.t_pad;
+  const float* negdelta = p.negdelta + (int64_t)bh * p.t_pad;
 
   const int kv0 = kvblk * kBwdBlk;
   const int kvw0 = kv0 + 32 * wave;
   const int kvrow = kvw0 + (lane & 31);
+
+  const int first_tile = kv0 / kBwdStep;
+  const int n_tiles = (T + kBwdStep - 1) / kBwdStep;  // query tiles first_tile .. n_tiles-1
+
+  // ---- asynchronous loads of query tile t into ring slot t % NS ----
+  const uint32_t lds0 = lds_address(smem);
+  const int sqt = (int)p.sq.t, sdot = (int)p.sdo.t;
+  const int tail_tile = (T - 1) / kBwdStep;
+  uint32_t ld_q[NWLW], ld_do[NWLW], ld_q_tail[NWLW], ld_do_tail[NWLW];
+#pragma unroll
+  for (int i = 0; i < NWLW; ++i) {
+    const int row = (wave * NWLW + i) * RPW + lane / CH;
+    const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
+    const int row_tail = min(row, T - 1 - tail_tile * kBwdStep);
+    ld_q[i] = (uint32_t)(row * sqt * 2 + col);
+    ld_do[i] = (uint32_t)(row * sdot * 2 + col);
+    ld_q_tail[i] = (uint32_t)(row_tail * sqt * 2 + col);
+    ld_do_tail[i] = (uint32_t)(row_tail * sdot * 2 + col);
+  }
+  auto request = [&](int t) {
+    const int tc = min(t, n_tiles - 1);  // clamped repeats are never consumed
+    const uint32_t slot = lds0 + (t % NS) * SLOT_B;
+    const half_t* qbase = Q + (uint32_t)(tc * kBwdStep * sqt);
+    const half_t* dobase = dO + (uint32_t)(tc * kBwdStep * sdot);
+#pragma unroll
+    for (int i = 0; i < NWLW; ++i) {
+      const uint32_t dst = slot + (wave * NWLW + i) * 1024;
+      async_load16_to_lds(qbase, tc == tail_tile ? ld_q_tail[i] : ld_q[i], dst);
+      async_load16_to_lds(dobase, tc == tail_tile ? ld_do_tail[i] : ld_do[i], dst + TILE_B);
+    }
+    // per-row vectors (the workspace rows are padded, no clamp needed)
+    const float* vec = ((wave & 1) ? negdelta : lse2) + tc * kBwdStep;
+    async_load4_to_lds(vec, lane * 4, slot + 2 * TILE_B + (wave & 1) * VEC_B);
+  };
+
+#pragma unroll
+  for (int i = 0; i < P; ++i) request(first_tile + i);
 
   // K^T and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.
   half8 kf[KS], vf[KS];
@@ -84,112 +198,107 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f16_kernel(BwdParams p) {
     }
   }
 
+  // ---- per-lane swizzled read offsets (bytes within a tile) ----
+  int aoff[KS];  // row-major A operand: row lane%32 (+32 for the second block), chunk 2ks+g
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    aoff[ks] = (lane & 31) * RB + (((2 * ks + g) ^ lds_swizzle<CH>(lane & 31)) << 4);
+  int toff_lo[DB], toff_hi[DB];  // transposed A operand (see lds_read_tr16)
+  {
+    const int lrow = 4 * g + ((lane & 15) >> 2);
+    const int c4 = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + (c4 >> 1);
+      toff_lo[db] = lrow * RB + ((chunk ^ lds_swizzle<CH>(lrow)) << 4) + (c4 & 1) * 8;
+      toff_hi[db] = (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
+    }
+  }
+
   floatx16 dkacc[DB], dvacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) {
     dkacc[i] = ZERO16;
     dvacc[i] = ZERO16;
   }
+  const float c = p.scale_log2;
 
-  const int first_tile = kv0 / kBwdStep;
-  const int n_tiles = (T + kBwdStep - 1) / kBwdStep;
-
-  half8 qreg[NLOAD], doreg[NLOAD];
-  float lreg = 0.f, dreg = 0.f;
-  auto prefetch = [&](int tile) {
-    const int q0 = tile * kBwdStep;
+  // One 32-query block of the tile in `slot`: MASKED applies the causal element mask.
+  auto block = [&](auto masked, const char* slot, int mb, int qb0) {
+    constexpr bool MASKED = decltype(masked)::value;
+    const char* Qt = slot + 32 * mb * RB;
+    const char* dOt = slot + TILE_B + 32 * mb * RB;
+    const float* l2v = (const float*)(slot + 2 * TILE_B) + 32 * mb + 4 * g;
+    const float* ndv = (const float*)(slot + 2 * TILE_B + VEC_B) + 32 * mb + 4 * g;
+    // dP starts from -delta[q] (row value of every accumulator register)
+    floatx16 s = ZERO16, dp;
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const int idx = tid + 256 * i;
-      const int row = idx / CH, ch = idx % CH;
-      const int qr = q0 + row;
-      if (qr < T) {
-        qreg[i] = *(const half8*)(Q + (int64_t)qr * p.sq.t + 8 * ch);
-        doreg[i] = *(const half8*)(dO + (int64_t)qr * p.sdo.t + 8 * ch);
-      } else {
-        qreg[i] = ZEROH8;
-        doreg[i] = ZEROH8;
+    for (int rq = 0; rq < 4; ++rq) {
+      const floatx4 nd = *(const floatx4*)(ndv + 8 * rq);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dp[4 * rq + e] = nd[e];
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      s = mfma_f16(*(const half8*)(Qt + aoff[ks]), kf[ks], s);
+      dp = mfma_f16(*(const half8*)(dOt + aoff[ks]), vf[ks], dp);
+    }
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const floatx4 l4 = *(const floatx4*)(l2v + 8 * rq);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int r = 4 * rq + e;
+        float pv = fast_exp2(__builtin_fmaf(s[r], c, -l4[e]));
+        if constexpr (MASKED) {
+          if (kvrow > qb0 + 8 * rq + 4 * g + e) pv = 0.f;
+        }
+        s[r] = pv;
+        dp[r] = pv * dp[r];
       }
     }
-    if (tid < kBwdStep) {
-      const int qr = q0 + tid;
-      lreg = qr < T ? lse[qr] * kLog2e : 0.f;
-      dreg = qr < T ? delta[qr] : 0.f;
-    }
-  };
-  auto commit = [&]() {
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const int idx = tid + 256 * i;
-      const int row = idx / CH, ch = idx % CH;
-      *(half8*)(Qs + row * LD + 8 * ch) = qreg[i];
-      *(half8*)(dOs + row * LD + 8 * ch) = doreg[i];
-    }
-    if (tid < kBwdStep) {
-      lse2s[tid] = lreg;
-      deltas[tid] = dreg;
+    for (int st = 0; st < 2; ++st) {
+      const half8 pf = pack_half8(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                                  s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+      const half8 dsf =
+          pack_half8(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
+                     dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const char* tb = dOt + 16 * st * RB;
+        const half4 lo = lds_read_tr16((const half_t*)(tb + toff_lo[db]));
+        const half4 hi = lds_read_tr16((const half_t*)(tb + toff_hi[db]));
+        dvacc[db] = mfma_f16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf,
+                             dvacc[db]);
+        const char* tq = Qt + 16 * st * RB;
+        const half4 qlo = lds_read_tr16((const half_t*)(tq + toff_lo[db]));
+        const half4 qhi = lds_read_tr16((const half_t*)(tq + toff_hi[db]));
+        dkacc[db] = mfma_f16(__builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7), dsf,
+                             dkacc[db]);
+      }
     }
   };
 
-  if (first_tile < n_tiles) prefetch(first_tile);
+  constexpr std::true_type yes{};
+  constexpr std::false_type no{};
   for (int j = first_tile; j < n_tiles; ++j) {
+    // tile j was requested P iterations ago; at most the P-1 younger groups may
+    // still be in flight.  The barrier also retires all reads of the slot that the
+    // next request overwrites (tile j-1's).
+    wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
-    commit();
-    __syncthreads();
-    if (j + 1 < n_tiles) prefetch(j + 1);
-
+    request(j + P);
+    const char* slot = smem + (j % NS) * SLOT_B;
     const int q0 = j * kBwdStep;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
-      const int qb0 = q0 + 32 * mb;        // first query row of this 32-block
-      if (qb0 + 31 < kvw0) continue;       // every query here precedes the wave's keys
-
-      // S[q, kv] and dP[q, kv]
-      floatx16 s = ZERO16, dp = ZERO16;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const half8 aq = *(const half8*)(Qs + (32 * mb + (lane & 31)) * LD + 16 * ks + 8 * g);
-        s = mfma_f16(aq, kf[ks], s);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const half8 ad = *(const half8*)(dOs + (32 * mb + (lane & 31)) * LD + 16 * ks + 8 * g);
-        dp = mfma_f16(ad, vf[ks], dp);
-      }
-
-      const bool need_mask = (qb0 < kvw0 + 31);
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const floatx4 l4 = *(const floatx4*)(lse2s + 32 * mb + 8 * rq + 4 * g);
-        const floatx4 d4 = *(const floatx4*)(deltas + 32 * mb + 8 * rq + 4 * g);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * rq + e;
-          float pv = fast_exp2(s[r] * p.scale_log2 - l4[e]);
-          if (need_mask) {
-            const int qr = qb0 + 8 * rq + 4 * g + e;
-            if (kvrow > qr) pv = 0.f;
-          }
-          s[r] = pv;
-          dp[r] = pv * (dp[r] - d4[e]);
-        }
-      }
-
-#pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        const half8 pf = pack_half8(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                                    s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
-        const half8 dsf =
-            pack_half8(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
-                       dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const half8 dot = lds_frag_transposed(dOs, LD, 32 * mb + 16 * st, 32 * db, lane);
-          dvacc[db] = mfma_f16(dot, pf, dvacc[db]);
-          const half8 qt = lds_frag_transposed(Qs, LD, 32 * mb + 16 * st, 32 * db, lane);
-          dkacc[db] = mfma_f16(qt, dsf, dkacc[db]);
-        }
-      }
+      const int qb0 = q0 + 32 * mb;   // first query row of this 32-block
+      if (qb0 + 31 < kvw0) continue;  // every query here precedes the wave's keys
+      if (qb0 < kvw0 + 31)
+        block(yes, slot, mb, qb0);
+      else
+        block(no, slot, mb, qb0);
     }
   }
 
@@ -216,23 +325,28 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f16_kernel(BwdParams p) {
 // dQ
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dq_f16_kernel(BwdParams p) {
-  constexpr int LD = D + 8;
+__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kernel(BwdParams p, int BH, int n_blocks,
+                                                                 int heads_per_xcd) {
+  using Cfg = BwdCfg<D>;
+  constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
   constexpr int CH = D / 8;
-  constexpr int NLOAD = kBwdStep * CH / 256;
+  constexpr int RPW = 1024 / RB;
+  constexpr int NWLW = TILE_B / 4096;
+  constexpr int LPI = 2 * NWLW;
 
-  __shared__ __attribute__((aligned(16))) half_t Ks[kBwdStep * LD];
-  __shared__ __attribute__((aligned(16))) half_t Vs[kBwdStep * LD];
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  const int qtile = gridDim.x - 1 - blockIdx.x;  // longest rows first
-  const int bh = blockIdx.y;
+
+  int bh, rank;
+  if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  const int qtile = n_blocks - 1 - rank;  // the last query block walks the most key tiles
   const int b = bh / p.H, h = bh % p.H;
 
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
@@ -245,6 +359,40 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f16_kernel(BwdParams p) {
   const int qw0 = q0 + 32 * wave;
   const int qrow = qw0 + (lane & 31);
 
+  int last_q = q0 + kBwdBlk - 1;
+  if (last_q > T - 1) last_q = T - 1;
+  const int n_tiles = last_q / kBwdStep + 1;
+
+  // ---- asynchronous loads of key/value tile t into ring slot t % NS ----
+  const uint32_t lds0 = lds_address(smem);
+  const int skt = (int)p.sk.t, svt = (int)p.sv.t;
+  const int tail_tile = (T - 1) / kBwdStep;
+  uint32_t ld_k[NWLW], ld_v[NWLW], ld_k_tail[NWLW], ld_v_tail[NWLW];
+#pragma unroll
+  for (int i = 0; i < NWLW; ++i) {
+    const int row = (wave * NWLW + i) * RPW + lane / CH;
+    const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
+    const int row_tail = min(row, T - 1 - tail_tile * kBwdStep);
+    ld_k[i] = (uint32_t)(row * skt * 2 + col);
+    ld_v[i] = (uint32_t)(row * svt * 2 + col);
+    ld_k_tail[i] = (uint32_t)(row_tail * skt * 2 + col);
+    ld_v_tail[i] = (uint32_t)(row_tail * svt * 2 + col);
+  }
+  auto request = [&](int t) {
+    const int tc = min(t, n_tiles - 1);
+    const uint32_t slot = lds0 + (t % NS) * 2 * TILE_B;
+    const half_t* kbase = K + (uint32_t)(tc * kBwdStep * skt);
+    const half_t* vbase = V + (uint32_t)(tc * kBwdStep * svt);
+#pragma unroll
+    for (int i = 0; i < NWLW; ++i) {
+      const uint32_t dst = slot + (wave * NWLW + i) * 1024;
+      async_load16_to_lds(kbase, tc == tail_tile ? ld_k_tail[i] : ld_k[i], dst);
+      async_load16_to_lds(vbase, tc == tail_tile ? ld_v_tail[i] : ld_v[i], dst + TILE_B);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < P; ++i) request(i);
+
   half8 qf[KS], dof[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -256,93 +404,85 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f16_kernel(BwdParams p) {
       dof[ks] = ZEROH8;
     }
   }
-  const float lse2 = qrow < T ? p.lse[(int64_t)bh * T + qrow] * kLog2e : 0.f;
-  const float dlt = qrow < T ? p.delta[(int64_t)bh * T + qrow] : 0.f;
+  // padded rows read lse2 = +inf / negdelta = 0 from the padded workspace: P = 0
+  const int qclamp = min(qrow, p.t_pad - 1);
+  const float l2 = p.lse2[(int64_t)bh * p.t_pad + qclamp];
+  const float nd = p.negdelta[(int64_t)bh * p.t_pad + qclamp];
+  floatx16 nd16;  // initial value of every dP^T accumulator: -delta of this lane's query
+#pragma unroll
+  for (int r = 0; r < 16; ++r) nd16[r] = nd;
+
+  int aoff[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    aoff[ks] = (lane & 31) * RB + (((2 * ks + g) ^ lds_swizzle<CH>(lane & 31)) << 4);
+  int toff_lo[DB], toff_hi[DB];
+  {
+    const int lrow = 4 * g + ((lane & 15) >> 2);
+    const int c4 = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + (c4 >> 1);
+      toff_lo[db] = lrow * RB + ((chunk ^ lds_swizzle<CH>(lrow)) << 4) + (c4 & 1) * 8;
+      toff_hi[db] = (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
+    }
+  }
 
   floatx16 dqacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) dqacc[i] = ZERO16;
+  const float c = p.scale_log2;
 
-  int last_q = q0 + kBwdBlk - 1;
-  if (last_q > T - 1) last_q = T - 1;
-  const int n_tiles = last_q / kBwdStep + 1;
-
-  half8 kreg[NLOAD], vreg[NLOAD];
-  auto prefetch = [&](int tile) {
-    const int kv0 = tile * kBwdStep;
+  auto block = [&](auto masked, const char* slot, int mb, int kvb0) {
+    constexpr bool MASKED = decltype(masked)::value;
+    const char* Kt = slot + 32 * mb * RB;
+    const char* Vt = slot + TILE_B + 32 * mb * RB;
+    floatx16 s = ZERO16, dp = nd16;
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const int idx = tid + 256 * i;
-      const int row = idx / CH, ch = idx % CH;
-      const int kv = kv0 + row;
-      if (kv < T) {
-        kreg[i] = *(const half8*)(K + (int64_t)kv * p.sk.t + 8 * ch);
-        vreg[i] = *(const half8*)(V + (int64_t)kv * p.sv.t + 8 * ch);
-      } else {
-        kreg[i] = ZEROH8;
-        vreg[i] = ZEROH8;
+    for (int ks = 0; ks < KS; ++ks) {
+      s = mfma_f16(*(const half8*)(Kt + aoff[ks]), qf[ks], s);
+      dp = mfma_f16(*(const half8*)(Vt + aoff[ks]), dof[ks], dp);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float pv = fast_exp2(__builtin_fmaf(s[r], c, -l2));
+      if constexpr (MASKED) {
+        if (kvb0 + 8 * (r >> 2) + 4 * g + (r & 3) > qrow) pv = 0.f;
+      }
+      dp[r] = pv * dp[r];
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const half8 dsf =
+          pack_half8(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
+                     dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const char* tb = Kt + 16 * st * RB;
+        const half4 lo = lds_read_tr16((const half_t*)(tb + toff_lo[db]));
+        const half4 hi = lds_read_tr16((const half_t*)(tb + toff_hi[db]));
+        dqacc[db] = mfma_f16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), dsf,
+                             dqacc[db]);
       }
     }
   };
-  auto commit = [&]() {
-#pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const int idx = tid + 256 * i;
-      const int row = idx / CH, ch = idx % CH;
-      *(half8*)(Ks + row * LD + 8 * ch) = kreg[i];
-      *(half8*)(Vs + row * LD + 8 * ch) = vreg[i];
-    }
-  };
 
-  prefetch(0);
+  constexpr std::true_type yes{};
+  constexpr std::false_type no{};
   for (int j = 0; j < n_tiles; ++j) {
+    wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
-    commit();
-    __syncthreads();
-    if (j + 1 < n_tiles) prefetch(j + 1);
-
+    request(j + P);
+    const char* slot = smem + (j % NS) * 2 * TILE_B;
     const int kv0 = j * kBwdStep;
-    if (kv0 > qw0 + 31) continue;
-
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
       const int kvb0 = kv0 + 32 * mb;
-      if (kvb0 > qw0 + 31) continue;
-
-      floatx16 s = ZERO16, dp = ZERO16;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const half8 ak = *(const half8*)(Ks + (32 * mb + (lane & 31)) * LD + 16 * ks + 8 * g);
-        s = mfma_f16(ak, qf[ks], s);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const half8 av = *(const half8*)(Vs + (32 * mb + (lane & 31)) * LD + 16 * ks + 8 * g);
-        dp = mfma_f16(av, dof[ks], dp);
-      }
-
-      const bool need_mask = (kvb0 + 31 > qw0);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float pv = fast_exp2(s[r] * p.scale_log2 - lse2);
-        if (need_mask) {
-          const int kv = kvb0 + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (kv > qrow) pv = 0.f;
-        }
-        dp[r] = pv * (dp[r] - dlt);
-      }
-
-#pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        const half8 dsf =
-            pack_half8(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
-                       dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const half8 kt = lds_frag_transposed(Ks, LD, 32 * mb + 16 * st, 32 * db, lane);
-          dqacc[db] = mfma_f16(kt, dsf, dqacc[db]);
-        }
-      }
+      if (kvb0 > qw0 + 31) continue;  // block lies entirely in this wave's future
+      if (kvb0 + 31 > qw0)
+        block(yes, slot, mb, kvb0);
+      else
+        block(no, slot, mb, kvb0);
     }
   }
 
@@ -362,22 +502,38 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f16_kernel(BwdParams p) {
 
 template <int D>
 static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
-  const int64_t rows = (int64_t)B * p.H * p.T;
+  const int BH = B * p.H;
   constexpr int LPR = D / 8;
-  const int64_t threads = rows * LPR;
+  const int64_t threads = (int64_t)BH * p.t_pad * LPR;
   {
-    LaunchScope scope("attn_bwd_delta", stream);
-    hipLaunchKernelGGL((attn_bwd_delta_kernel<half_t, D>), dim3((threads + 255) / 256),
-                       dim3(256), 0, stream, p, B);
+    LaunchScope scope("attn_bwd_prep", stream);
+    hipLaunchKernelGGL(attn_bwd_prep_f16_kernel<D>, dim3((threads + 255) / 256), dim3(256), 0,
+                       stream, p, B);
   }
-  dim3 grid((p.T + kBwdBlk - 1) / kBwdBlk, B * p.H);
+  const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
+  const int heads_per_xcd = (BH + 7) / 8;
+  const dim3 grid(8 * n_blocks * heads_per_xcd);
+  static bool attr_set = false;  // launches are serialised by the caller
+  if (!attr_set) {
+    if (BwdCfg<D>::kLdsDkdv > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dkdv_f16_kernel<D>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)BwdCfg<D>::kLdsDkdv);
+    if (BwdCfg<D>::kLdsDq > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_f16_kernel<D>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)BwdCfg<D>::kLdsDq);
+    attr_set = true;
+  }
   {
     LaunchScope scope("attn_bwd_dkdv_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_dkdv_f16_kernel<D>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(attn_bwd_dkdv_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDkdv, stream,
+                       p, BH, n_blocks, heads_per_xcd);
   }
   {
     LaunchScope scope("attn_bwd_dq_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_dq_f16_kernel<D>, grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(attn_bwd_dq_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDq, stream, p,
+                       BH, n_blocks, heads_per_xcd);
   }
 }
 

@@ -40,7 +40,19 @@ __device__ __forceinline__ floatx16 mfma_f32(float a, float b, floatx16 c) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// Exchange with the lane 32 away (the other half of the wave).
+// Reductions over the lane pair (l, l^32) with v_permlane32_swap: called with
+// (x, x) it returns {low half broadcast to both halves, high half broadcast}.
+__device__ __forceinline__ float pair_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// Kept for the f32 kernels: exchange with the lane 32 away.
 __device__ __forceinline__ float swap32(float x) { return __shfl_xor(x, 32, 64); }
 
 // ds_read_b64_tr_b16: within each group of 16 lanes, lane 4r+c supplies the
@@ -67,12 +79,81 @@ __device__ __forceinline__ half8 lds_frag_transposed(const half_t* tile, int ld,
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Asynchronous global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4):
+// lane i's 16 bytes land at lds_addr + 16*i, where lds_addr is a wave-uniform LDS
+// byte address.  Completion is tracked by vmcnt; pair with wait_vmcnt<N>() and a
+// barrier before other waves read the data.
+__device__ __forceinline__ void async_load16_to_lds(const void* gptr, uint32_t lds_addr) {
+  const uint32_t uniform = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(uniform)
+               : "memory");
+}
+// Same copy with the address split into a wave-uniform 64-bit base (SGPR pair) and a
+// per-lane unsigned 32-bit byte offset, so advancing to the next tile is scalar work.
+__device__ __forceinline__ void async_load16_to_lds(const void* uniform_base, uint32_t lane_off,
+                                                    uint32_t lds_addr) {
+  const uint32_t uniform = __builtin_amdgcn_readfirstlane(lds_addr);
+  const uint64_t b = (uint64_t)uniform_base;
+  // readfirstlane returns a signed int: widen through uint32_t, never sign-extend
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sbase = ((uint64_t)hi << 32) | (uint64_t)lo;
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sbase),
+               "s"(uniform)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(size_t)(DEERS_LDS const void*)p;
+}
+
+// XOR swizzle of 16-byte chunks for unpadded row-major f16 tiles in LDS (rows of
+// CH chunks).  Chunk c of row r is stored at chunk position c ^ lds_swizzle(r), so
+// that 8 consecutive rows read at the same logical chunk hit 8 different 16-byte
+// bank groups.  Invariant under r -> r + 32 (and r + 16 for CH <= 16).
+template <int CH>
+__device__ __forceinline__ int lds_swizzle(int row) {
+  // Two access patterns must be conflict-free.  (a) 16-byte reads by 16 lanes on 16
+  // consecutive rows at one logical chunk: rows that share a 256-byte bank line
+  // position need distinct swizzles.  (b) transposed 8-byte reads by 32 lanes on 4
+  // consecutive rows x 4 consecutive chunks: rows on the same bank line position
+  // must move the aligned group of 4 chunks as a whole, i.e. differ in chunk bit 2+.
+  if constexpr (CH == 4) return (row >> 2) & 3;  // 4 rows per bank line
+  if constexpr (CH == 8) {                       // 2 rows per bank line
+    const int t = (row >> 1) & 7;
+    return ((t & 1) << 2) | (t >> 1);
+  }
+  return ((row & 3) << 2) | ((row >> 2) & 3);    // CH == 16: every row on the same banks
+}
+
+// 4 bytes per lane variant (global_load_lds_dword): lane i's dword lands at
+// lds_addr + 4*i.
+__device__ __forceinline__ void async_load4_to_lds(const void* uniform_base, uint32_t lane_off,
+                                                   uint32_t lds_addr) {
+  const uint32_t uniform = __builtin_amdgcn_readfirstlane(lds_addr);
+  const uint64_t b = (uint64_t)uniform_base;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sbase = ((uint64_t)hi << 32) | (uint64_t)lo;
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_off), "s"(sbase),
+               "s"(uniform)
+               : "memory");
+}
+
 __device__ __forceinline__ half8 pack_half8(float a0, float a1, float a2, float a3, float a4,
                                             float a5, float a6, float a7) {
   half8 r;
   r[0] = (half_t)a0; r[1] = (half_t)a1; r[2] = (half_t)a2; r[3] = (half_t)a3;
   r[4] = (half_t)a4; r[5] = (half_t)a5; r[6] = (half_t)a6; r[7] = (half_t)a7;
   return r;
+}
+
+// sum += a.x + a.y in f32 (v_dot2_f32_f16 against (1,1)).
+__device__ __forceinline__ float add_half2(half2v a, float sum) {
+  return __builtin_amdgcn_fdot2(a, half2v{(half_t)1.f, (half_t)1.f}, sum, false);
 }
 
 // Element strides of one [B,H,T,D] tensor (D stride is 1).
@@ -90,6 +171,9 @@ struct FwdParams {
 struct BwdParams {
   const void* q; const void* k; const void* v; const void* o; const void* d_o;
   const float* lse; float* delta;  // delta: [B,H,T] workspace, rowsum(dO o O)
+  // f16 path workspace, rows padded to a multiple of 64 per head (t_pad):
+  // lse2 = LSE*log2(e) (+inf in the padding), negdelta = -rowsum(dO o O) (0 in the padding)
+  float* lse2; float* negdelta; int t_pad;
   void* dq; void* dk; void* dv;
   Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
   int H, T;

@@ -107,6 +107,11 @@ int resolve_strides(const char* name, const void* ptr, const int64_t* strides, i
     return fail(DEERS_ROCM_ERR_LAYOUT,
                 "%s: rows must be 16-byte aligned (ptr %p, strides %lld,%lld,%lld)", name, ptr,
                 (long long)sb, (long long)sh, (long long)st);
+  if (sb < 0 || sh < 0 || st < D || T * st >= (int64_t(1) << 30))
+    return fail(DEERS_ROCM_ERR_LAYOUT,
+                "%s: strides must be non-negative, rows must not overlap and T * row stride "
+                "must stay below 2^30 elements (strides %lld,%lld,%lld)",
+                name, (long long)sb, (long long)sh, (long long)st);
   out->b = sb;
   out->h = sh;
   out->t = st;
@@ -123,6 +128,14 @@ int check_problem(int dtype, int64_t B, int64_t H, int64_t T, int64_t D) {
     return fail(DEERS_ROCM_ERR_ARG, "head dim %lld unsupported (32, 64 or 128)", (long long)D);
   if (B * H > 65535 || T > (int64_t(1) << 24))
     return fail(DEERS_ROCM_ERR_ARG, "B*H must be <= 65535 and T <= 2^24");
+  return DEERS_ROCM_OK;
+}
+
+// The kernels track the running maximum on raw scores and apply the scale inside
+// the exponent, which needs scale > 0 (the reference uses 1/sqrt(D)).
+int check_scale(float scale) {
+  if (!(scale > 0.f) || !std::isfinite(scale))
+    return fail(DEERS_ROCM_ERR_ARG, "scale must be positive and finite (got %g)", (double)scale);
   return DEERS_ROCM_OK;
 }
 
@@ -375,6 +388,7 @@ int deers_rocm_attn_fwd(int dtype, const void* q, const int64_t* q_strides, cons
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   if (int rc = check_problem(dtype, B, H, T, D)) return rc;
+  if (int rc = check_scale(scale)) return rc;
   if (!lse) return fail(DEERS_ROCM_ERR_ARG, "attn_fwd: null lse");
   const size_t elem = dtype == DEERS_ROCM_F16 ? 2 : 4;
   deers::FwdParams p{};
@@ -403,6 +417,7 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   if (int rc = check_problem(dtype, B, H, T, D)) return rc;
+  if (int rc = check_scale(scale)) return rc;
   if (!lse) return fail(DEERS_ROCM_ERR_ARG, "attn_bwd: null lse");
   const size_t elem = dtype == DEERS_ROCM_F16 ? 2 : 4;
   deers::BwdParams p{};
@@ -414,10 +429,16 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   if (int rc = resolve_strides("dq", dq, dq_strides, H, T, D, elem, &p.sdq)) return rc;
   if (int rc = resolve_strides("dk", dk, dk_strides, H, T, D, elem, &p.sdk)) return rc;
   if (int rc = resolve_strides("dv", dv, dv_strides, H, T, D, elem, &p.sdv)) return rc;
+  // f32: delta[B,H,T].  f16: lse2 and negdelta, rows padded to a multiple of 64 per head.
+  const int64_t t_pad = (T + 63) / 64 * 64;
+  const size_t ws_floats = dtype == DEERS_ROCM_F16 ? (size_t)(2 * B * H * t_pad) : (size_t)(B * H * T);
   void* ws = nullptr;
-  if (int rc = workspace((size_t)(B * H * T) * sizeof(float), &ws)) return rc;
+  if (int rc = workspace(ws_floats * sizeof(float), &ws)) return rc;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
   p.delta = static_cast<float*>(ws);
+  p.lse2 = static_cast<float*>(ws);
+  p.negdelta = static_cast<float*>(ws) + B * H * t_pad;
+  p.t_pad = (int)t_pad;
   p.dq = dq; p.dk = dk; p.dv = dv;
   p.H = (int)H; p.T = (int)T;
   p.scale = scale;
@@ -443,6 +464,7 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
     return fail(DEERS_ROCM_ERR_ARG, "attn_decode: head dim %lld unsupported (64 or 128)",
                 (long long)D);
   if (!q || !k_cache || !v_cache || !o) return fail(DEERS_ROCM_ERR_ARG, "attn_decode: null pointer");
+  if (int rc = check_scale(scale)) return rc;
   deers::DecodeParams p{};
   p.skb = H * L * D; p.skh = L * D; p.skl = D;
   if (kv_strides) { p.skb = kv_strides[0]; p.skh = kv_strides[1]; p.skl = kv_strides[2]; }
