@@ -7,23 +7,22 @@
 //     dP = dO V^T                           dS = P o (dP - delta),  delta = rowsum(dO o O)
 //     dQ = scale dS K                       dK = scale dS^T Q
 //
-// Three launches, no atomics, bit-reproducible:
-//   1. prep    : negdelta[b,h,t] = -sum_d dO*O and lse2 = LSE*log2(e), both f32 in a
-//                workspace whose rows are padded to a multiple of 64 per head
-//                (lse2 = +inf, negdelta = 0 in the padding, so padded query rows
-//                get probability exactly 0).
+// Two launches, no atomics, bit-reproducible (dQ runs first and publishes, for the
+// rows it owns, negdelta[b,h,t] = -sum_d dO*O and lse2 = LSE*log2(e) as f32 in a
+// workspace whose rows are padded to a multiple of 64 per head, with lse2 = +inf and
+// negdelta = 0 in the padding so padded query rows get probability exactly 0):
 //   2. dK/dV   : a workgroup owns 128 key rows (32 per wave, K^T and V^T held in
 //                registers as B operands) and walks the 64-row query tiles at or
 //                below the diagonal.  Orientation S[q,kv] (one key column per lane)
 //                so P and dS leave the accumulators directly as B operands of
 //                dV^T += dO^T P and dK^T += Q^T dS; dO^T / Q^T fragments come
 //                from the row-major LDS tiles via ds_read_b64_tr_b16.
-//   3. dQ      : a workgroup owns 128 query rows (32 per wave, Q and dO in
+//   1. dQ      : a workgroup owns 128 query rows (32 per wave, Q and dO in
 //                registers) and walks 64-row key tiles up to the diagonal.
 //                Orientation S^T[kv,q] (one query column per lane, LSE and delta are
 //                per-lane scalars); dS^T leaves the accumulators as the B operand of
 //                dQ^T += K^T dS^T with K^T fragments read transposed from LDS.
-// Recomputing S and dP in both 2 and 3 costs 7 tile GEMMs instead of 5 but
+// Recomputing S and dP in both kernels costs 7 tile GEMMs instead of 5 but
 // keeps every product in registers and needs no dQ accumulation buffer.
 //
 // The "- delta" of dS is folded into the dP accumulator's initial value, so the
@@ -70,37 +69,6 @@ __device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int B
   *bh = (idx % heads_per_xcd) * 8 + xcd;
   *rank = idx / heads_per_xcd;
   return *bh < BH;
-}
-
-// ---------------------------------------------------------------------------
-// prep: negdelta and lse2, LPR lanes share one row.
-// ---------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_prep_f16_kernel(BwdParams p, int B) {
-  constexpr int LPR = D / 8;  // lanes per row
-  const int64_t rows = (int64_t)B * p.H * p.t_pad;
-  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
-  const int part = threadIdx.x % LPR;
-  float acc = 0.f;
-  const int t = row < rows ? (int)(row % p.t_pad) : 0;
-  const int bh = row < rows ? (int)(row / p.t_pad) : 0;
-  const bool live = row < rows && t < p.T;
-  if (live) {
-    const int b = bh / p.H, h = bh % p.H;
-    const half_t* o = (const half_t*)p.o + b * p.so.b + h * p.so.h + (int64_t)t * p.so.t + 8 * part;
-    const half_t* d =
-        (const half_t*)p.d_o + b * p.sdo.b + h * p.sdo.h + (int64_t)t * p.sdo.t + 8 * part;
-    const half8 ov = *(const half8*)o;
-    const half8 dv = *(const half8*)d;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv[e];
-  }
-#pragma unroll
-  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (row < rows && part == 0) {
-    p.negdelta[row] = live ? -acc : 0.f;
-    p.lse2[row] = live ? p.lse[(int64_t)bh * p.T + t] * kLog2e : INFINITY;
-  }
 }
 
 // ---------------------------------------------------------------------------
@@ -394,20 +362,29 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   for (int i = 0; i < P; ++i) request(i);
 
   half8 qf[KS], dof[KS];
+  float dsum = 0.f;  // this lane's half of rowsum(dO o O)
+  const half_t* O = (const half_t*)p.o + b * p.so.b + h * p.so.h;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     if (qrow < T) {
       qf[ks] = *(const half8*)(Q + (int64_t)qrow * p.sq.t + 16 * ks + 8 * g);
       dof[ks] = *(const half8*)(dO + (int64_t)qrow * p.sdo.t + 16 * ks + 8 * g);
+      const half8 of = *(const half8*)(O + (int64_t)qrow * p.so.t + 16 * ks + 8 * g);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dsum += (float)dof[ks][e] * (float)of[e];
     } else {
       qf[ks] = ZEROH8;
       dof[ks] = ZEROH8;
     }
   }
-  // padded rows read lse2 = +inf / negdelta = 0 from the padded workspace: P = 0
-  const int qclamp = min(qrow, p.t_pad - 1);
-  const float l2 = p.lse2[(int64_t)bh * p.t_pad + qclamp];
-  const float nd = p.negdelta[(int64_t)bh * p.t_pad + qclamp];
+  // Per-row statistics, also published for the dK/dV kernel that runs next: rows in
+  // the padding [T, t_pad) get lse2 = +inf and negdelta = 0, i.e. probability 0.
+  const float nd = -pair_sum(dsum);
+  const float l2 = qrow < T ? p.lse[(int64_t)bh * T + qrow] * kLog2e : INFINITY;
+  if (g == 0 && qrow < p.t_pad) {
+    p.lse2[(int64_t)bh * p.t_pad + qrow] = l2;
+    p.negdelta[(int64_t)bh * p.t_pad + qrow] = nd;
+  }
   floatx16 nd16;  // initial value of every dP^T accumulator: -delta of this lane's query
 #pragma unroll
   for (int r = 0; r < 16; ++r) nd16[r] = nd;
@@ -503,13 +480,6 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
 template <int D>
 static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
   const int BH = B * p.H;
-  constexpr int LPR = D / 8;
-  const int64_t threads = (int64_t)BH * p.t_pad * LPR;
-  {
-    LaunchScope scope("attn_bwd_prep", stream);
-    hipLaunchKernelGGL(attn_bwd_prep_f16_kernel<D>, dim3((threads + 255) / 256), dim3(256), 0,
-                       stream, p, B);
-  }
   const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
   const int heads_per_xcd = (BH + 7) / 8;
   const dim3 grid(8 * n_blocks * heads_per_xcd);
@@ -525,15 +495,16 @@ static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
                                 (int)BwdCfg<D>::kLdsDq);
     attr_set = true;
   }
-  {
-    LaunchScope scope("attn_bwd_dkdv_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_dkdv_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDkdv, stream,
-                       p, BH, n_blocks, heads_per_xcd);
-  }
+  // dQ first: it also publishes lse2 / negdelta for the dK/dV kernel
   {
     LaunchScope scope("attn_bwd_dq_f16", stream);
     hipLaunchKernelGGL(attn_bwd_dq_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDq, stream, p,
                        BH, n_blocks, heads_per_xcd);
+  }
+  {
+    LaunchScope scope("attn_bwd_dkdv_f16", stream);
+    hipLaunchKernelGGL(attn_bwd_dkdv_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDkdv, stream,
+                       p, BH, n_blocks, heads_per_xcd);
   }
 }
 
