@@ -43,7 +43,7 @@ def attn_flops(B, H, T, D):
     return fwd, 2.5 * fwd
 
 
-def bench_train(steps: int, warmup: int):
+def bench_train(steps: int, warmup: int, only: str = "all"):
     B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
     x = synth.attention_inputs("c2", B, H, T, D, np.float16, base_seed=0)
     q, k, v, do = (rocm.DeviceBuffer.from_numpy(x[n]) for n in ("q", "k", "v", "do"))
@@ -52,10 +52,20 @@ def bench_train(steps: int, warmup: int):
     dq, dk, dv = (rocm.DeviceBuffer((B, H, T, D), np.float16) for _ in range(3))
     scale = rocm.default_scale(D)
 
-    def step():
+    def fwd():
         rocm.attn_fwd_raw(np.float16, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, B, H, T, D, scale)
+
+    def bwd():
         rocm.attn_bwd_raw(np.float16, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, do.ptr, dq.ptr, dk.ptr,
                           dv.ptr, B, H, T, D, scale)
+
+    fwd()  # the backward needs a forward's O and LSE whatever is timed
+
+    def step():
+        if only in ("all", "fwd"):
+            fwd()
+        if only in ("all", "bwd"):
+            bwd()
 
     for _ in range(warmup):
         step()
@@ -148,6 +158,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode"], default="all",
+                    help="profiling aid: launch only this part and print its kernel times "
+                         "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the attention path has no cross-GPU exchange "
@@ -155,6 +168,14 @@ def main():
     if not rocm.available():
         sys.exit("no gfx950 device visible: the attention path has no CPU fallback")
     rocm.init(0)
+
+    if args.only != "all":
+        if args.only == "decode":
+            print(json.dumps({"only": "decode", **bench_decode(args.steps, args.warmup)}))
+        else:
+            tr = bench_train(args.steps, args.warmup, args.only)
+            print(json.dumps({"only": args.only, "kernels": tr["kernels"]}))
+        return
 
     B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
     fwd_f, bwd_f = attn_flops(B, H, T, D)
