@@ -41,6 +41,10 @@ constexpr int kBwdStep = 64;  // rows of the streamed operand per iteration
 
 #define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
+// Hook for a timestamp-tracing build of these kernels; expands to nothing in the library.
+#ifndef DEERS_TRACE_POINT
+#define DEERS_TRACE_POINT(slot)
+#endif
 
 template <int D>
 struct BwdCfg {
@@ -53,23 +57,6 @@ struct BwdCfg {
   static constexpr size_t kLdsDkdv = NS * SLOT_B;
   static constexpr size_t kLdsDq = NS * 2 * TILE_B;      // dQ: K, V
 };
-
-// Maps blockIdx.x to (head, block rank) so that a head stays on one XCD and the
-// workgroups an XCD's CUs receive in turn (items i, i+32, i+64, ...) have even
-// total length: the XCD's list is sorted longest first and every second group of
-// 32 is reversed.  rank 0 is the longest block.  Returns false for padding ids.
-__device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int BH, int* bh,
-                                          int* rank) {
-  const int xcd = blockIdx.x & 7;
-  int idx = blockIdx.x >> 3;
-  const int per_xcd = n_blocks * heads_per_xcd;
-  const int grp = idx >> 5, pos = idx & 31;
-  const int grp_len = min(32, per_xcd - 32 * grp);
-  if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
-  *bh = (idx % heads_per_xcd) * 8 + xcd;
-  *rank = idx / heads_per_xcd;
-  return *bh < BH;
-}
 
 // ---------------------------------------------------------------------------
 // dK / dV
@@ -101,6 +88,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
   int bh, rank;
   if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
   const int kvblk = rank;  // key block 0 walks the most query tiles
+  set_block_priority(rank, n_blocks);
   const int b = bh / p.H, h = bh % p.H;
 
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
@@ -112,6 +100,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
   const float* lse2 = p.lse2 + (int64_t)bh * p.t_pad;
   const float* negdelta = p.negdelta + (int64_t)bh * p.t_pad;
 
+  DEERS_TRACE_POINT(0);
   const int kv0 = kvblk * kBwdBlk;
   const int kvw0 = kv0 + 32 * wave;
   const int kvrow = kvw0 + (lane & 31);
@@ -268,6 +257,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
       else
         block(no, slot, mb, qb0);
     }
+    DEERS_TRACE_POINT(2 + j - first_tile);
   }
 
   if (kvrow < T) {
@@ -287,6 +277,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
         *(half4*)(dvrow + 32 * db + 8 * rq + 4 * g) = ov;
       }
   }
+  DEERS_TRACE_POINT(30);
 }
 
 // ---------------------------------------------------------------------------
@@ -315,6 +306,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   int bh, rank;
   if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
   const int qtile = n_blocks - 1 - rank;  // the last query block walks the most key tiles
+  set_block_priority(rank, n_blocks);
   const int b = bh / p.H, h = bh % p.H;
 
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
@@ -323,6 +315,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   const half_t* dO = (const half_t*)p.d_o + b * p.sdo.b + h * p.sdo.h;
   half_t* dQ = (half_t*)p.dq + b * p.sdq.b + h * p.sdq.h;
 
+  DEERS_TRACE_POINT(0);
   const int q0 = qtile * kBwdBlk;
   const int qw0 = q0 + 32 * wave;
   const int qrow = qw0 + (lane & 31);
@@ -461,6 +454,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
       else
         block(no, slot, mb, kvb0);
     }
+    DEERS_TRACE_POINT(2 + j);
   }
 
   if (qrow < T) {
@@ -475,6 +469,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
         *(half4*)(dqrow + 32 * db + 8 * rq + 4 * g) = out;
       }
   }
+  DEERS_TRACE_POINT(30);
 }
 
 template <int D>

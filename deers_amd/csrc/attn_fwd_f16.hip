@@ -186,31 +186,54 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
   float m = -INFINITY, lsum = 0.f;
   const float c = p.scale_log2;
 
+  // Operand fetch and MFMA issue are separate steps: all LDS reads of an iteration
+  // are issued right after its barrier, so their latency is covered by the row-maximum
+  // pass, and the MFMAs later find their fragments in registers.  Reads use explicit
+  // 32-bit LDS addresses (slot base + per-lane offset, one add each per iteration) so
+  // the row-block offsets become instruction immediates.
+  auto load_k = [&](int kt, half8* kfr) {  // kfr[2ks + blk]
+    const uint32_t kb = lds0 + (kt % NS) * TILE_B;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint32_t addr = opaque(kb + koff[ks]);
+      kfr[2 * ks] = *(DEERS_LDS const half8*)(uintptr_t)addr;
+      kfr[2 * ks + 1] = *(DEERS_LDS const half8*)(uintptr_t)(addr + 32 * RB);
+    }
+  };
   // S^T(tile) into (a0, a1): two 32-row blocks, independent accumulators interleaved.
-  auto compute_s = [&](int kt, floatx16& a0, floatx16& a1) {
-    const char* Kt = smem + (kt % NS) * TILE_B;
+  auto mfma_s = [&](const half8* kfr, floatx16& a0, floatx16& a1) {
     a0 = ZERO16;
     a1 = ZERO16;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      a0 = mfma_f16(*(const half8*)(Kt + koff[ks]), qf[ks], a0);
-      a1 = mfma_f16(*(const half8*)(Kt + koff[ks] + 32 * RB), qf[ks], a1);
+      a0 = mfma_f16(kfr[2 * ks], qf[ks], a0);
+      a1 = mfma_f16(kfr[2 * ks + 1], qf[ks], a1);
     }
   };
-
-  half8 pf[4];  // P of the previous tile, packed as B operands: index 2*mb + st
-  auto compute_pv_half = [&](int vt, int mb) {
-    const char* Vt = smem + (NS + vt % NS) * TILE_B;
+  auto load_v = [&](int vt, half8* vfr) {  // vfr[(2mb + st) * DB + db]
+    const uint32_t vb = lds0 + (NS + vt % NS) * TILE_B;
+    uint32_t alo[DB], ahi[DB];
 #pragma unroll
-    for (int st = 0; st < 2; ++st)
+    for (int db = 0; db < DB; ++db) {
+      alo[db] = opaque(vb + voff_lo[db]);
+      ahi[db] = opaque(vb + voff_hi[db]);
+    }
+#pragma unroll
+    for (int ms = 0; ms < 4; ++ms)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const char* base = Vt + (32 * mb + 16 * st) * RB;
-        const half4 lo = lds_read_tr16((const half_t*)(base + voff_lo[db]));
-        const half4 hi = lds_read_tr16((const half_t*)(base + voff_hi[db]));
-        const half8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[db] = mfma_f16(vf, pf[2 * mb + st], oacc[db]);
+        const uint32_t ro = 16 * ms * RB;
+        const half4 lo = lds_read_tr16_at(alo[db] + ro);
+        const half4 hi = lds_read_tr16_at(ahi[db] + ro);
+        vfr[ms * DB + db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
+  };
+  half8 pf[4];  // P of the previous tile, packed as B operands: index 2*mb + st
+  auto mfma_pv = [&](const half8* vfr) {
+#pragma unroll
+    for (int ms = 0; ms < 4; ++ms)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] = mfma_f16(vfr[ms * DB + db], pf[ms], oacc[db]);
   };
 
   // One pipelined iteration: softmax of (c0,c1) = S(j); if HAS_S, S(j+1) into
@@ -229,6 +252,10 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
     request(j + 1 + P, j - 1 + P);
+    half8 kfr[HAS_S ? 2 * KS : 1], vfr[HAS_PV ? 4 * DB : 1];
+    if constexpr (HAS_PV) load_v(j - 1, vfr);
+    if constexpr (HAS_S) load_k(j + 1, kfr);
+    __builtin_amdgcn_sched_barrier(0);  // keep the fetches ahead of the vector work below
 
     if (kv0 + kFwdBN - 1 > qw0) {  // tile reaches past this wave's first row: element mask
 #pragma unroll
@@ -259,11 +286,8 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
     }
     const float mc = m * c;
     // ---- one straight-line block: 16 MFMAs beside the exponentials ----
-    if constexpr (HAS_PV) {
-      compute_pv_half(j - 1, 0);
-      compute_pv_half(j - 1, 1);
-    }
-    if constexpr (HAS_S) compute_s(j + 1, n0, n1);
+    if constexpr (HAS_PV) mfma_pv(vfr);
+    if constexpr (HAS_S) mfma_s(kfr, n0, n1);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       c0[r] = fast_exp2(__builtin_fmaf(c0[r], c, -mc));
@@ -283,15 +307,15 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
 #pragma unroll
       for (int e = 0; e < 8; e += 2)
         lsum = add_half2(half2v{pn[i][e], pn[i][e + 1]}, lsum);
-    // Ask the scheduler for the interleaving: per MFMA, the LDS reads of a later
-    // MFMA, two exponentials and a few plain vector ops.
+    // Ask the scheduler for the interleaving: per MFMA, two exponentials and a few
+    // plain vector ops.
     if constexpr (HAS_PV || HAS_S) {
+      constexpr int NM = (HAS_PV ? 8 : 0) + (HAS_S ? 8 : 0);
 #pragma unroll
-      for (int i = 0; i < (HAS_PV ? 8 : 0) + (HAS_S ? 8 : 0); ++i) {
+      for (int i = 0; i < NM; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // DS read
-        __builtin_amdgcn_sched_group_barrier(0x400, (HAS_PV && HAS_S) ? 2 : 4, 0);  // exp
-        __builtin_amdgcn_sched_group_barrier(0x002, (HAS_PV && HAS_S) ? 4 : 8, 0);  // VALU
+        __builtin_amdgcn_sched_group_barrier(0x400, (NM == 16) ? 2 : 4, 0);  // exp
+        __builtin_amdgcn_sched_group_barrier(0x002, (NM == 16) ? 5 : 10, 0);  // VALU
       }
     }
     // Pin P(j) and the row sum here: without a use in this block the compiler sinks
@@ -310,7 +334,11 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
   wait_vmcnt<P * LPI>();
   __syncthreads();
   floatx16 sa0, sa1, sb0, sb1;
-  compute_s(0, sa0, sa1);
+  {
+    half8 kfr[2 * KS];
+    load_k(0, kfr);
+    mfma_s(kfr, sa0, sa1);
+  }
   DEERS_TRACE_POINT(1);
 
   constexpr std::true_type yes{};
@@ -334,8 +362,11 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
   // ---- drain: O += V(n-1) P(n-1) ----
   wait_vmcnt<(P - 1) * LPI>();  // V(n-1) precedes the last P-1 (never consumed) groups
   __syncthreads();
-  compute_pv_half(n_tiles - 1, 0);
-  compute_pv_half(n_tiles - 1, 1);
+  {
+    half8 vfr[4 * DB];
+    load_v(n_tiles - 1, vfr);
+    mfma_pv(vfr);
+  }
 
   // ---- epilogue: O = acc / l, LSE = ln(l) + m*scale ----
   lsum = pair_sum(lsum);

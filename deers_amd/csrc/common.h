@@ -63,6 +63,22 @@ __device__ __forceinline__ half4 lds_read_tr16(const half_t* p) {
   return __builtin_bit_cast(half4, r);
 }
 
+// Hides a value's provenance from the optimiser.  Used on per-iteration LDS base
+// addresses: without it the compiler re-associates (slot base + lane offset + row
+// constant) into one add per read instead of one add per iteration plus an
+// instruction immediate.
+__device__ __forceinline__ uint32_t opaque(uint32_t x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
+// Same read from a 32-bit LDS byte address.
+__device__ __forceinline__ half4 lds_read_tr16_at(uint32_t lds_addr) {
+  fp16x4_raw r =
+      __builtin_amdgcn_ds_read_tr16_b64_v4f16((DEERS_LDS fp16x4_raw*)(uintptr_t)lds_addr);
+  return __builtin_bit_cast(half4, r);
+}
+
 // A-operand fragment (8 halfs) for the lane's fixed column `col_base + l%32` of a
 // row-major LDS tile, contraction rows {4g..4g+3} + row_base and {8+4g..} + row_base:
 // the transposed operand that pairs with accumulator regs 8s..8s+7 used as B.
@@ -187,6 +203,49 @@ struct DecodeParams {
   int H, L, splits, chunk;
   float scale_log2;
 };
+
+#ifndef DEERS_SNAKE
+#define DEERS_SNAKE 0
+#endif
+#ifndef DEERS_PRIO
+#define DEERS_PRIO 1
+#endif
+
+// Maps blockIdx.x to (head, block rank).  Workgroups are dealt round-robin to the 8
+// XCDs, so blockIdx.x % 8 is the XCD: every block of one head is given to one XCD
+// (its operands stay in that XCD's L2) and each XCD's list is ordered longest
+// first (rank 0 = the block with the most iterations), which is what the
+// dispatcher's in-order hand-out to free slots needs for an even finish.
+// Returns false for padding ids.
+__device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int BH, int* bh,
+                                          int* rank) {
+  const int xcd = blockIdx.x & 7;
+  int idx = blockIdx.x >> 3;
+#if DEERS_SNAKE
+  // variant for launches where every workgroup is resident at once: a CU then holds
+  // items i, i+32, i+64 of the list, and reversing every second group of 32 evens
+  // out the per-CU sums
+  const int per_xcd = n_blocks * heads_per_xcd;
+  const int grp = idx >> 5, pos = idx & 31;
+  const int grp_len = min(32, per_xcd - 32 * grp);
+  if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
+#endif
+  *bh = (idx % heads_per_xcd) * 8 + xcd;
+  *rank = idx / heads_per_xcd;
+  return *bh < BH;
+}
+
+// Long blocks are the critical path of a causal launch: waves of the longest
+// blocks ask the instruction arbiter for priority over the short blocks that share
+// their SIMD, which then fill the gaps.
+__device__ __forceinline__ void set_block_priority(int rank, int n_blocks) {
+#if DEERS_PRIO
+  const int q = (4 * rank) / max(n_blocks, 1);  // 0 = longest quarter
+  if (q == 0) __builtin_amdgcn_s_setprio(3);
+  else if (q == 1) __builtin_amdgcn_s_setprio(2);
+  else if (q == 2) __builtin_amdgcn_s_setprio(1);
+#endif
+}
 
 // Brackets one kernel launch with a hipEvent pair when per-kernel profiling is
 // switched on (deers_rocm_profile_enable); a no-op otherwise.  Defined in

@@ -15,7 +15,7 @@ import numpy as np
 
 F16, F32 = 0, 1
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdeers_rocm.so")
+LIB_PATH = os.environ.get("DEERS_ROCM_LIB") or os.path.join(_HERE, "libdeers_rocm.so")
 
 _lib = None
 _inited = False
