@@ -143,15 +143,18 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
   for (int i = 0; i < P; ++i) request(first_tile + i);
 
   // K^T and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.
+  // Rows past T-1 read row T-1 instead: their keys are masked for every valid query
+  // and their dK/dV rows are not stored, and without a branch the loads issue as one
+  // batch with a single wait.
   half8 kf[KS], vf[KS];
+  {
+    const int krow = min(kvrow, T - 1);
+    const half_t* kp = K + (int64_t)krow * p.sk.t + 8 * g;
+    const half_t* vp = V + (int64_t)krow * p.sv.t + 8 * g;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (kvrow < T) {
-      kf[ks] = *(const half8*)(K + (int64_t)kvrow * p.sk.t + 16 * ks + 8 * g);
-      vf[ks] = *(const half8*)(V + (int64_t)kvrow * p.sv.t + 16 * ks + 8 * g);
-    } else {
-      kf[ks] = ZEROH8;
-      vf[ks] = ZEROH8;
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks] = *(const half8*)(kp + 16 * ks);
+      vf[ks] = *(const half8*)(vp + 16 * ks);
     }
   }
 
@@ -239,6 +242,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
 
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
+  wait_all_vmem();  // K/V fragments are in registers; see wait_all_vmem
   for (int j = first_tile; j < n_tiles; ++j) {
     // tile j was requested P iterations ago; at most the P-1 younger groups may
     // still be in flight.  The barrier also retires all reads of the slot that the
@@ -356,24 +360,35 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
 
   half8 qf[KS], dof[KS];
   float dsum = 0.f;  // this lane's half of rowsum(dO o O)
+  float lse_clamped;
   const half_t* O = (const half_t*)p.o + b * p.so.b + h * p.so.h;
+  // Rows past T-1 read row T-1 instead (their dQ rows are not stored and a query owns
+  // its accumulator column, so nothing leaks into valid rows): without a branch all
+  // loads issue as one batch with a single wait.
+  {
+    const int lrow = min(qrow, T - 1);
+    const half_t* qp = Q + (int64_t)lrow * p.sq.t + 8 * g;
+    const half_t* dop = dO + (int64_t)lrow * p.sdo.t + 8 * g;
+    const half_t* op = O + (int64_t)lrow * p.so.t + 8 * g;
+    half8 of[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (qrow < T) {
-      qf[ks] = *(const half8*)(Q + (int64_t)qrow * p.sq.t + 16 * ks + 8 * g);
-      dof[ks] = *(const half8*)(dO + (int64_t)qrow * p.sdo.t + 16 * ks + 8 * g);
-      const half8 of = *(const half8*)(O + (int64_t)qrow * p.so.t + 16 * ks + 8 * g);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) dsum += (float)dof[ks][e] * (float)of[e];
-    } else {
-      qf[ks] = ZEROH8;
-      dof[ks] = ZEROH8;
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = *(const half8*)(qp + 16 * ks);
+      dof[ks] = *(const half8*)(dop + 16 * ks);
+      of[ks] = *(const half8*)(op + 16 * ks);
     }
+    const float lse_row = p.lse[(int64_t)bh * T + lrow];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dsum += (float)dof[ks][e] * (float)of[ks][e];
+    if (qrow >= T) dsum = 0.f;
+    lse_clamped = lse_row;
   }
   // Per-row statistics, also published for the dK/dV kernel that runs next: rows in
   // the padding [T, t_pad) get lse2 = +inf and negdelta = 0, i.e. probability 0.
   const float nd = -pair_sum(dsum);
-  const float l2 = qrow < T ? p.lse[(int64_t)bh * T + qrow] * kLog2e : INFINITY;
+  const float l2 = qrow < T ? lse_clamped * kLog2e : INFINITY;
   if (g == 0 && qrow < p.t_pad) {
     p.lse2[(int64_t)bh * p.t_pad + qrow] = l2;
     p.negdelta[(int64_t)bh * p.t_pad + qrow] = nd;
@@ -439,6 +454,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
 
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
+  wait_all_vmem();  // Q/dO fragments are in registers; see wait_all_vmem
   for (int j = 0; j < n_tiles; ++j) {
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();

@@ -78,23 +78,9 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
   const int g = lane >> 5;
   const int T = p.T;
 
-  // Workgroups are dealt round-robin to the 8 XCDs.  Keep every tile of one head
-  // on one XCD (its K/V stay in that XCD's L2) and give each XCD the same mix of
-  // long and short rows, longest first.
-  // Within an XCD the dispatcher deals workgroups to its 32 CUs in order, so a CU
-  // receives items i, i+32, i+64, ... of the XCD's list: the list is sorted longest
-  // first and every second group of 32 is reversed, which evens out the per-CU sums.
-  const int xcd = blockIdx.x & 7;
-  int idx = blockIdx.x >> 3;
-  const int per_xcd = n_qtiles * heads_per_xcd;
-  {
-    const int grp = idx >> 5, pos = idx & 31;
-    const int grp_len = min(32, per_xcd - 32 * grp);
-    if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
-  }
-  const int bh = (idx % heads_per_xcd) * 8 + xcd;
-  if (bh >= BH) return;
-  const int qtile = n_qtiles - 1 - idx / heads_per_xcd;
+  int bh, rank;
+  if (!map_block(n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
+  const int qtile = n_qtiles - 1 - rank;  // longest rows first
   const int b = bh / p.H, h = bh % p.H;
 
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
@@ -151,12 +137,12 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
 
   // Q fragments: B operand of S^T = K Q^T, lane holds Q[qrow][16ks + 8g .. +7].
   half8 qf[KS];
+  // Rows past T-1 read row T-1 instead (they are not stored, and a query owns its
+  // accumulator column), so the loads issue as one batch without a branch.
+  {
+    const half_t* qp = Q + (int64_t)min(qrow, T - 1) * p.sq.t + 8 * g;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (qrow < T)
-      qf[ks] = *(const half8*)(Q + (int64_t)qrow * p.sq.t + 16 * ks + 8 * g);
-    else
-      qf[ks] = ZEROH8;
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const half8*)(qp + 16 * ks);
   }
 
   // ---- per-lane swizzled read offsets (bytes within a tile) ----
@@ -285,38 +271,63 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
       }
     }
     const float mc = m * c;
-    // ---- one straight-line block: 16 MFMAs beside the exponentials ----
-    if constexpr (HAS_PV) mfma_pv(vfr);
-    if constexpr (HAS_S) mfma_s(kfr, n0, n1);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      c0[r] = fast_exp2(__builtin_fmaf(c0[r], c, -mc));
-      c1[r] = fast_exp2(__builtin_fmaf(c1[r], c, -mc));
+    // ---- one straight-line block of 16 fenced chunks ----
+    // Chunk i issues its share of the MFMAs (S(j+1) first: the next iteration's row
+    // maxima wait on it; then PV(j-1)), the exponentials of two scores, and the f16
+    // packing of the previous chunk's pair, so that no instruction waits on the one
+    // just before it.  The fences keep the compiler from regrouping the chunks: left
+    // alone it issues the MFMAs back to back and the vector work after them.
+    // Row sums use v_dot2_f32_f16 against (1,1): one vector issue slot per pair.  It
+    // executes on the matrix pipe, which has slack here (the vector issue port is the
+    // busier one), so it is cheaper than two f32 adds.
+    constexpr int NMS = HAS_S ? 2 * KS : 0;
+    constexpr int NM = NMS + (HAS_PV ? 4 * DB : 0);
+    if constexpr (HAS_S) {
+      n0 = ZERO16;
+      n1 = ZERO16;
     }
+    uint32_t pw[16];  // P(j) as packed f16 pairs; words 4k..4k+3 form B operand k
+    auto row_sum = [&](int i) {  // from the f16-rounded pair, i.e. exactly what PV multiplies
+      lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
+      asm volatile("" : "+v"(lsum));
+    };
+    auto pack_pair = [&](int i) {  // scores 2(i%8), 2(i%8)+1 of block i/8
+      const floatx16& cc = (i < 8) ? c0 : c1;
+      const int r = 2 * (i & 7);
+      pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)cc[r], (half_t)cc[r + 1]});
+      asm volatile("" : "+v"(pw[i]));  // keep the conversion in its chunk
+    };
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+#pragma unroll
+      for (int mi = i * NM / 16; mi < (i + 1) * NM / 16; ++mi) {
+        if (mi < NMS) {
+          const int ks = mi >> 1;
+          if (mi & 1)
+            n1 = mfma_f16(kfr[2 * ks + 1], qf[ks], n1);
+          else
+            n0 = mfma_f16(kfr[2 * ks], qf[ks], n0);
+        } else {
+          const int ms = (mi - NMS) / DB, db = (mi - NMS) % DB;
+          oacc[db] = mfma_f16(vfr[ms * DB + db], pf[ms], oacc[db]);
+        }
+      }
+      floatx16& cc = (i < 8) ? c0 : c1;
+      const int r = 2 * (i & 7);
+      cc[r] = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
+      cc[r + 1] = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
+      if (i > 0) pack_pair(i - 1);
+      if (i > 1) row_sum(i - 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    pack_pair(15);
+    row_sum(14);
+    row_sum(15);
     half8 pn[4];
 #pragma unroll
-    for (int st = 0; st < 2; ++st) {
-      pn[st] = pack_half8(c0[8 * st + 0], c0[8 * st + 1], c0[8 * st + 2], c0[8 * st + 3],
-                          c0[8 * st + 4], c0[8 * st + 5], c0[8 * st + 6], c0[8 * st + 7]);
-      pn[2 + st] = pack_half8(c1[8 * st + 0], c1[8 * st + 1], c1[8 * st + 2], c1[8 * st + 3],
-                              c1[8 * st + 4], c1[8 * st + 5], c1[8 * st + 6], c1[8 * st + 7]);
-    }
-    // row sums from the f16-rounded probabilities, i.e. exactly what PV multiplies
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int e = 0; e < 8; e += 2)
-        lsum = add_half2(half2v{pn[i][e], pn[i][e + 1]}, lsum);
-    // Ask the scheduler for the interleaving: per MFMA, two exponentials and a few
-    // plain vector ops.
-    if constexpr (HAS_PV || HAS_S) {
-      constexpr int NM = (HAS_PV ? 8 : 0) + (HAS_S ? 8 : 0);
-#pragma unroll
-      for (int i = 0; i < NM; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x400, (NM == 16) ? 2 : 4, 0);  // exp
-        __builtin_amdgcn_sched_group_barrier(0x002, (NM == 16) ? 5 : 10, 0);  // VALU
-      }
+    for (int k = 0; k < 4; ++k) {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      pn[k] = __builtin_bit_cast(half8, u32x4{pw[4 * k], pw[4 * k + 1], pw[4 * k + 2], pw[4 * k + 3]});
     }
     // Pin P(j) and the row sum here: without a use in this block the compiler sinks
     // the exponentials past the barrier into the next iteration, away from the MFMAs

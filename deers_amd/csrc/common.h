@@ -122,6 +122,15 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
+// Waits for every outstanding vector-memory operation with an instruction the
+// compiler can see.  The compiler's own wait insertion knows nothing of the
+// asynchronous copies above; if a register filled by an ordinary global load might
+// still be pending when a loop is entered, it puts "s_waitcnt vmcnt(0)" at the
+// first use inside the loop, which also waits for the copies prefetched for later
+// iterations.  Call this once after the prologue's ordinary loads.
+__device__ __forceinline__ void wait_all_vmem() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt untouched
+}
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(size_t)(DEERS_LDS const void*)p;
 }
@@ -230,8 +239,16 @@ __device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int B
   const int grp_len = min(32, per_xcd - 32 * grp);
   if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
 #endif
+  // The division runs on the vector unit; without the readfirstlane every value
+  // derived from the head or rank (base pointers, trip counts, tile addresses) would
+  // be kept in vector registers and computed with vector instructions.
+#ifdef DEERS_UNIFORM_IDS
+  *bh = __builtin_amdgcn_readfirstlane((idx % heads_per_xcd) * 8 + xcd);
+  *rank = __builtin_amdgcn_readfirstlane(idx / heads_per_xcd);
+#else
   *bh = (idx % heads_per_xcd) * 8 + xcd;
   *rank = idx / heads_per_xcd;
+#endif
   return *bh < BH;
 }
 
