@@ -242,7 +242,10 @@ __device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int B
   // The division runs on the vector unit; without the readfirstlane every value
   // derived from the head or rank (base pointers, trip counts, tile addresses) would
   // be kept in vector registers and computed with vector instructions.
-#ifdef DEERS_UNIFORM_IDS
+#if DEERS_UNIFORM_IDS == 1
+  *bh = __builtin_amdgcn_readfirstlane((idx % heads_per_xcd) * 8 + xcd);
+  *rank = idx / heads_per_xcd;
+#elif DEERS_UNIFORM_IDS == 2
   *bh = __builtin_amdgcn_readfirstlane((idx % heads_per_xcd) * 8 + xcd);
   *rank = __builtin_amdgcn_readfirstlane(idx / heads_per_xcd);
 #else
