@@ -24,6 +24,12 @@ void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream);
 int decode_pick_splits(int64_t BH, int64_t L, int* chunk);
+void launch_fill(int dtype_f16, void* dst, size_t n, float value, hipStream_t stream);
+void launch_add(int dtype_f16, const void* a, const void* b, void* out, size_t n,
+                hipStream_t stream);
+void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t stream);
+void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
+                         const int64_t* strides, int ndim, void* dst, hipStream_t stream);
 }  // namespace deers
 
 namespace {
@@ -484,6 +490,62 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
   p.H = (int)H; p.L = (int)L; p.splits = splits; p.chunk = chunk;
   p.scale_log2 = (float)((double)scale * 1.4426950408889634);
   deers::launch_attn_decode_f16(p, (int)B, (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- element-wise helpers of the storage backend ----
+
+static int check_dtype(int dtype) {
+  if (dtype != DEERS_ROCM_F16 && dtype != DEERS_ROCM_F32)
+    return fail(DEERS_ROCM_ERR_ARG, "unknown dtype %d", dtype);
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_fill(int dtype, void* dst, size_t n, float value) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!dst) return fail(DEERS_ROCM_ERR_ARG, "fill: null pointer");
+  deers::launch_fill(dtype == DEERS_ROCM_F16, dst, n, value, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_add(int dtype, const void* a, const void* b, void* out, size_t n) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!a || !b || !out) return fail(DEERS_ROCM_ERR_ARG, "add: null pointer");
+  deers::launch_add(dtype == DEERS_ROCM_F16, a, b, out, n, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_neg(int dtype, const void* a, void* out, size_t n) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!a || !out) return fail(DEERS_ROCM_ERR_ARG, "neg: null pointer");
+  deers::launch_neg(dtype == DEERS_ROCM_F16, a, out, n, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
+                            const int64_t* strides, int ndim, void* dst) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (ndim < 1 || ndim > 6) return fail(DEERS_ROCM_ERR_ARG, "copy_compact: ndim %d not in 1..6", ndim);
+  if (!src || !dst || !shape || !strides) return fail(DEERS_ROCM_ERR_ARG, "copy_compact: null pointer");
+  for (int d = 0; d < ndim; ++d)
+    if (shape[d] < 0 || strides[d] < 0)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "copy_compact: negative extent or stride in dim %d", d);
+  deers::launch_copy_strided(dtype == DEERS_ROCM_F16, src, shape, strides, ndim, dst, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -1,0 +1,250 @@
+// Test driver of the C++ host side.
+//   host_test graph            graph / layout logic on unbacked tensors (no GPU)
+//   host_test gpu <dir>        runs the fused op on the inputs in <dir> (written by
+//                              the Python tests) and writes its outputs there
+// The graph cases restate the reference's own autograd tests
+// (src/backprop.rs:142-201): linear chain, diamond, no-grad skip, accumulation = 2.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <string>
+#include <vector>
+
+#include "../../include/deers_rocm.h"
+#include "ops.h"
+
+using namespace deers_host;
+
+static int g_failed = 0;
+#define EXPECT(cond)                                                        \
+  do {                                                                      \
+    if (!(cond)) {                                                          \
+      std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);           \
+      ++g_failed;                                                           \
+    }                                                                       \
+  } while (0)
+
+static void test_layout() {
+  Layout l({2, 3, 4, 5});
+  EXPECT(l.is_compact());
+  EXPECT((l.strides == std::vector<int64_t>{60, 20, 5, 1}));
+  Layout p = l.permute({0, 2, 1, 3});
+  EXPECT((p.shape == std::vector<int64_t>{2, 4, 3, 5}));
+  EXPECT((p.strides == std::vector<int64_t>{60, 5, 20, 1}));
+  EXPECT(!p.is_compact());
+  EXPECT(p.permute({0, 2, 1, 3}).is_compact());
+  EXPECT(l.transpose(2, 3).strides.back() == 5);
+  EXPECT(l.size() == 120);
+  bool threw = false;
+  try { (void)l.permute({0, 1}); } catch (const std::logic_error&) { threw = true; }
+  EXPECT(threw);
+  std::printf("ok layout\n");
+}
+
+static void test_sorted_nodes_linear_chain() {
+  Tensor a = Tensor::unbacked({2, 3}, DType::F32).attach();
+  Tensor b = a.neg(), c = b.neg(), d = c.neg();
+  auto sorted = d.sorted_nodes();
+  EXPECT(sorted.size() == 4);
+  if (sorted.size() == 4) {
+    EXPECT(*sorted[0] == d);
+    EXPECT(*sorted[1] == c);
+    EXPECT(*sorted[2] == b);
+    EXPECT(*sorted[3] == a);
+  }
+  std::printf("ok sorted_nodes_linear_chain\n");
+}
+
+static void test_sorted_nodes_diamond() {
+  Tensor a = Tensor::unbacked({2}, DType::F32).attach();
+  Tensor b = a.neg(), c = a.neg();
+  Tensor d = b.add(c);
+  auto sorted = d.sorted_nodes();
+  EXPECT(sorted.size() == 4);  // no duplicates
+  if (sorted.size() == 4) {
+    EXPECT(*sorted.front() == d);
+    EXPECT(*sorted.back() == a);  // shared input last
+  }
+  std::printf("ok sorted_nodes_diamond\n");
+}
+
+static void test_sorted_nodes_skips_no_grad() {
+  Tensor a = Tensor::unbacked({2}, DType::F32).attach();
+  Tensor b = Tensor::unbacked({2}, DType::F32);  // no grad
+  Tensor c = a.add(b);
+  auto sorted = c.sorted_nodes();
+  EXPECT(sorted.size() == 2);
+  if (sorted.size() == 2) {
+    EXPECT(*sorted[0] == c);
+    EXPECT(*sorted[1] == a);
+  }
+  // nothing requires grad: the op is dropped and the sweep is empty
+  Tensor e = b.neg();
+  EXPECT(!e.requires_grad());
+  EXPECT(e.op() == nullptr);
+  EXPECT(e.sorted_nodes().empty());
+  // NO_GRAD drops tracking even for attached inputs
+  {
+    NoGradGuard g;
+    Tensor f = a.neg();
+    EXPECT(!f.requires_grad());
+    EXPECT(f.op() == nullptr);
+  }
+  EXPECT(a.neg().requires_grad());
+  std::printf("ok sorted_nodes_skips_no_grad\n");
+}
+
+static void test_graph_of_attention_views() {
+  // the shape of the sub-graph at src/models/gpt.rs:135-144: projections [B,T,H,D],
+  // permuted to [B,H,T,D]; backward through Permute returns the gradient to the
+  // [B,T,H,D] leaf as the inverse-permuted view
+  Tensor x = Tensor::unbacked({2, 5, 3, 8}, DType::F16).attach();
+  Tensor v = x.permute({0, 2, 1, 3});
+  EXPECT((v.shape() == std::vector<int64_t>{2, 3, 5, 8}));
+  EXPECT((v.layout().strides == std::vector<int64_t>{120, 8, 24, 1}));
+  EXPECT(v.requires_grad());
+  EXPECT(std::string(v.op()->name()) == "Permute");
+  GradientStore grads = v.backward();
+  const Tensor* gx = grads.get(x.id());
+  EXPECT(gx != nullptr);
+  if (gx) EXPECT(gx->shape() == x.shape());
+  std::printf("ok graph_of_attention_views\n");
+}
+
+// ---- GPU cases ----
+
+static std::vector<char> read_file(const std::string& path) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) { std::printf("FAIL cannot read %s\n", path.c_str()); std::exit(2); }
+  return std::vector<char>((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+}
+static void write_file(const std::string& path, const void* p, size_t n) {
+  std::ofstream f(path, std::ios::binary);
+  f.write(static_cast<const char*>(p), (std::streamsize)n);
+}
+static void dump(const Tensor& t, const std::string& path) {
+  std::vector<char> host(t.layout().size() * size_in_bytes(t.dtype()));
+  t.to_host(host.data());
+  write_file(path, host.data(), host.size());
+}
+
+static void test_backward_accumulates_diamond_grads() {
+  Tensor a = Tensor::ones({2}, DType::F32).attach();
+  Tensor b = a.add(a);
+  GradientStore grads = b.backward();  // seeded with ones, like sum().backward()
+  const Tensor* ga = grads.get(a.id());
+  EXPECT(ga != nullptr);
+  if (ga) {
+    float h[2] = {0, 0};
+    ga->to_host(h);
+    EXPECT(h[0] == 2.0f && h[1] == 2.0f);  // a is used twice
+  }
+  std::printf("ok backward_accumulates_diamond_grads\n");
+}
+
+static int run_gpu(const std::string& dir) {
+  check(deers_rocm_init(0));
+  test_backward_accumulates_diamond_grads();
+
+  // case.txt: dtype B H T D L   (dtype 0 = f16, 1 = f32; L = decode cache length or 0)
+  int dt, B, H, T, D, L;
+  {
+    std::ifstream f(dir + "/case.txt");
+    if (!(f >> dt >> B >> H >> T >> D >> L)) { std::printf("FAIL bad case.txt\n"); return 2; }
+  }
+  const DType dtype = dt == 0 ? DType::F16 : DType::F32;
+  const std::vector<int64_t> bthd{B, T, H, D};
+  auto load = [&](const char* name, const std::vector<int64_t>& shape) {
+    auto bytes = read_file(dir + "/" + name);
+    Layout l(shape);
+    if (bytes.size() != l.size() * size_in_bytes(dtype)) { std::printf("FAIL size of %s\n", name); std::exit(2); }
+    return Tensor::from_host(bytes.data(), shape, dtype);
+  };
+  // Projections arrive as [B,T,H,D] and are permuted to [B,H,T,D] (gpt.rs:135-137).
+  Tensor xq = load("q.bin", bthd).attach(), xk = load("k.bin", bthd).attach(), xv = load("v.bin", bthd).attach();
+  Tensor seed = load("do.bin", bthd);  // d loss / d y in the [B,T,H,D] order y is reshaped from
+  Tensor q = xq.permute({0, 2, 1, 3}), k = xk.permute({0, 2, 1, 3}), v = xv.permute({0, 2, 1, 3});
+  Tensor y = causal_self_attention(q, k, v);           // compact [B,H,T,D]
+  EXPECT(y.is_compact());
+  EXPECT(std::string(y.op()->name()) == "FusedCausalAttention");
+  Tensor y_bthd = y.permute({0, 2, 1, 3}).compact();   // what reshape does (ops.rs:913)
+  dump(y_bthd, dir + "/y.bin");
+  GradientStore grads = y_bthd.backward_from(seed);
+  for (auto [t, name] : {std::pair<const Tensor*, const char*>{&xq, "dq.bin"}, {&xk, "dk.bin"}, {&xv, "dv.bin"}}) {
+    const Tensor* g = grads.get(t->id());
+    EXPECT(g != nullptr);
+    if (g) {
+      EXPECT(g->shape() == t->shape());
+      dump(*g, dir + "/" + name);
+    }
+  }
+  // the same inputs through two attention ops: every gradient doubles exactly
+  {
+    Tensor y2 = causal_self_attention(q, k, v).add(causal_self_attention(q, k, v));
+    GradientStore g2 = y2.permute({0, 2, 1, 3}).compact().backward_from(seed);
+    const Tensor* a = grads.get(xv.id());
+    const Tensor* b2 = g2.get(xv.id());
+    EXPECT(a && b2);
+    if (a && b2) {
+      const size_t n = a->layout().size();
+      if (dtype == DType::F32) {
+        std::vector<float> ha(n), hb(n);
+        a->to_host(ha.data());
+        b2->to_host(hb.data());
+        size_t bad = 0;
+        for (size_t i = 0; i < n; ++i) bad += (hb[i] != 2.0f * ha[i]);
+        EXPECT(bad == 0);
+      } else {
+        dump(*b2, dir + "/dv_twice.bin");
+      }
+    }
+  }
+  // no-grad inputs: the op is dropped, nothing to sweep
+  {
+    Tensor yn = causal_self_attention(q.detach(), k.detach(), v.detach());
+    EXPECT(!yn.requires_grad() && yn.op() == nullptr);
+  }
+  if (L > 0) {
+    Tensor dq = load("dec_q.bin", {B, H, D});
+    Tensor kc = load("dec_k.bin", {B, H, L, D}), vc = load("dec_v.bin", {B, H, L, D});
+    dump(attention_decode(dq, kc, vc), dir + "/dec_o.bin");
+  }
+  // backend failures surface as RocmError carrying the library's message
+  {
+    bool threw = false;
+    try {
+      Tensor bad = Tensor::zeros({1, 1, 8, 48}, dtype);  // head_dim 48 is not supported
+      (void)causal_self_attention(bad, bad, bad);
+    } catch (const RocmError& e) {
+      threw = std::strlen(e.what()) > 0;
+    }
+    EXPECT(threw);
+  }
+  check(deers_rocm_sync());
+  std::printf("ok gpu\n");
+  return 0;
+}
+
+int main(int argc, char** argv) {
+  const std::string mode = argc > 1 ? argv[1] : "graph";
+  try {
+    if (mode == "graph") {
+      test_layout();
+      test_sorted_nodes_linear_chain();
+      test_sorted_nodes_diamond();
+      test_sorted_nodes_skips_no_grad();
+      test_graph_of_attention_views();
+    } else if (mode == "gpu" && argc > 2) {
+      if (int rc = run_gpu(argv[2])) return rc;
+    } else {
+      std::printf("usage: host_test graph | gpu <dir>\n");
+      return 2;
+    }
+  } catch (const std::exception& e) {
+    std::printf("FAIL exception: %s\n", e.what());
+    return 1;
+  }
+  std::printf(g_failed ? "FAILED %d checks\n" : "all passed\n", g_failed);
+  return g_failed ? 1 : 0;
+}

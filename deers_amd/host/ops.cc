@@ -1,0 +1,164 @@
+// Operators of the C++ host side; see ops.h for the reference ops each follows.
+#include "ops.h"
+
+#include <cmath>
+
+#include "../../include/deers_rocm.h"
+
+namespace deers_host {
+
+namespace {
+
+bool backed(const Tensor& t) { return t.storage()->ptr() != nullptr; }
+
+// Fresh compact storage shaped like `shape`.
+Tensor empty(const std::vector<int64_t>& shape, DType dtype, bool is_backed) {
+  Layout l(shape);
+  auto st = std::make_shared<RocmStorage>(l.size(), dtype, is_backed);
+  return Tensor(std::move(st), std::move(l), false, nullptr);
+}
+
+// A [B,H,T,D] view the kernels take as is: unit D stride (alignment is the
+// library's check).  Anything else is compacted.
+Tensor kernel_ready(const Tensor& t) {
+  const Layout& l = t.layout();
+  const int64_t per16 = 16 / (int64_t)size_in_bytes(t.dtype());
+  bool ok = l.strides.back() == 1 && l.offset % per16 == 0;
+  for (size_t d = 0; d + 1 < l.ndim(); ++d) ok = ok && l.strides[d] >= 0 && l.strides[d] % per16 == 0;
+  return ok ? t : t.compact();
+}
+
+}  // namespace
+
+// ---- Neg ----
+Tensor Neg::forward(std::unique_ptr<Neg> self) {
+  const Tensor a = self->arg_.compact();
+  Tensor out = empty(a.shape(), a.dtype(), backed(a));
+  if (backed(a)) check(deers_rocm_neg((int)a.dtype(), a.data(), out.data(), a.layout().size()));
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void Neg::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(arg_, out_grad.neg());
+}
+
+// ---- EWiseAdd ----
+EWiseAdd::EWiseAdd(Tensor a, Tensor b) : a_(std::move(a)), b_(std::move(b)) {
+  if (a_.shape() != b_.shape()) throw std::logic_error("EWiseAdd: shapes differ");
+  if (a_.dtype() != b_.dtype()) throw std::logic_error("EWiseAdd: dtypes differ");
+}
+Tensor EWiseAdd::forward(std::unique_ptr<EWiseAdd> self) {
+  const Tensor a = self->a_.compact(), b = self->b_.compact();
+  Tensor out = empty(a.shape(), a.dtype(), backed(a));
+  if (backed(a))
+    check(deers_rocm_add((int)a.dtype(), a.data(), b.data(), out.data(), a.layout().size()));
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void EWiseAdd::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(a_, out_grad);
+  grads.accumulate(b_, out_grad);
+}
+
+// ---- Permute ----
+Permute::Permute(Tensor arg, std::vector<size_t> axes) : arg_(std::move(arg)), axes_(std::move(axes)) {
+  if (arg_.layout().ndim() != axes_.size())
+    throw std::logic_error("permute: tensor has " + std::to_string(arg_.layout().ndim()) +
+                           " dims but got " + std::to_string(axes_.size()) + " axes");
+}
+Tensor Permute::forward(std::unique_ptr<Permute> self) {
+  auto storage = self->arg_.storage();
+  Layout layout = self->arg_.layout().permute(self->axes_);
+  return Tensor(std::move(storage), std::move(layout), false, std::move(self));
+}
+void Permute::backward(GradientStore& grads, const Tensor& out_grad) const {
+  std::vector<size_t> inverse(axes_.size());
+  for (size_t new_axis = 0; new_axis < axes_.size(); ++new_axis) inverse[axes_[new_axis]] = new_axis;
+  grads.accumulate(arg_, out_grad.permute(inverse));
+}
+
+// ---- Compact ----
+Tensor Compact::forward(std::unique_ptr<Compact> self) {
+  const Tensor& a = self->arg_;
+  Tensor out = empty(a.shape(), a.dtype(), backed(a));
+  if (backed(a) && a.layout().size())
+    check(deers_rocm_copy_compact((int)a.dtype(), a.data(), a.layout().shape.data(),
+                                  a.layout().strides.data(), (int)a.layout().ndim(), out.data()));
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void Compact::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(arg_, out_grad);
+}
+
+// ---- Tensor conveniences that build ops ----
+Tensor Tensor::permute(const std::vector<size_t>& dims) const {
+  return Permute::forward(std::make_unique<Permute>(*this, dims));
+}
+Tensor Tensor::compact() const {
+  if (is_compact()) return *this;
+  return Compact::forward(std::make_unique<Compact>(*this));
+}
+Tensor Tensor::neg() const { return Neg::forward(std::make_unique<Neg>(*this)); }
+Tensor Tensor::add(const Tensor& other) const {
+  return EWiseAdd::forward(std::make_unique<EWiseAdd>(*this, other));
+}
+
+// ---- FusedCausalAttention ----
+FusedCausalAttention::FusedCausalAttention(Tensor q, Tensor k, Tensor v, double scale)
+    : q_(std::move(q)), k_(std::move(k)), v_(std::move(v)), scale_(scale) {
+  if (q_.layout().ndim() != 4) throw std::logic_error("FusedCausalAttention: q must be [B,H,T,D]");
+  if (q_.shape() != k_.shape() || q_.shape() != v_.shape())
+    throw std::logic_error("FusedCausalAttention: q, k, v shapes differ");
+  if (q_.dtype() != k_.dtype() || q_.dtype() != v_.dtype())
+    throw std::logic_error("FusedCausalAttention: dtypes differ");
+}
+
+Tensor FusedCausalAttention::forward(std::unique_ptr<FusedCausalAttention> self) {
+  const Tensor q = kernel_ready(self->q_), k = kernel_ready(self->k_), v = kernel_ready(self->v_);
+  const auto& s = q.shape();
+  const int64_t B = s[0], H = s[1], T = s[2], D = s[3];
+  Tensor o = empty(s, q.dtype(), true);
+  Tensor lse = empty({B, H, T}, DType::F32, true);
+  check(deers_rocm_attn_fwd((int)q.dtype(), q.data(), q.layout().strides.data(), k.data(),
+                            k.layout().strides.data(), v.data(), v.layout().strides.data(), o.data(),
+                            nullptr, (float*)lse.data(), B, H, T, D, (float)self->scale_));
+  self->saved_o_ = o;
+  self->saved_lse_ = lse;
+  return Tensor(o.storage(), o.layout(), false, std::move(self));
+}
+
+void FusedCausalAttention::backward(GradientStore& grads, const Tensor& out_grad) const {
+  if (!saved_o_.defined()) throw std::logic_error("forward must run before backward");
+  // out_grad usually arrives as the inverse-permuted view of the reshape gradient:
+  // logical [B,H,T,D] over [B,T,H,D] memory, which the kernels read directly.
+  const Tensor q = kernel_ready(q_), k = kernel_ready(k_), v = kernel_ready(v_);
+  const Tensor g = kernel_ready(out_grad);
+  const auto& s = q.shape();
+  const int64_t B = s[0], H = s[1], T = s[2], D = s[3];
+  Tensor dq = empty(s, q.dtype(), true), dk = empty(s, q.dtype(), true), dv = empty(s, q.dtype(), true);
+  check(deers_rocm_attn_bwd((int)q.dtype(), q.data(), q.layout().strides.data(), k.data(),
+                            k.layout().strides.data(), v.data(), v.layout().strides.data(),
+                            saved_o_.data(), nullptr, (const float*)saved_lse_.data(), g.data(),
+                            g.layout().strides.data(), dq.data(), nullptr, dk.data(), nullptr,
+                            dv.data(), nullptr, B, H, T, D, (float)scale_));
+  grads.accumulate(q_, dq);
+  grads.accumulate(k_, dk);
+  grads.accumulate(v_, dv);
+}
+
+Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v) {
+  const double scale = 1.0 / std::sqrt((double)q.shape().at(3));
+  return FusedCausalAttention::forward(std::make_unique<FusedCausalAttention>(q, k, v, scale));
+}
+
+Tensor attention_decode(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache) {
+  if (q.layout().ndim() != 3 || k_cache.layout().ndim() != 4 || k_cache.shape() != v_cache.shape())
+    throw std::logic_error("attention_decode: q [B,H,D], caches [B,H,L,D]");
+  const Tensor qc = q.compact(), kc = k_cache.compact(), vc = v_cache.compact();
+  const int64_t B = kc.shape()[0], H = kc.shape()[1], L = kc.shape()[2], D = kc.shape()[3];
+  Tensor o = empty({B, H, D}, q.dtype(), true);
+  const double scale = 1.0 / std::sqrt((double)D);
+  check(deers_rocm_attn_decode((int)q.dtype(), qc.data(), kc.data(), vc.data(), nullptr, o.data(), B, H,
+                               L, D, (float)scale));
+  return o;
+}
+
+}  // namespace deers_host

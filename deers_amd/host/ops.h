@@ -1,0 +1,91 @@
+// Operators of the C++ host side.  Neg, EWiseAdd, Permute and Compact follow the
+// reference ops of the same names (src/ops.rs:100-127, 130-173, 687-727,
+// 1254-1287); FusedCausalAttention is the new op that replaces the composed
+// attention core of src/models/gpt.rs:139-144 on the ROCm device, shaped after
+// FusedLogSoftmax (src/ops.rs:1186-1251).
+#ifndef DEERS_HOST_OPS_H
+#define DEERS_HOST_OPS_H
+
+#include "tensor.h"
+
+namespace deers_host {
+
+class Neg : public TensorOp {
+ public:
+  explicit Neg(Tensor arg) : arg_(std::move(arg)) {}
+  static Tensor forward(std::unique_ptr<Neg> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "Neg"; }
+
+ private:
+  Tensor arg_;
+};
+
+class EWiseAdd : public TensorOp {
+ public:
+  EWiseAdd(Tensor a, Tensor b);  // shapes must match (std::logic_error otherwise)
+  static Tensor forward(std::unique_ptr<EWiseAdd> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&a_, &b_}; }
+  const char* name() const override { return "EWiseAdd"; }
+
+ private:
+  Tensor a_, b_;
+};
+
+class Permute : public TensorOp {
+ public:
+  Permute(Tensor arg, std::vector<size_t> axes);
+  static Tensor forward(std::unique_ptr<Permute> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "Permute"; }
+
+ private:
+  Tensor arg_;
+  std::vector<size_t> axes_;
+};
+
+class Compact : public TensorOp {
+ public:
+  explicit Compact(Tensor arg) : arg_(std::move(arg)) {}
+  static Tensor forward(std::unique_ptr<Compact> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "Compact"; }
+
+ private:
+  Tensor arg_;
+};
+
+// y = softmax(q k^T * scale + causal mask) v for q, k, v logical [B,H,T,D] (views
+// welcome: any strides with a unit D stride go to the kernels as they are, other
+// views are compacted first, as FusedLogSoftmax::forward compacts its argument,
+// src/ops.rs:1205).  Returns a compact [B,H,T,D] tensor and keeps (O, LSE) for the
+// backward, which overwrites fresh dq/dk/dv buffers and hands them to
+// GradientStore::accumulate.
+class FusedCausalAttention : public TensorOp {
+ public:
+  FusedCausalAttention(Tensor q, Tensor k, Tensor v, double scale);
+  static Tensor forward(std::unique_ptr<FusedCausalAttention> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&q_, &k_, &v_}; }
+  const char* name() const override { return "FusedCausalAttention"; }
+
+ private:
+  Tensor q_, k_, v_;
+  double scale_;
+  Tensor saved_o_, saved_lse_;  // set by forward, created with no op
+};
+
+// The call site of src/models/gpt.rs:139-144: scale = 1/sqrt(head_dim) computed in
+// f64 and narrowed to f32 (src/storage.rs:115-117).
+Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
+
+// One query token per (b,h) against a KV cache: q [B,H,D], caches [B,H,L,D] compact;
+// not differentiable (inference only).
+Tensor attention_decode(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache);
+
+}  // namespace deers_host
+#endif

@@ -167,6 +167,31 @@ int deers_rocm_attn_decode(int dtype,
                            void* o,
                            int64_t B, int64_t H, int64_t L, int64_t D, float scale);
 
+/* ---- element-wise helpers of the storage backend ---------------------------
+ * The fused op's contract needs four more things from its backend: the seed of
+ * the reverse sweep, gradient accumulation, compaction of strided views, and (for
+ * the autograd contract tests) a unary op.  All work on `n` elements of `dtype`,
+ * are enqueued on the library stream and may alias (`out` == `a`). */
+
+/* dst[i] = value.  Replaces the backend half of Tensor::ones_like / zeros_like
+ * (src/backprop.rs:54, 96-98). */
+int deers_rocm_fill(int dtype, void* dst, size_t n, float value);
+
+/* out[i] = a[i] + b[i] on compact operands: what GradientStore::accumulate does
+ * through `&*existing + &grad` (src/backprop.rs:101-112; BinaryOp dispatch
+ * src/storage.rs:231-236).  f16 adds round once from the f32 sum. */
+int deers_rocm_add(int dtype, const void* a, const void* b, void* out, size_t n);
+
+/* out[i] = -a[i] (UnaryOp Neg, src/ops.rs:100-127). */
+int deers_rocm_neg(int dtype, const void* a, void* out, size_t n);
+
+/* dst (compact row-major over `shape`) <- src read through element `strides`;
+ * ndim in 1..6, strides non-negative (0 = broadcast).  Replaces
+ * BackendStorage::copy_compact (src/storage.rs:305; src/storage/cpu.rs:1063-1102),
+ * which the fused op calls on inputs whose innermost stride is not 1. */
+int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
+                            const int64_t* strides, int ndim, void* dst);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,76 @@
+"""The C++ host side (deers_amd/host): tensor / autograd slice and the fused attention op.
+
+The graph cases are the reference's own autograd tests (src/backprop.rs:142-201)
+restated in C++ and run on unbacked tensors, so they need no GPU.  The GPU case
+drives the op the way src/models/gpt.rs:135-147 does (projections [B,T,H,D],
+permuted views in, reshape copy out, reverse sweep through Permute / Compact /
+FusedCausalAttention) and is checked here against the CPU oracle.
+"""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from deers_amd import synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST_TEST = os.path.join(ROOT, "deers_amd", "host", "host_test")
+
+
+def _run(*args):
+    if not os.path.exists(HOST_TEST):
+        pytest.fail("deers_amd/host/host_test is not built (run __graft_entry__.build())")
+    return subprocess.run([HOST_TEST, *args], capture_output=True, text=True, timeout=300)
+
+
+def test_host_graph_contract():
+    r = _run("graph")
+    assert r.returncode == 0, r.stdout + r.stderr
+    for name in ("layout", "sorted_nodes_linear_chain", "sorted_nodes_diamond",
+                 "sorted_nodes_skips_no_grad", "graph_of_attention_views"):
+        assert f"ok {name}" in r.stdout
+    assert "all passed" in r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,B,H,T,D,L,tol", [
+    (np.float16, 2, 3, 200, 64, 300, 5e-3),
+    (np.float32, 1, 2, 130, 32, 0, 1e-4),
+])
+def test_host_fused_attention_matches_oracle(tmp_path, dtype, B, H, T, D, L, tol):
+    import oracle
+    x = synth.attention_inputs("host", B, H, T, D, dtype, base_seed=3)
+    bthd = lambda a: np.ascontiguousarray(a.transpose(0, 2, 1, 3))
+    for name in ("q", "k", "v", "do"):
+        bthd(x[name]).tofile(tmp_path / f"{name}.bin")
+    if L:
+        d = synth.attention_inputs("hostdec", B, H, 1, D, dtype, base_seed=4, kv_len=L,
+                                   names=("q", "k", "v"))
+        d["q"][:, :, 0].tofile(tmp_path / "dec_q.bin")
+        d["k"].tofile(tmp_path / "dec_k.bin")
+        d["v"].tofile(tmp_path / "dec_v.bin")
+    (tmp_path / "case.txt").write_text(f"{0 if dtype == np.float16 else 1} {B} {H} {T} {D} {L}\n")
+
+    r = _run("gpu", str(tmp_path))
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ok backward_accumulates_diamond_grads" in r.stdout and "all passed" in r.stdout
+
+    def out(name, shape=(B, T, H, D)):
+        return np.fromfile(tmp_path / name, dtype=dtype).reshape(shape).astype(np.float64)
+
+    f32 = {n: x[n].astype(np.float32) for n in ("q", "k", "v", "do")}
+    want_o = oracle.attn_fwd(f32["q"], f32["k"], f32["v"])
+    want = oracle.attn_bwd(f32["q"], f32["k"], f32["v"], f32["do"])
+    err = lambda got, ref: float(np.max(np.abs(got - bthd(ref))))
+    assert err(out("y.bin"), want_o) <= tol
+    for name, ref in zip(("dq.bin", "dk.bin", "dv.bin"), want):
+        assert err(out(name), ref) <= tol, name
+    if dtype == np.float16:
+        # two ops on the same inputs give the same bits, and x + x is exact in f16
+        assert np.array_equal(out("dv_twice.bin"), 2 * out("dv.bin"))
+    if L:
+        got = np.fromfile(tmp_path / "dec_o.bin", dtype=dtype).reshape(B, H, D).astype(np.float64)
+        ref = oracle.attn_fwd(d["q"].astype(np.float32), d["k"].astype(np.float32),
+                              d["v"].astype(np.float32))[:, :, 0]
+        assert float(np.max(np.abs(got - ref))) <= tol
