@@ -13,16 +13,23 @@
 //   Each lane group keeps a private online softmax (m, l, o[8] per lane) over
 //   the rows it visits; groups are merged once at the end through LDS in a
 //   fixed order, and the split partial (m, l, o[D]) goes to the workspace.
-//   A second tiny kernel merges the splits and writes f16 output.
+//   With one split per head (enough heads to give every CU a workgroup) the
+//   workgroup writes the f16 output itself; otherwise a second tiny kernel merges
+//   the splits in split order.
 #include "common.h"
 
 namespace deers {
 
-constexpr int kDecRowsPerIt = 4;
+#ifndef DEERS_DEC_ROWS
+#define DEERS_DEC_ROWS 4
+#endif
+constexpr int kDecRowsPerIt = DEERS_DEC_ROWS;  // cache rows in flight per lane group
 
+// Fewer, longer streams measure faster than many short ones (each workgroup pays a
+// start-up and a reduction): split a head only until every CU has a workgroup.
 int decode_pick_splits(int64_t BH, int64_t L, int* chunk) {
   int splits = 1;
-  while (BH * splits < 2048 && L / (splits * 2) >= 256) splits *= 2;
+  while (BH * splits < 256 && L / (splits * 2) >= 256) splits *= 2;
   int64_t c = (L + splits - 1) / splits;
   c = (c + 63) / 64 * 64;
   *chunk = (int)c;
@@ -66,8 +73,10 @@ __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
     for (int u = 0; u < kDecRowsPerIt; ++u) {
       const int row = r0 + u * GROUPS;
       if (row < row_end) {
-        kk[u] = *(const half8*)(K + (int64_t)row * p.skl);
-        vv[u] = *(const half8*)(V + (int64_t)row * p.skl);
+        // every cache byte is used once: non-temporal loads keep the stream from
+        // displacing itself in the caches and measurably raise the achieved HBM rate
+        kk[u] = __builtin_nontemporal_load((const half8*)(K + (int64_t)row * p.skl));
+        vv[u] = __builtin_nontemporal_load((const half8*)(V + (int64_t)row * p.skl));
       } else {
         kk[u] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         vv[u] = half8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -109,16 +118,21 @@ __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) red_o[grp * D + 8 * part + e] = o[e];
   __syncthreads();
+  float M = -INFINITY, lsum = 0.f, osum = 0.f;
   if (tid < D) {
-    float M = -INFINITY;
     for (int gi = 0; gi < GROUPS; ++gi) M = fmaxf(M, red_m[gi]);
-    float lsum = 0.f, osum = 0.f;
     for (int gi = 0; gi < GROUPS; ++gi) {
       const float mg = red_m[gi];
       const float w = (mg == -INFINITY) ? 0.f : fast_exp2(mg - M);
       lsum += w * red_l[gi];
       osum += w * red_o[gi * D + tid];
     }
+  }
+  if (p.splits == 1) {  // nothing to merge
+    if (tid < D) ((half_t*)p.o)[(int64_t)bh * D + tid] = (half_t)(osum / lsum);
+    return;
+  }
+  if (tid < D) {
     const int64_t slot = (int64_t)bh * p.splits + split;
     p.part_o[slot * D + tid] = osum;
     if (tid == 0) {
@@ -128,6 +142,9 @@ __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
   }
 }
 
+// Merges the split partials of a head in split order and writes the f16 output.
+// (A merge by the last split to arrive inside the main kernel was tried: the
+// device-scope fences it needs cost several times the whole stream.)
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_kernel(DecodeParams p) {
   const int bh = blockIdx.x;
@@ -147,20 +164,19 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(DecodeParams p) {
 
 void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream) {
   dim3 grid(p.splits, B * p.H);
-  if (D == 64) {
-    {
-      LaunchScope scope("attn_decode_f16", stream);
+  {
+    LaunchScope scope("attn_decode_f16", stream);
+    if (D == 64)
       hipLaunchKernelGGL(attn_decode_f16_kernel<64>, grid, dim3(256), 0, stream, p);
-    }
-    LaunchScope scope("attn_decode_merge", stream);
-    hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(B * p.H), dim3(64), 0, stream, p);
-  } else {
-    {
-      LaunchScope scope("attn_decode_f16", stream);
+    else
       hipLaunchKernelGGL(attn_decode_f16_kernel<128>, grid, dim3(256), 0, stream, p);
-    }
+  }
+  if (p.splits > 1) {
     LaunchScope scope("attn_decode_merge", stream);
-    hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(B * p.H), dim3(128), 0, stream, p);
+    if (D == 64)
+      hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(B * p.H), dim3(64), 0, stream, p);
+    else
+      hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(B * p.H), dim3(128), 0, stream, p);
   }
 }
 
