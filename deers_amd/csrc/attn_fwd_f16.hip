@@ -251,9 +251,14 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
         if (kv + 32 > qrow) c1[r] = -INFINITY;
       }
     }
-    float mx = fmaxf(c0[0], c1[0]);
+    // four independent max3 chains: a dependent vector op issues only every other
+    // slot, and with two waves per SIMD nothing else fills the gaps
+    float mx4[4];
 #pragma unroll
-    for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, c0[r]), c1[r]);
+    for (int i = 0; i < 4; ++i) mx4[i] = fmaxf(c0[i], c1[i]);
+#pragma unroll
+    for (int r = 4; r < 16; ++r) mx4[r & 3] = fmaxf(fmaxf(mx4[r & 3], c0[r]), c1[r]);
+    float mx = fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3]));
     mx = pair_max(mx);
     if (__any((mx - m) * c > kLazyRescale)) {
       // Rare after the first tiles: move O, l and the not yet multiplied P(j-1)
