@@ -129,6 +129,27 @@ def bench_decode(steps: int, warmup: int, rotate: int = 4):
                 gbs_call=nbytes / (total_us * 1e-6) / 1e9)
 
 
+def bench_copy(steps: int, warmup: int):
+    """Plain device copy of known size through the library's copy kernel: 256 MiB read
+    and 256 MiB written per launch.  It exists to calibrate hardware byte counters
+    (what FETCH_SIZE / WRITE_SIZE report for a kernel whose traffic is known)."""
+    n = 128 * 1024 * 1024  # f16 elements
+    src = rocm.DeviceBuffer((n,), np.float16, zeros=True)
+    dst = rocm.DeviceBuffer((n,), np.float16)
+    for _ in range(warmup):
+        rocm.copy_compact_raw(np.float16, src.ptr, (n,), (1,), dst.ptr)
+    rocm.sync()
+    timer = rocm.Timer()
+    timer.start()
+    for _ in range(steps):
+        rocm.copy_compact_raw(np.float16, src.ptr, (n,), (1,), dst.ptr)
+    timer.stop()
+    rocm.sync()
+    us = 1e3 * timer.elapsed_ms() / steps
+    return dict(bytes_read=2 * n, bytes_written=2 * n, kernel_us=us,
+                gbs=4.0 * n / (us * 1e-6) / 1e9)
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -160,7 +181,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -174,6 +195,8 @@ def main():
     if args.only != "all":
         if args.only == "decode":
             print(json.dumps({"only": "decode", **bench_decode(args.steps, args.warmup)}))
+        elif args.only == "copy":
+            print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
         else:
             tr = bench_train(args.steps, args.warmup, args.only)
             print(json.dumps({"only": args.only, "kernels": tr["kernels"]}))
@@ -197,9 +220,14 @@ def main():
             st["tflops"] = kernel_flops[n] / (st["avg_us"] * 1e-6) / 1e12
             st["frac_mfma_peak"] = st["tflops"] / PEAK_F16_TFLOPS
     achieved = kern[dom].get("tflops")
+    # HBM bytes per launch at this shape from the FETCH_SIZE / WRITE_SIZE passes of
+    # profiles/c2_c4_hbm_traffic_fetch_write.txt (scaled by what the same counters read
+    # for a copy of known size); a profiler measurement, not taken in this run.
+    measured_traffic = {"attn_bwd_dkdv_f16": 80.1e6, "attn_bwd_dq_f16": 83.5e6,
+                        "attn_fwd_f16": 53.2e6}
     roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": (achieved / PEAK_F16_TFLOPS) if achieved else None,
-                "traffic": None, "avg_launch_us": kern[dom]["avg_us"],
+                "traffic": measured_traffic.get(dom), "avg_launch_us": kern[dom]["avg_us"],
                 "flops_per_launch": kernel_flops.get(dom)}
 
     dec = bench_decode(args.steps, args.warmup)

@@ -185,6 +185,28 @@ def attn_decode_raw(dtype, q, k_cache, v_cache, o, B, H, L, D, scale, kv_strides
         ctypes.c_int64(H), ctypes.c_int64(L), ctypes.c_int64(D), ctypes.c_float(scale)))
 
 
+def fill_raw(dtype, dst, n, value):
+    _check(load().deers_rocm_fill(ctypes.c_int(dtype_code(dtype)), dst, ctypes.c_size_t(n),
+                                  ctypes.c_float(value)))
+
+
+def add_raw(dtype, a, b, out, n):
+    _check(load().deers_rocm_add(ctypes.c_int(dtype_code(dtype)), a, b, out, ctypes.c_size_t(n)))
+
+
+def neg_raw(dtype, a, out, n):
+    _check(load().deers_rocm_neg(ctypes.c_int(dtype_code(dtype)), a, out, ctypes.c_size_t(n)))
+
+
+def copy_compact_raw(dtype, src, shape, strides, dst):
+    """dst (compact over `shape`) <- src read through element `strides`."""
+    nd = len(shape)
+    sh = (ctypes.c_int64 * nd)(*[int(x) for x in shape])
+    st = (ctypes.c_int64 * nd)(*[int(x) for x in strides])
+    _check(load().deers_rocm_copy_compact(ctypes.c_int(dtype_code(dtype)), src, sh, st,
+                                          ctypes.c_int(nd), dst))
+
+
 def default_scale(D: int) -> float:
     """1/sqrt(D) in double, narrowed to f32 (src/models/gpt.rs:139, src/storage.rs:115-117)."""
     return float(np.float32(1.0 / np.sqrt(float(D))))

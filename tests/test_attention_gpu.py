@@ -219,3 +219,58 @@ def test_error_paths_report_messages():
         rocm.attn_fwd_raw(np.float16, None, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, T, D, 0.1)
     with pytest.raises(rocm.RocmError, match=">= 1"):
         rocm.attn_fwd_raw(np.float16, buf.ptr, buf.ptr, buf.ptr, buf.ptr, lse.ptr, B, H, 0, D, 0.1)
+
+
+# ---- element-wise helpers of the storage backend (fill, add, neg, copy_compact) ----
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_elementwise_helpers_match_numpy(dtype):
+    rng = np.random.default_rng(5)
+    n = 100003  # not a multiple of the block size
+    a = rng.standard_normal(n).astype(dtype)
+    b = rng.standard_normal(n).astype(dtype)
+    da, db = rocm.DeviceBuffer.from_numpy(a), rocm.DeviceBuffer.from_numpy(b)
+    out = rocm.DeviceBuffer((n,), dtype)
+    rocm.add_raw(dtype, da.ptr, db.ptr, out.ptr, n)
+    assert np.array_equal(out.numpy(), (a.astype(np.float32) + b.astype(np.float32)).astype(dtype))
+    rocm.neg_raw(dtype, da.ptr, out.ptr, n)
+    assert np.array_equal(out.numpy(), -a)
+    rocm.fill_raw(dtype, out.ptr, n, 1.0)
+    assert np.array_equal(out.numpy(), np.ones(n, dtype))
+    rocm.add_raw(dtype, out.ptr, out.ptr, out.ptr, n)  # aliasing is allowed
+    assert np.array_equal(out.numpy(), np.full(n, 2, dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_copy_compact_of_permuted_and_broadcast_views(dtype):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((3, 5, 4, 8)).astype(dtype)  # [B,T,H,D]
+    dx = rocm.DeviceBuffer.from_numpy(x)
+    # the [B,H,T,D] view of a [B,T,H,D] buffer (src/models/gpt.rs:135-137)
+    B, T, H, D = x.shape
+    out = rocm.DeviceBuffer((B, H, T, D), dtype)
+    rocm.copy_compact_raw(dtype, dx.ptr, (B, H, T, D), (T * H * D, D, H * D, 1), out.ptr)
+    assert np.array_equal(out.numpy(), x.transpose(0, 2, 1, 3))
+    # the D-slowest view apply_rotary_emb's cat leaves behind (innermost stride != 1)
+    y = np.ascontiguousarray(x.transpose(3, 0, 1, 2))  # memory [D,B,T,H]
+    dy = rocm.DeviceBuffer.from_numpy(y)
+    rocm.copy_compact_raw(dtype, dy.ptr, (B, T, H, D), (T * H, H, 1, B * T * H), out.ptr)
+    assert np.array_equal(out.numpy().reshape(B, T, H, D), x)
+    # stride 0 broadcasts (the mask's head axis, src/ops.rs:730-804)
+    row = rocm.DeviceBuffer.from_numpy(x[0, 0, 0])
+    outb = rocm.DeviceBuffer((6, D), dtype)
+    rocm.copy_compact_raw(dtype, row.ptr, (6, D), (0, 1), outb.ptr)
+    assert np.array_equal(outb.numpy(), np.broadcast_to(x[0, 0, 0], (6, D)))
+
+
+@pytest.mark.gpu
+def test_elementwise_helper_errors():
+    buf = rocm.DeviceBuffer((8,), np.float32)
+    with pytest.raises(rocm.RocmError):
+        rocm.copy_compact_raw(np.float32, buf.ptr, (2,) * 7, (1,) * 7, buf.ptr)  # ndim > 6
+    with pytest.raises(rocm.RocmError):
+        rocm.copy_compact_raw(np.float32, buf.ptr, (8,), (-1,), buf.ptr)  # negative stride
+    with pytest.raises(rocm.RocmError):
+        rocm.add_raw(np.float32, None, buf.ptr, buf.ptr, 8)  # null pointer
