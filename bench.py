@@ -150,6 +150,37 @@ def bench_copy(steps: int, warmup: int):
                 gbs=4.0 * n / (us * 1e-6) / 1e9)
 
 
+def bench_rope(steps: int, warmup: int):
+    """RoPE + head split (forward) and inverse RoPE + head merge (backward) at the C2
+    geometry; HBM-bound: each launch reads one [B,T,H,D] tensor and writes one."""
+    B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
+    import oracle  # only for the cos/sin tables of this profiling aid
+    cos, sin = oracle.rope_tables(T, D, dtype=np.float16)
+    x = synth.normal((B, T, H, D), synth.tensor_seed(0, "rope", "x"), 1.0).astype(np.float16)
+    dx, dc, ds = (rocm.DeviceBuffer.from_numpy(a) for a in (x, cos, sin))
+    y = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    g = rocm.DeviceBuffer((B, T, H, D), np.float16)
+
+    def step():
+        rocm.rope_fwd_raw(np.float16, dx.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, D)
+        rocm.rope_bwd_raw(np.float16, y.ptr, dc.ptr, ds.ptr, g.ptr, B, T, H, D)
+
+    for _ in range(warmup):
+        step()
+    rocm.sync()
+    rocm.profile_enable(True)
+    for _ in range(steps):
+        step()
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    nbytes = 2.0 * B * T * H * D * 2
+    out = {"bytes_per_launch": nbytes}
+    for name, (calls, ms) in prof.items():
+        us = 1e3 * ms / calls
+        out[name] = {"avg_us": us, "GB/s": nbytes / (us * 1e-6) / 1e9}
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -181,7 +212,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -195,6 +226,8 @@ def main():
     if args.only != "all":
         if args.only == "decode":
             print(json.dumps({"only": "decode", **bench_decode(args.steps, args.warmup)}))
+        elif args.only == "rope":
+            print(json.dumps({"only": "rope", **bench_rope(args.steps, args.warmup)}))
         elif args.only == "copy":
             print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
         else:

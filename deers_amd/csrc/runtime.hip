@@ -30,6 +30,9 @@ void launch_add(int dtype_f16, const void* a, const void* b, void* out, size_t n
 void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t stream);
 void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
                          const int64_t* strides, int ndim, void* dst, hipStream_t stream);
+void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
+                 const void* cos, const void* sin, void* dst, int B, int T, int H, int D,
+                 hipStream_t stream);
 }  // namespace deers
 
 namespace {
@@ -546,6 +549,65 @@ int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
     if (shape[d] < 0 || strides[d] < 0)
       return fail(DEERS_ROCM_ERR_LAYOUT, "copy_compact: negative extent or stride in dim %d", d);
   deers::launch_copy_strided(dtype == DEERS_ROCM_F16, src, shape, strides, ndim, dst, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- rotary embedding fused with the head split / merge ----
+
+static int rope_common(const char* what, int dtype, const void* src, const int64_t* strides,
+                       const void* cos, const void* sin, void* dst, int64_t B, int64_t T,
+                       int64_t H, int64_t D, int64_t* resolved, bool inverse) {
+  if (int rc = check_dtype(dtype)) return rc;
+  if (!src || !cos || !sin || !dst) return fail(DEERS_ROCM_ERR_ARG, "%s: null pointer", what);
+  const int64_t per16 = dtype == DEERS_ROCM_F16 ? 8 : 4;
+  if (B < 1 || T < 1 || H < 1 || D < 2 || (D / 2) % per16 || D % 2 ||
+      B * T * H * D >= (int64_t(1) << 40) || B > INT32_MAX || T > INT32_MAX || H > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG,
+                "%s: need B,T,H >= 1 and D/2 a multiple of %lld elements (16 bytes)", what,
+                (long long)per16);
+  // compact defaults: forward input [B,T,H,D], backward input [B,H,T,D]
+  resolved[0] = T * H * D;
+  resolved[1] = inverse ? T * D : H * D;
+  resolved[2] = D;
+  int64_t last = 1;
+  if (strides) {
+    resolved[0] = strides[0]; resolved[1] = strides[1]; resolved[2] = strides[2];
+    last = strides[3];
+  }
+  if (last != 1)
+    return fail(DEERS_ROCM_ERR_LAYOUT, "%s: innermost stride is %lld, need 1", what, (long long)last);
+  for (int d = 0; d < 3; ++d)
+    if (resolved[d] < 0 || resolved[d] % per16)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "%s: strides must be non-negative multiples of 16 bytes", what);
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) |
+       reinterpret_cast<uintptr_t>(cos) | reinterpret_cast<uintptr_t>(sin)) & 15)
+    return fail(DEERS_ROCM_ERR_LAYOUT, "%s: pointers must be 16-byte aligned", what);
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides, const void* cos,
+                        const void* sin, void* y, int64_t B, int64_t T, int64_t H, int64_t D) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  int64_t st[3];
+  if (int rc = rope_common("rope_fwd", dtype, x, x_strides, cos, sin, y, B, T, H, D, st, false))
+    return rc;
+  deers::launch_rope(dtype == DEERS_ROCM_F16, false, x, st, cos, sin, y, (int)B, (int)T, (int)H,
+                     (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_rope_bwd(int dtype, const void* dy, const int64_t* dy_strides, const void* cos,
+                        const void* sin, void* dx, int64_t B, int64_t T, int64_t H, int64_t D) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  int64_t st[3];
+  if (int rc = rope_common("rope_bwd", dtype, dy, dy_strides, cos, sin, dx, B, T, H, D, st, true))
+    return rc;
+  deers::launch_rope(dtype == DEERS_ROCM_F16, true, dy, st, cos, sin, dx, (int)B, (int)T, (int)H,
+                     (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

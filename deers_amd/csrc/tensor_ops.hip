@@ -55,9 +55,31 @@ __global__ __launch_bounds__(256) void copy_strided_kernel(const T* src, T* dst,
   }
 }
 
+// Fast path of copy_strided for views whose rows are contiguous runs of 16-byte
+// chunks (unit innermost stride, everything 16-byte aligned): one thread moves one
+// chunk, index arithmetic is 32-bit and runs once per 16 bytes instead of once per
+// element.  `v` describes the view in chunks.
+struct View6u {
+  uint32_t shape[6];
+  uint32_t stride[6];
+};
+__global__ __launch_bounds__(256) void copy_chunks_kernel(const uint4* src, uint4* dst, View6u v,
+                                                          uint32_t n) {
+  for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    uint32_t rem = i, off = 0;
+#pragma unroll
+    for (int d = 5; d >= 0; --d) {
+      const uint32_t q = rem / v.shape[d];
+      off += (rem - q * v.shape[d]) * v.stride[d];
+      rem = q;
+    }
+    dst[i] = src[off];
+  }
+}
+
 inline unsigned grid_for(size_t n) {
   const size_t blocks = (n + 255) / 256;
-  return (unsigned)(blocks < 1 ? 1 : (blocks > 8192 ? 8192 : blocks));
+  return (unsigned)(blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks));
 }
 
 }  // namespace
@@ -99,6 +121,28 @@ void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
     n *= (size_t)v.shape[d];
   }
   if (n == 0) return;
+  // rows of whole 16-byte chunks, everything aligned, offsets within 32 bits
+  const int64_t per16 = dtype_f16 ? 8 : 4;
+  bool chunked = v.stride[5] == 1 && v.shape[5] % per16 == 0 && n / per16 < (size_t(1) << 31) &&
+                 ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+  int64_t span = 0;
+  for (int d = 0; d < 5 && chunked; ++d) {
+    chunked = v.stride[d] % per16 == 0;
+    span += (v.shape[d] - 1) * v.stride[d];
+  }
+  if (chunked && (span + v.shape[5]) / per16 < (int64_t(1) << 32)) {
+    View6u u;
+    for (int d = 0; d < 5; ++d) {
+      u.shape[d] = (uint32_t)v.shape[d];
+      u.stride[d] = (uint32_t)(v.stride[d] / per16);
+    }
+    u.shape[5] = (uint32_t)(v.shape[5] / per16);
+    u.stride[5] = 1;
+    const uint32_t nc = (uint32_t)(n / per16);
+    hipLaunchKernelGGL(copy_chunks_kernel, dim3(grid_for(nc)), dim3(256), 0, stream,
+                       (const uint4*)src, (uint4*)dst, u, nc);
+    return;
+  }
   if (dtype_f16)
     hipLaunchKernelGGL(copy_strided_kernel<half_t>, dim3(grid_for(n)), dim3(256), 0, stream,
                        (const half_t*)src, (half_t*)dst, v, n);

@@ -205,6 +205,25 @@ static int run_gpu(const std::string& dir) {
     Tensor yn = causal_self_attention(q.detach(), k.detach(), v.detach());
     EXPECT(!yn.requires_grad() && yn.op() == nullptr);
   }
+  // the whole sub-graph of src/models/gpt.rs:135-147: RoPE on the q and k projections,
+  // v as a permuted view, fused attention, head merge, reverse sweep
+  {
+    auto [cos, sin] = precompute_rotary_embeddings(T, D, 10000.0f, dtype);
+    Tensor qr = rotary_heads(xq, cos, sin), kr = rotary_heads(xk, cos, sin);
+    EXPECT(qr.is_compact() && (qr.shape() == std::vector<int64_t>{B, H, T, D}));
+    EXPECT(std::string(qr.op()->name()) == "RotaryHeads");
+    Tensor yr = causal_self_attention(qr, kr, v).permute({0, 2, 1, 3}).compact();
+    dump(yr, dir + "/y_rope.bin");
+    GradientStore gr = yr.backward_from(seed);
+    for (auto [t, name] : {std::pair<const Tensor*, const char*>{&xq, "dq_rope.bin"}, {&xk, "dk_rope.bin"}, {&xv, "dv_rope.bin"}}) {
+      const Tensor* g = gr.get(t->id());
+      EXPECT(g != nullptr);
+      if (g) {
+        EXPECT(g->shape() == t->shape());
+        dump(*g, dir + "/" + name);
+      }
+    }
+  }
   if (L > 0) {
     Tensor dq = load("dec_q.bin", {B, H, D});
     Tensor kc = load("dec_k.bin", {B, H, L, D}), vc = load("dec_v.bin", {B, H, L, D});

@@ -2,6 +2,8 @@
 #include "ops.h"
 
 #include <cmath>
+#include <cstring>
+#include <vector>
 
 #include "../../include/deers_rocm.h"
 
@@ -16,6 +18,25 @@ Tensor empty(const std::vector<int64_t>& shape, DType dtype, bool is_backed) {
   Layout l(shape);
   auto st = std::make_shared<RocmStorage>(l.size(), dtype, is_backed);
   return Tensor(std::move(st), std::move(l), false, nullptr);
+}
+
+// IEEE binary16 bits of a float, round to nearest even (what f16::from_f32 does).
+uint16_t f32_to_f16_bits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (x > 0x7f800000u ? 0x200u : 0));
+  if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);  // rounds to infinity
+  if (x < 0x38800000u) {                                    // subnormal or zero
+    if (x < 0x33000000u) return (uint16_t)sign;
+    const int shift = 126 - (int)(x >> 23);                 // 14..24
+    const uint32_t mant = (x & 0x7fffffu) | 0x800000u;
+    const uint32_t q = mant >> shift, rem = mant & ((1u << shift) - 1), half = 1u << (shift - 1);
+    return (uint16_t)(sign | (q + ((rem > half) || (rem == half && (q & 1)))));
+  }
+  const uint32_t q = (x - 0x38000000u) >> 13, rem = x & 0x1fffu;
+  return (uint16_t)(sign | (q + ((rem > 0x1000u) || (rem == 0x1000u && (q & 1)))));
 }
 
 // A [B,H,T,D] view the kernels take as is: unit D stride (alignment is the
@@ -142,6 +163,69 @@ void FusedCausalAttention::backward(GradientStore& grads, const Tensor& out_grad
   grads.accumulate(q_, dq);
   grads.accumulate(k_, dk);
   grads.accumulate(v_, dv);
+}
+
+// ---- RotaryHeads ----
+RotaryHeads::RotaryHeads(Tensor x, Tensor cos, Tensor sin)
+    : x_(std::move(x)), cos_(std::move(cos)), sin_(std::move(sin)) {
+  if (x_.layout().ndim() != 4) throw std::logic_error("RoPE expects a 4D attention tensor");
+  if (cos_.shape() != sin_.shape()) throw std::logic_error("RoPE cos/sin shapes must match");
+  const int64_t D = x_.shape()[3];
+  if (D % 2) throw std::logic_error("RoPE requires an even head dimension");
+  if (cos_.layout().ndim() != 4 || cos_.shape()[3] != D / 2)
+    throw std::logic_error("RoPE cache last dimension must equal head_dim / 2");
+  if (cos_.shape()[1] != x_.shape()[1]) throw std::logic_error("RoPE cache must match sequence length");
+  if (cos_.dtype() != x_.dtype() || sin_.dtype() != x_.dtype())
+    throw std::logic_error("RoPE cache dtype must match the tensor");
+}
+
+Tensor RotaryHeads::forward(std::unique_ptr<RotaryHeads> self) {
+  const Tensor x = kernel_ready(self->x_);
+  const Tensor cos = self->cos_.compact(), sin = self->sin_.compact();
+  const int64_t B = x.shape()[0], T = x.shape()[1], H = x.shape()[2], D = x.shape()[3];
+  Tensor y = empty({B, H, T, D}, x.dtype(), true);
+  check(deers_rocm_rope_fwd((int)x.dtype(), x.data(), x.layout().strides.data(), cos.data(),
+                            sin.data(), y.data(), B, T, H, D));
+  return Tensor(y.storage(), y.layout(), false, std::move(self));
+}
+
+void RotaryHeads::backward(GradientStore& grads, const Tensor& out_grad) const {
+  const Tensor g = kernel_ready(out_grad);  // logical [B,H,T,D]
+  const Tensor cos = cos_.compact(), sin = sin_.compact();
+  const int64_t B = g.shape()[0], H = g.shape()[1], T = g.shape()[2], D = g.shape()[3];
+  Tensor dx = empty({B, T, H, D}, g.dtype(), true);
+  check(deers_rocm_rope_bwd((int)g.dtype(), g.data(), g.layout().strides.data(), cos.data(),
+                            sin.data(), dx.data(), B, T, H, D));
+  grads.accumulate(x_, dx);
+}
+
+std::pair<Tensor, Tensor> precompute_rotary_embeddings(int64_t seq_len, int64_t head_dim,
+                                                       float base, DType dtype) {
+  if (head_dim % 2) throw std::logic_error("RoPE requires an even head dimension");
+  const int64_t half = head_dim / 2;
+  std::vector<float> inv_freq(half);
+  for (int64_t i = 0; i < half; ++i)
+    inv_freq[i] = 1.0f / std::pow(base, (float)(2 * i) / (float)head_dim);
+  std::vector<float> c(seq_len * half), s(seq_len * half);
+  for (int64_t t = 0; t < seq_len; ++t)
+    for (int64_t i = 0; i < half; ++i) {
+      const float a = (float)t * inv_freq[i];
+      c[t * half + i] = std::cos(a);
+      s[t * half + i] = std::sin(a);
+    }
+  const std::vector<int64_t> shape{1, seq_len, 1, half};
+  if (dtype == DType::F32)
+    return {Tensor::from_host(c.data(), shape, dtype), Tensor::from_host(s.data(), shape, dtype)};
+  std::vector<uint16_t> ch(c.size()), sh(s.size());
+  for (size_t i = 0; i < c.size(); ++i) {
+    ch[i] = f32_to_f16_bits(c[i]);
+    sh[i] = f32_to_f16_bits(s[i]);
+  }
+  return {Tensor::from_host(ch.data(), shape, dtype), Tensor::from_host(sh.data(), shape, dtype)};
+}
+
+Tensor rotary_heads(const Tensor& x, const Tensor& cos, const Tensor& sin) {
+  return RotaryHeads::forward(std::make_unique<RotaryHeads>(x, cos, sin));
 }
 
 Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v) {

@@ -6,6 +6,8 @@
 #ifndef DEERS_HOST_OPS_H
 #define DEERS_HOST_OPS_H
 
+#include <utility>
+
 #include "tensor.h"
 
 namespace deers_host {
@@ -78,6 +80,28 @@ class FusedCausalAttention : public TensorOp {
   double scale_;
   Tensor saved_o_, saved_lse_;  // set by forward, created with no op
 };
+
+// apply_rotary_emb on a [B,T,H,D] projection followed by permute([0,2,1,3])
+// (src/models/gpt.rs:49-73, 135-136) as one op: returns the rotated heads as compact
+// [B,H,T,D]; the backward hands the [B,T,H,D] gradient to the projection.  cos and
+// sin are the tables of precompute_rotary_embeddings and carry no gradient.
+class RotaryHeads : public TensorOp {
+ public:
+  RotaryHeads(Tensor x, Tensor cos, Tensor sin);
+  static Tensor forward(std::unique_ptr<RotaryHeads> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&x_}; }
+  const char* name() const override { return "RotaryHeads"; }
+
+ private:
+  Tensor x_, cos_, sin_;
+};
+
+// cos, sin tables [1,T,1,D/2] in `dtype` (src/models/gpt.rs:12-47): f32 arithmetic on
+// the host, then one cast.
+std::pair<Tensor, Tensor> precompute_rotary_embeddings(int64_t seq_len, int64_t head_dim,
+                                                       float base, DType dtype);
+Tensor rotary_heads(const Tensor& x, const Tensor& cos, const Tensor& sin);
 
 // The call site of src/models/gpt.rs:139-144: scale = 1/sqrt(head_dim) computed in
 // f64 and narrowed to f32 (src/storage.rs:115-117).

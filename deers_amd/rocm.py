@@ -207,6 +207,20 @@ def copy_compact_raw(dtype, src, shape, strides, dst):
                                           ctypes.c_int(nd), dst))
 
 
+def rope_fwd_raw(dtype, x, cos, sin, y, B, T, H, D, x_strides=None):
+    """deers_rocm_rope_fwd: x logical [B,T,H,D] -> y compact [B,H,T,D]."""
+    _check(load().deers_rocm_rope_fwd(
+        ctypes.c_int(dtype_code(dtype)), x, _strides(x_strides), cos, sin, y, ctypes.c_int64(B),
+        ctypes.c_int64(T), ctypes.c_int64(H), ctypes.c_int64(D)))
+
+
+def rope_bwd_raw(dtype, dy, cos, sin, dx, B, T, H, D, dy_strides=None):
+    """deers_rocm_rope_bwd: dy logical [B,H,T,D] -> dx compact [B,T,H,D]."""
+    _check(load().deers_rocm_rope_bwd(
+        ctypes.c_int(dtype_code(dtype)), dy, _strides(dy_strides), cos, sin, dx, ctypes.c_int64(B),
+        ctypes.c_int64(T), ctypes.c_int64(H), ctypes.c_int64(D)))
+
+
 def default_scale(D: int) -> float:
     """1/sqrt(D) in double, narrowed to f32 (src/models/gpt.rs:139, src/storage.rs:115-117)."""
     return float(np.float32(1.0 / np.sqrt(float(D))))

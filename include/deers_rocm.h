@@ -192,6 +192,27 @@ int deers_rocm_neg(int dtype, const void* a, void* out, size_t n);
 int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
                             const int64_t* strides, int ndim, void* dst);
 
+/* ---- rotary embedding fused with the head split / merge -----------------------
+ * The neighbours of the attention core in CausalSelfAttention::forward
+ * (src/models/gpt.rs:115-137): apply_rotary_emb on the [B,T,H,D] projections
+ * (src/models/gpt.rs:49-73: narrow, 4 multiplies, 2 adds, cat) followed by
+ * permute([0,2,1,3]).  cos and sin are the [1,T,1,D/2] tables of
+ * precompute_rotary_embeddings (src/models/gpt.rs:12-47), compact, in the tensor's
+ * dtype.  D/2 must be a multiple of 16 bytes; arithmetic is f32 with one rounding. */
+
+/* y (compact [B,H,T,D]) = permute(apply_rotary_emb(x)), x logical [B,T,H,D] with
+ * element strides x_strides = {b,t,h,d} (NULL = compact, d must be 1). */
+int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides,
+                        const void* cos, const void* sin, void* y,
+                        int64_t B, int64_t T, int64_t H, int64_t D);
+
+/* Backward of the above (Permute::backward then the element-wise backward bodies,
+ * src/ops.rs:687-727, 130-260): dx (compact [B,T,H,D]) from dy logical [B,H,T,D]
+ * with element strides dy_strides = {b,h,t,d} (NULL = compact, d must be 1). */
+int deers_rocm_rope_bwd(int dtype, const void* dy, const int64_t* dy_strides,
+                        const void* cos, const void* sin, void* dx,
+                        int64_t B, int64_t T, int64_t H, int64_t D);
+
 #ifdef __cplusplus
 }
 #endif

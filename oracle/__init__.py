@@ -3,8 +3,9 @@
 Only tests, the smoke check and the CPU-baseline leg of the benchmark may import
 this package; the shipped library never does.  The arithmetic lives in
 ``attention_ref.cc`` (a restatement of the reference's CPU attention,
-src/models/gpt.rs:139-144 and its autograd backward); this module only moves
-numpy arrays across the C boundary.
+src/models/gpt.rs:139-144 and its autograd backward); this module moves numpy
+arrays across the C boundary and restates the rotary embedding around the core
+(src/models/gpt.rs:12-73) directly in numpy.
 """
 from __future__ import annotations
 
@@ -178,3 +179,45 @@ def attn_bwd(q, k, v, dy, scale: float | None = None, dtype=np.float32, nthreads
            _I64(H), _I64(tq), _I64(tk), _I64(D), ctypes.c_double(scale), _ptr(dq[b0:b1]),
            _ptr(dk[b0:b1]), _ptr(dv[b0:b1]), ctypes.c_int(nthreads))
     return dq, dk, dv
+
+
+# ---- rotary embedding (numpy restatement; byte/float arithmetic in the reference's order) ----
+
+def rope_tables(seq_len: int, head_dim: int, base: float = 10000.0, dtype=np.float32):
+    """cos, sin [seq_len, head_dim/2] as precompute_rotary_embeddings builds them
+    (src/models/gpt.rs:12-47): inv_freq_i = 1 / base^(2i/D) in f32, angle = t * inv_freq
+    in f32, cos/sin in f32, then cast to `dtype`."""
+    assert head_dim % 2 == 0, "RoPE requires an even head dimension"
+    half = head_dim // 2
+    channel = (2 * np.arange(half)).astype(np.float32)
+    inv_freq = (np.float32(1.0) / np.power(np.float32(base), channel / np.float32(head_dim))
+                ).astype(np.float32)
+    t = np.arange(seq_len, dtype=np.float32)[:, None]
+    freqs = (t * inv_freq[None, :]).astype(np.float32)
+    return np.cos(freqs).astype(dtype), np.sin(freqs).astype(dtype)
+
+
+def rope_apply(x: np.ndarray, cos: np.ndarray, sin: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """apply_rotary_emb on x [B,T,H,D] (src/models/gpt.rs:49-73):
+    y1 = x1*cos + x2*sin, y2 = x1*(sin*-1) + x2*cos, cat along D; evaluated in `dtype`
+    (float32 for the f32 path and as the oracle of the f16 path on rounded inputs)."""
+    x = np.asarray(x, dtype=dtype)
+    half = x.shape[3] // 2
+    c = np.asarray(cos, dtype=dtype)[None, :, None, :]
+    s = np.asarray(sin, dtype=dtype)[None, :, None, :]
+    x1, x2 = x[..., :half], x[..., half:]
+    y1 = x1 * c + x2 * s
+    y2 = x1 * (s * dtype(-1.0)) + x2 * c
+    return np.concatenate([y1, y2], axis=3)
+
+
+def rope_apply_bwd(dy: np.ndarray, cos: np.ndarray, sin: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """Gradient of rope_apply w.r.t. x for upstream dy [B,T,H,D], from the backward
+    bodies of cat / add / mul (src/ops.rs:130-260): dx1 = dy1*cos + dy2*(-sin),
+    dx2 = dy1*sin + dy2*cos."""
+    dy = np.asarray(dy, dtype=dtype)
+    half = dy.shape[3] // 2
+    c = np.asarray(cos, dtype=dtype)[None, :, None, :]
+    s = np.asarray(sin, dtype=dtype)[None, :, None, :]
+    d1, d2 = dy[..., :half], dy[..., half:]
+    return np.concatenate([d1 * c + d2 * (s * dtype(-1.0)), d1 * s + d2 * c], axis=3)

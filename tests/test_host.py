@@ -66,6 +66,19 @@ def test_host_fused_attention_matches_oracle(tmp_path, dtype, B, H, T, D, L, tol
     assert err(out("y.bin"), want_o) <= tol
     for name, ref in zip(("dq.bin", "dk.bin", "dv.bin"), want):
         assert err(out(name), ref) <= tol, name
+    # RoPE on q and k around the core, against the composed oracle
+    cos, sin = oracle.rope_tables(T, D, dtype=dtype)
+    c32, s32 = cos.astype(np.float32), sin.astype(np.float32)
+    hd = lambda a: a.transpose(0, 2, 1, 3)  # [B,T,H,D] <-> [B,H,T,D]
+    qr = hd(oracle.rope_apply(bthd(f32["q"]), c32, s32))
+    kr = hd(oracle.rope_apply(bthd(f32["k"]), c32, s32))
+    want_yr = oracle.attn_fwd(qr, kr, f32["v"])
+    gq, gk, gv = oracle.attn_bwd(qr, kr, f32["v"], f32["do"])
+    want_r = (oracle.rope_apply_bwd(bthd(gq), c32, s32), oracle.rope_apply_bwd(bthd(gk), c32, s32),
+              bthd(gv))
+    assert float(np.max(np.abs(out("y_rope.bin") - bthd(want_yr)))) <= tol
+    for name, ref in zip(("dq_rope.bin", "dk_rope.bin", "dv_rope.bin"), want_r):
+        assert float(np.max(np.abs(out(name) - ref))) <= tol, name
     if dtype == np.float16:
         # two ops on the same inputs give the same bits, and x + x is exact in f16
         assert np.array_equal(out("dv_twice.bin"), 2 * out("dv.bin"))

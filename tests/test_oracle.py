@@ -218,3 +218,87 @@ def test_fixture_inputs_regenerate_from_seed():
     x = synth.attention_inputs("f16_b2h3t33d64", B, H, T, D, np.float16, base_seed=seed)
     for name in ("q", "k", "v", "do"):
         np.testing.assert_array_equal(x[name], f[name])
+
+
+# ---- rotary embedding oracle: pinned by closed forms and invariants, not by retyping ----
+
+def test_rope_tables_closed_forms():
+    cos, sin = oracle.rope_tables(5, 8, base=10000.0)
+    assert cos.shape == (5, 4) and sin.shape == (5, 4)
+    # t = 0 is the identity rotation
+    assert np.array_equal(cos[0], np.ones(4, np.float32)) and np.array_equal(sin[0], np.zeros(4, np.float32))
+    # channel 0 has inv_freq 1: the angle is t itself
+    assert np.allclose(cos[:, 0], np.cos(np.arange(5.0)), atol=1e-6)
+    assert np.allclose(sin[:, 0], np.sin(np.arange(5.0)), atol=1e-6)
+    # channel i has inv_freq base^(-2i/D): last channel of D=8 is 10000^(-6/8) = 10^-3
+    assert np.allclose(sin[3, 3], np.sin(3.0 * 1e-3), atol=1e-7)
+    # half tables in f16 are the rounded f32 ones
+    ch, sh = oracle.rope_tables(5, 8, dtype=np.float16)
+    assert np.array_equal(ch, cos.astype(np.float16)) and np.array_equal(sh, sin.astype(np.float16))
+
+
+def test_rope_apply_known_rotation_and_sign():
+    # D = 2, one channel, angle = t: a plain 2-D rotation by -t of (x1, x2)
+    cos, sin = oracle.rope_tables(3, 2)
+    x = np.zeros((1, 3, 1, 2), np.float32)
+    x[0, :, 0] = [1.0, 0.0]
+    y = oracle.rope_apply(x, cos, sin)
+    # (1,0) -> (cos t, -sin t): a dropped sign or swapped halves fails here
+    assert np.allclose(y[0, :, 0, 0], np.cos(np.arange(3.0)), atol=1e-6)
+    assert np.allclose(y[0, :, 0, 1], -np.sin(np.arange(3.0)), atol=1e-6)
+    x[0, :, 0] = [0.0, 1.0]
+    y = oracle.rope_apply(x, cos, sin)
+    assert np.allclose(y[0, :, 0, 0], np.sin(np.arange(3.0)), atol=1e-6)
+    assert np.allclose(y[0, :, 0, 1], np.cos(np.arange(3.0)), atol=1e-6)
+
+
+def test_rope_apply_invariants():
+    rng = np.random.default_rng(11)
+    B, T, H, D = 2, 7, 3, 8
+    cos, sin = oracle.rope_tables(T, D)
+    q = rng.standard_normal((B, T, H, D))
+    k = rng.standard_normal((B, T, H, D))
+    c64, s64 = cos.astype(np.float64), sin.astype(np.float64)
+    yq = oracle.rope_apply(q, c64, s64, dtype=np.float64)
+    yk = oracle.rope_apply(k, c64, s64, dtype=np.float64)
+    half = D // 2
+    # each (x1_i, x2_i) pair is rotated: its norm is preserved
+    n_in = q[..., :half] ** 2 + q[..., half:] ** 2
+    n_out = yq[..., :half] ** 2 + yq[..., half:] ** 2
+    assert np.allclose(n_in, n_out, atol=1e-6)
+    # relative-position property: <rope(q,t1), rope(k,t2)> depends on t1 - t2 only.
+    # Use the same q, k vector at every position and compare (t1,t2) = (5,3) with (4,2), (2,0).
+    qs = np.broadcast_to(q[:, :1], q.shape).copy()
+    ks = np.broadcast_to(k[:, :1], k.shape).copy()
+    yqs = oracle.rope_apply(qs, c64, s64, dtype=np.float64)
+    yks = oracle.rope_apply(ks, c64, s64, dtype=np.float64)
+    dot = lambda t1, t2: np.einsum("bhd,bhd->bh", yqs[:, t1], yks[:, t2])
+    # the f32 tables make angles exact only to ~1e-7 relative
+    assert np.allclose(dot(5, 3), dot(4, 2), atol=1e-5) and np.allclose(dot(5, 3), dot(2, 0), atol=1e-5)
+    # position 0 is the identity
+    assert np.array_equal(yq[:, 0], q[:, 0])
+
+
+def test_rope_backward_is_the_transpose():
+    rng = np.random.default_rng(12)
+    B, T, H, D = 1, 5, 2, 8
+    cos, sin = oracle.rope_tables(T, D)
+    c64, s64 = cos.astype(np.float64), sin.astype(np.float64)
+    x = rng.standard_normal((B, T, H, D))
+    dy = rng.standard_normal((B, T, H, D))
+    # the op is linear: <rope(x), dy> = <x, rope_bwd(dy)>, and central differences agree
+    lhs = np.sum(oracle.rope_apply(x, c64, s64, dtype=np.float64) * dy)
+    dx = oracle.rope_apply_bwd(dy, c64, s64, dtype=np.float64)
+    assert np.isclose(lhs, np.sum(x * dx), rtol=1e-12)
+    eps = 1e-6
+    for idx in [(0, 1, 0, 2), (0, 4, 1, 6), (0, 3, 1, 0)]:
+        xp, xm = x.copy(), x.copy()
+        xp[idx] += eps
+        xm[idx] -= eps
+        fd = (np.sum(oracle.rope_apply(xp, c64, s64, dtype=np.float64) * dy)
+              - np.sum(oracle.rope_apply(xm, c64, s64, dtype=np.float64) * dy)) / (2 * eps)
+        assert np.isclose(fd, dx[idx], atol=1e-8)
+    # a rotation's transpose is its inverse
+    back = oracle.rope_apply_bwd(oracle.rope_apply(x, c64, s64, dtype=np.float64), c64, s64,
+                                 dtype=np.float64)
+    assert np.allclose(back, x, atol=1e-6)

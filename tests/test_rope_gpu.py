@@ -1,0 +1,103 @@
+"""RoPE fused with the head split / merge (deers_rocm_rope_fwd / _bwd) against the numpy
+restatement of apply_rotary_emb + permute (src/models/gpt.rs:49-73, 135-137)."""
+import numpy as np
+import pytest
+
+import oracle
+from deers_amd import rocm, synth
+
+TOL = {np.dtype(np.float16): 5e-3, np.dtype(np.float32): 1e-4}
+
+SHAPES = [(1, 1, 1, 32), (2, 5, 3, 32), (2, 33, 3, 64), (1, 130, 2, 128), (8, 1024, 12, 64)]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    if not rocm.available():
+        pytest.skip("no gfx950 device")
+    rocm.init(0)
+
+
+def _inputs(B, T, H, D, dtype, seed):
+    x = synth.normal((B, T, H, D), synth.tensor_seed(seed, "rope", "x"), 1.0).astype(dtype)
+    dy = synth.normal((B, H, T, D), synth.tensor_seed(seed, "rope", "dy"), 1.0).astype(dtype)
+    cos, sin = oracle.rope_tables(T, D, dtype=dtype)
+    return x, dy, cos, sin
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("B,T,H,D", SHAPES)
+def test_rope_fwd_bwd_match_oracle(dtype, B, T, H, D):
+    x, dy, cos, sin = _inputs(B, T, H, D, dtype, 21)
+    dx_, dc, ds = (rocm.DeviceBuffer.from_numpy(a) for a in (x, cos, sin))
+    y = rocm.DeviceBuffer((B, H, T, D), dtype)
+    rocm.rope_fwd_raw(dtype, dx_.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, D)
+    want = oracle.rope_apply(x.astype(np.float32), cos.astype(np.float32),
+                             sin.astype(np.float32)).transpose(0, 2, 1, 3)
+    assert np.max(np.abs(y.numpy().astype(np.float64) - want)) <= TOL[np.dtype(dtype)]
+    # position 0 passes through bit-exactly (cos = 1, sin = 0)
+    assert np.array_equal(y.numpy()[:, :, 0], x.transpose(0, 2, 1, 3)[:, :, 0])
+
+    ddy = rocm.DeviceBuffer.from_numpy(dy)
+    gx = rocm.DeviceBuffer((B, T, H, D), dtype)
+    rocm.rope_bwd_raw(dtype, ddy.ptr, dc.ptr, ds.ptr, gx.ptr, B, T, H, D)
+    want_dx = oracle.rope_apply_bwd(dy.astype(np.float32).transpose(0, 2, 1, 3),
+                                    cos.astype(np.float32), sin.astype(np.float32))
+    assert np.max(np.abs(gx.numpy().astype(np.float64) - want_dx)) <= TOL[np.dtype(dtype)]
+
+
+@pytest.mark.gpu
+def test_rope_round_trip_and_norms_at_full_size():
+    # size-independent properties at the C2 geometry: forward then backward is the identity
+    # up to two f16 roundings, and every (x1_i, x2_i) pair keeps its norm
+    B, T, H, D = 8, 1024, 12, 64
+    x, _, cos, sin = _inputs(B, T, H, D, np.float16, 22)
+    dx_, dc, ds = (rocm.DeviceBuffer.from_numpy(a) for a in (x, cos, sin))
+    y = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    back = rocm.DeviceBuffer((B, T, H, D), np.float16)
+    rocm.rope_fwd_raw(np.float16, dx_.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, D)
+    rocm.rope_bwd_raw(np.float16, y.ptr, dc.ptr, ds.ptr, back.ptr, B, T, H, D)
+    assert np.max(np.abs(back.numpy().astype(np.float32) - x.astype(np.float32))) <= 5e-3
+    yn = y.numpy().astype(np.float32).transpose(0, 2, 1, 3)
+    xf = x.astype(np.float32)
+    n_in = xf[..., :32] ** 2 + xf[..., 32:] ** 2
+    n_out = yn[..., :32] ** 2 + yn[..., 32:] ** 2
+    # f16 rounding of the tables and of the result: a few 2^-11 relative on the squared norm
+    assert np.all(np.abs(n_in - n_out) <= 4e-3 * n_in + 1e-3)
+
+
+@pytest.mark.gpu
+def test_rope_strided_views_and_errors():
+    B, T, H, D = 2, 9, 3, 64
+    x, dy, cos, sin = _inputs(B, T, H, D, np.float16, 23)
+    dc, ds = rocm.DeviceBuffer.from_numpy(cos), rocm.DeviceBuffer.from_numpy(sin)
+    # x as the q third of a fused [B,T,3,H,D] projection buffer
+    qkv = np.zeros((B, T, 3, H, D), np.float16)
+    qkv[:, :, 1] = x
+    dq = rocm.DeviceBuffer.from_numpy(qkv)
+    y = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    import ctypes
+    off = ctypes.c_void_p(dq.ptr.value + H * D * 2)
+    rocm.rope_fwd_raw(np.float16, off, dc.ptr, ds.ptr, y.ptr, B, T, H, D,
+                      x_strides=(T * 3 * H * D, 3 * H * D, D, 1))
+    ref = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    dx_ = rocm.DeviceBuffer.from_numpy(x)
+    rocm.rope_fwd_raw(np.float16, dx_.ptr, dc.ptr, ds.ptr, ref.ptr, B, T, H, D)
+    assert np.array_equal(y.numpy(), ref.numpy())
+    # dy as the [B,T,H,D]-ordered gradient seen through its [B,H,T,D] view
+    dy_bthd = np.ascontiguousarray(dy.transpose(0, 2, 1, 3))
+    g1 = rocm.DeviceBuffer((B, T, H, D), np.float16)
+    g2 = rocm.DeviceBuffer((B, T, H, D), np.float16)
+    ddy, ddy_bthd = rocm.DeviceBuffer.from_numpy(dy), rocm.DeviceBuffer.from_numpy(dy_bthd)
+    rocm.rope_bwd_raw(np.float16, ddy.ptr, dc.ptr, ds.ptr, g1.ptr, B, T, H, D)
+    rocm.rope_bwd_raw(np.float16, ddy_bthd.ptr, dc.ptr, ds.ptr, g2.ptr, B, T, H, D,
+                      dy_strides=(T * H * D, D, H * D, 1))
+    assert np.array_equal(g1.numpy(), g2.numpy())
+    with pytest.raises(rocm.RocmError):  # D/2 not a multiple of 16 bytes
+        rocm.rope_fwd_raw(np.float16, dq.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, 24)
+    with pytest.raises(rocm.RocmError):  # innermost stride must be 1
+        rocm.rope_fwd_raw(np.float16, dq.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, D,
+                          x_strides=(T * H * D, H * D, D, 2))
+    with pytest.raises(rocm.RocmError):
+        rocm.rope_fwd_raw(np.float16, None, dc.ptr, ds.ptr, y.ptr, B, T, H, D)
