@@ -213,45 +213,21 @@ struct DecodeParams {
   float scale_log2;
 };
 
-#ifndef DEERS_SNAKE
-#define DEERS_SNAKE 0
-#endif
-#ifndef DEERS_PRIO
-#define DEERS_PRIO 1
-#endif
-
 // Maps blockIdx.x to (head, block rank).  Workgroups are dealt round-robin to the 8
 // XCDs, so blockIdx.x % 8 is the XCD: every block of one head is given to one XCD
 // (its operands stay in that XCD's L2) and each XCD's list is ordered longest
 // first (rank 0 = the block with the most iterations), which is what the
 // dispatcher's in-order hand-out to free slots needs for an even finish.
 // Returns false for padding ids.
+// (The head and rank stay in vector registers on purpose: forcing them into scalar
+// registers with readfirstlane was measured and raises the kernels' vector register
+// count through the address arithmetic the compiler then hoists out of the loops.)
 __device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int BH, int* bh,
                                           int* rank) {
   const int xcd = blockIdx.x & 7;
-  int idx = blockIdx.x >> 3;
-#if DEERS_SNAKE
-  // variant for launches where every workgroup is resident at once: a CU then holds
-  // items i, i+32, i+64 of the list, and reversing every second group of 32 evens
-  // out the per-CU sums
-  const int per_xcd = n_blocks * heads_per_xcd;
-  const int grp = idx >> 5, pos = idx & 31;
-  const int grp_len = min(32, per_xcd - 32 * grp);
-  if (grp & 1) idx = 32 * grp + (grp_len - 1 - pos);
-#endif
-  // The division runs on the vector unit; without the readfirstlane every value
-  // derived from the head or rank (base pointers, trip counts, tile addresses) would
-  // be kept in vector registers and computed with vector instructions.
-#if DEERS_UNIFORM_IDS == 1
-  *bh = __builtin_amdgcn_readfirstlane((idx % heads_per_xcd) * 8 + xcd);
-  *rank = idx / heads_per_xcd;
-#elif DEERS_UNIFORM_IDS == 2
-  *bh = __builtin_amdgcn_readfirstlane((idx % heads_per_xcd) * 8 + xcd);
-  *rank = __builtin_amdgcn_readfirstlane(idx / heads_per_xcd);
-#else
+  const int idx = blockIdx.x >> 3;
   *bh = (idx % heads_per_xcd) * 8 + xcd;
   *rank = idx / heads_per_xcd;
-#endif
   return *bh < BH;
 }
 
@@ -259,7 +235,7 @@ __device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int B
 // blocks ask the instruction arbiter for priority over the short blocks that share
 // their SIMD, which then fill the gaps.
 __device__ __forceinline__ void set_block_priority(int rank, int n_blocks) {
-#if DEERS_PRIO
+#ifndef DEERS_NO_BLOCK_PRIORITY
   const int q = (4 * rank) / max(n_blocks, 1);  // 0 = longest quarter
   if (q == 0) __builtin_amdgcn_s_setprio(3);
   else if (q == 1) __builtin_amdgcn_s_setprio(2);
