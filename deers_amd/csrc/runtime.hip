@@ -3,6 +3,7 @@
 // checks in front of every kernel launch.  The shape of the runtime follows what
 // the reference's CUDA backend keeps in its OnceLock (one context, one stream,
 // device ordinal fixed at init: src/storage/cuda.rs:462-528).
+#include <rocblas/rocblas.h>
 #include "../../include/deers_rocm.h"
 
 #include <hip/hip_runtime.h>
@@ -43,6 +44,7 @@ struct Runtime {
   hipStream_t stream = nullptr;
   void* workspace = nullptr;  // grows on demand, freed never (process lifetime)
   size_t workspace_bytes = 0;
+  rocblas_handle blas = nullptr;  // created by the first matmul, bound to `stream`
 };
 
 Runtime g_rt;
@@ -550,6 +552,63 @@ int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
       return fail(DEERS_ROCM_ERR_LAYOUT, "copy_compact: negative extent or stride in dim %d", d);
   deers::launch_copy_strided(dtype == DEERS_ROCM_F16, src, shape, strides, ndim, dst, g_rt.stream);
   HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- batched matrix product (library GEMM) ----
+
+int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+                      const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
+                      int64_t batch, int64_t m, int64_t n, int64_t k) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (batch < 0 || m < 0 || n < 0 || k < 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX ||
+      batch > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "matmul: sizes must be in [0, 2^31)");
+  if (batch == 0 || m == 0 || n == 0) return DEERS_ROCM_OK;
+  if (!a || !b || !c) return fail(DEERS_ROCM_ERR_ARG, "matmul: null pointer");
+  if (k == 0) {  // empty sum
+    deers::launch_fill(dtype == DEERS_ROCM_F16, c, (size_t)(batch * m * n), 0.f, g_rt.stream);
+    HIP_TRY(hipGetLastError());
+    return DEERS_ROCM_OK;
+  }
+  // A matrix the BLAS can take needs a unit stride along rows or along columns
+  // (a dimension of extent 1 has no stride to speak of).
+  auto unit = [](int64_t rows, int64_t cols, int64_t rs, int64_t cs, bool* transposed,
+                 int64_t* ld) {
+    if (cs == 1 || cols == 1) { *transposed = false; *ld = rows == 1 ? (rs > cols ? rs : cols) : rs; return rs >= cols || rows == 1; }
+    if (rs == 1 || rows == 1) { *transposed = true; *ld = cols == 1 ? (cs > rows ? cs : rows) : cs; return cs >= rows || cols == 1; }
+    return false;
+  };
+  bool a_t = false, b_t = false;
+  int64_t lda = 0, ldb = 0;
+  if (!unit(m, k, a_rs, a_cs, &a_t, &lda) || !unit(k, n, b_rs, b_cs, &b_t, &ldb) || a_bs < 0 ||
+      b_bs < 0)
+    return fail(DEERS_ROCM_ERR_LAYOUT,
+                "matmul: each operand needs a unit row or column stride and non-overlapping "
+                "lines (a %lld,%lld b %lld,%lld); compact the tensor first",
+                (long long)a_rs, (long long)a_cs, (long long)b_rs, (long long)b_cs);
+  if (!g_rt.blas) {
+    if (rocblas_create_handle(&g_rt.blas) != rocblas_status_success)
+      return fail(DEERS_ROCM_ERR_HIP, "rocblas_create_handle failed");
+    if (rocblas_set_stream(g_rt.blas, g_rt.stream) != rocblas_status_success)
+      return fail(DEERS_ROCM_ERR_HIP, "rocblas_set_stream failed");
+  }
+  // Row-major C = A B is column-major C^T = B^T A^T: the BLAS sees B first.  A
+  // row-major [rows x cols] matrix with unit column stride is, read column-major, its
+  // own transpose with leading dimension = row stride.
+  const rocblas_datatype ty = dtype == DEERS_ROCM_F16 ? rocblas_datatype_f16_r : rocblas_datatype_f32_r;
+  const float alpha = 1.f, beta = 0.f;
+  const rocblas_status st = rocblas_gemm_strided_batched_ex(
+      g_rt.blas, b_t ? rocblas_operation_transpose : rocblas_operation_none,
+      a_t ? rocblas_operation_transpose : rocblas_operation_none, (rocblas_int)n, (rocblas_int)m,
+      (rocblas_int)k, &alpha, b, ty, (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c,
+      ty, (rocblas_int)n, m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch,
+      rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+  if (st != rocblas_status_success)
+    return fail(DEERS_ROCM_ERR_HIP, "rocblas_gemm_strided_batched_ex failed: %s",
+                rocblas_status_to_string(st));
   return DEERS_ROCM_OK;
 }
 

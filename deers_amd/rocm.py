@@ -207,6 +207,15 @@ def copy_compact_raw(dtype, src, shape, strides, dst):
                                           ctypes.c_int(nd), dst))
 
 
+def matmul_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
+    """deers_rocm_matmul: c[batch,m,n] = a @ b; strides are (row, col, batch) in elements."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_matmul(
+        ctypes.c_int(dtype_code(dtype)), a, i64(a_strides[0]), i64(a_strides[1]), i64(a_strides[2]),
+        b, i64(b_strides[0]), i64(b_strides[1]), i64(b_strides[2]), c, i64(batch), i64(m), i64(n),
+        i64(k)))
+
+
 def rope_fwd_raw(dtype, x, cos, sin, y, B, T, H, D, x_strides=None):
     """deers_rocm_rope_fwd: x logical [B,T,H,D] -> y compact [B,H,T,D]."""
     _check(load().deers_rocm_rope_fwd(

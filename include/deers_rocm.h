@@ -192,6 +192,22 @@ int deers_rocm_neg(int dtype, const void* a, void* out, size_t n);
 int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
                             const int64_t* strides, int ndim, void* dst);
 
+/* ---- batched matrix product ---------------------------------------------------
+ * c[batch,m,n] (compact, row-major) = a[batch,m,k] @ b[batch,k,n].  Replaces
+ * BackendStorage::matmul (src/storage.rs:270-279; CPU src/storage/cpu.rs:688-753,
+ * CUDA src/storage/cuda.rs:1100-1125, which calls cuBLAS: this one calls rocBLAS, a
+ * plain library GEMM, f16 with f32 accumulation or f32).  Operands are described by
+ * element strides (row, column, batch) the way the CPU backend passes Layout strides
+ * to gemm: transposed views cost nothing, a batch stride of 0 broadcasts (weights).
+ * Each operand needs a unit row or column stride, otherwise DEERS_ROCM_ERR_LAYOUT
+ * and the caller compacts (MatMul::new does that for the Metal backend,
+ * src/ops.rs:1058-1062).  Used by the projections around the attention core
+ * (src/models/gpt.rs:101-133, 146-147). */
+int deers_rocm_matmul(int dtype,
+                      const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
+                      const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
+                      void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
+
 /* ---- rotary embedding fused with the head split / merge -----------------------
  * The neighbours of the attention core in CausalSelfAttention::forward
  * (src/models/gpt.rs:115-137): apply_rotary_emb on the [B,T,H,D] projections

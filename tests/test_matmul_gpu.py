@@ -1,0 +1,86 @@
+"""deers_rocm_matmul (library GEMM behind BackendStorage::matmul) against the CPU oracle's
+gemm_strided restatement and the reference's own integer-valued conformance cases
+(tests/tensor.rs:83-110)."""
+import numpy as np
+import pytest
+
+import oracle
+from deers_amd import rocm
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    if not rocm.available():
+        pytest.skip("no gfx950 device")
+    rocm.init(0)
+
+
+def _run(a, b, dtype, a_view=None, b_view=None):
+    """a [batch,m,k], b [batch,k,n] numpy; *_view = (buffer array, (rs, cs, bs))."""
+    batch, m, k = a.shape
+    n = b.shape[2]
+    abuf, astr = a_view if a_view else (np.ascontiguousarray(a), (k, 1, m * k))
+    bbuf, bstr = b_view if b_view else (np.ascontiguousarray(b), (n, 1, k * n))
+    da, db = rocm.DeviceBuffer.from_numpy(abuf.astype(dtype)), rocm.DeviceBuffer.from_numpy(bbuf.astype(dtype))
+    dc = rocm.DeviceBuffer((batch, m, n), dtype)
+    rocm.matmul_raw(dtype, da.ptr, astr, db.ptr, bstr, dc.ptr, batch, m, n, k)
+    return dc.numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_matmul_reference_integer_cases(dtype):
+    a = np.array([[[1, 2, 3], [4, 5, 6]]], np.float32)
+    b = np.array([[[7, 8], [9, 10], [11, 12]]], np.float32)
+    assert np.array_equal(_run(a, b, dtype)[0], np.array([[58, 64], [139, 154]], dtype))
+    # batched 2x2x3 @ 2x3x2
+    a2 = np.arange(12, dtype=np.float32).reshape(2, 2, 3)
+    b2 = np.arange(12, dtype=np.float32).reshape(2, 3, 2)
+    assert np.array_equal(_run(a2, b2, dtype), np.einsum("bmk,bkn->bmn", a2, b2).astype(dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float16, 2e-2), (np.float32, 1e-4)])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 1, 1, 1), (3, 5, 7, 9), (2, 130, 33, 64), (1, 1024, 768, 768)])
+def test_matmul_matches_oracle(dtype, tol, batch, m, n, k):
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal((batch, m, k)).astype(dtype)
+    b = (rng.standard_normal((batch, k, n)) / np.sqrt(k)).astype(dtype)
+    want = oracle.matmul(a.astype(np.float32), b.astype(np.float32))
+    got = _run(a, b, dtype).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float16, 2e-2), (np.float32, 1e-4)])
+def test_matmul_transposed_views_and_broadcast_weights(dtype, tol):
+    rng = np.random.default_rng(32)
+    batch, m, n, k = 4, 17, 24, 40
+    a = rng.standard_normal((batch, m, k)).astype(dtype)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(dtype)
+    want = np.einsum("bmk,kn->bmn", a.astype(np.float32), w.astype(np.float32))
+    # b is one [k,n] weight for every batch entry: batch stride 0
+    got = _run(a, np.broadcast_to(w, (batch, k, n)), dtype, b_view=(w, (n, 1, 0)))
+    assert np.max(np.abs(got.astype(np.float64) - want)) <= tol
+    # a given as the transposed view of an [batch,k,m] buffer (dB = A^T @ dC in MatMul::backward)
+    at = np.ascontiguousarray(a.transpose(0, 2, 1))
+    got_t = _run(a, np.broadcast_to(w, (batch, k, n)), dtype, a_view=(at, (1, m, k * m)),
+                 b_view=(w, (n, 1, 0)))
+    assert np.array_equal(got_t, got)
+    # b given as the transposed view of an [n,k] buffer (dA = dC @ B^T)
+    wt = np.ascontiguousarray(w.T)
+    got_bt = _run(a, np.broadcast_to(w, (batch, k, n)), dtype, b_view=(wt, (1, k, 0)))
+    assert np.max(np.abs(got_bt.astype(np.float64) - want)) <= tol
+
+
+@pytest.mark.gpu
+def test_matmul_edge_cases_and_errors():
+    buf = rocm.DeviceBuffer((64,), np.float32, zeros=True)
+    out = rocm.DeviceBuffer.from_numpy(np.ones((2, 3), np.float32))
+    rocm.matmul_raw(np.float32, buf.ptr, (0, 1, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 2, 3, 0)  # k = 0
+    assert np.array_equal(out.numpy(), np.zeros((2, 3), np.float32))
+    rocm.matmul_raw(np.float32, buf.ptr, (4, 1, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 0, 3, 4)  # m = 0: no-op
+    with pytest.raises(rocm.RocmError):  # neither stride of a is 1
+        rocm.matmul_raw(np.float32, buf.ptr, (8, 2, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 2, 3, 4)
+    with pytest.raises(rocm.RocmError):
+        rocm.matmul_raw(np.float32, None, (4, 1, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 2, 3, 4)
