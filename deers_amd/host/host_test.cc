@@ -2,6 +2,8 @@
 //   host_test graph            graph / layout logic on unbacked tensors (no GPU)
 //   host_test gpu <dir>        runs the fused op on the inputs in <dir> (written by
 //                              the Python tests) and writes its outputs there
+//   host_test module <dir>     the whole attention module (projections, RoPE, core,
+//                              head merge, output projection), forward and backward
 // The graph cases restate the reference's own autograd tests
 // (src/backprop.rs:142-201): linear chain, diamond, no-grad skip, accumulation = 2.
 #include <cstdio>
@@ -245,6 +247,55 @@ static int run_gpu(const std::string& dir) {
   return 0;
 }
 
+// The whole attention module (src/models/gpt.rs:101-147) forward and backward.
+static int run_module(const std::string& dir) {
+  check(deers_rocm_init(0));
+  int dt, B, T, C, H;
+  {
+    std::ifstream f(dir + "/module.txt");  // dtype B T C H
+    if (!(f >> dt >> B >> T >> C >> H)) { std::printf("FAIL bad module.txt\n"); return 2; }
+  }
+  const DType dtype = dt == 0 ? DType::F16 : DType::F32;
+  auto load = [&](const char* name, const std::vector<int64_t>& shape) {
+    auto bytes = read_file(dir + "/" + name);
+    Layout l(shape);
+    if (bytes.size() != l.size() * size_in_bytes(dtype)) { std::printf("FAIL size of %s\n", name); std::exit(2); }
+    return Tensor::from_host(bytes.data(), shape, dtype);
+  };
+  Tensor x = load("x.bin", {B, T, C}).attach();
+  Tensor wq = load("wq.bin", {C, C}).attach(), wk = load("wk.bin", {C, C}).attach();
+  Tensor wv = load("wv.bin", {C, C}).attach(), wo = load("wo.bin", {C, C}).attach();
+  Tensor seed = load("dy.bin", {B, T, C});
+  CausalSelfAttention attn(C, H, wq, wk, wv, wo);
+  auto [cos, sin] = precompute_rotary_embeddings(T, C / H, 10000.0f, dtype);
+  Tensor y = attn.forward(x, cos, sin);
+  EXPECT((y.shape() == std::vector<int64_t>{B, T, C}));
+  dump(y, dir + "/y.bin");
+  GradientStore grads = y.backward_from(seed);
+  for (auto [t, name] : {std::pair<const Tensor*, const char*>{&x, "dx.bin"}, {&wq, "dwq.bin"}, {&wk, "dwk.bin"},
+                         {&wv, "dwv.bin"}, {&wo, "dwo.bin"}}) {
+    const Tensor* g = grads.get(t->id());
+    EXPECT(g != nullptr);
+    if (g) {
+      EXPECT(g->shape() == t->shape());
+      dump(*g, dir + "/" + name);
+    }
+  }
+  // op names along the graph, output first: the fused ops are really in it
+  bool saw_attn = false, saw_rope = false, saw_matmul = false;
+  for (const Tensor* n : y.sorted_nodes())
+    if (n->op()) {
+      const std::string nm = n->op()->name();
+      saw_attn |= nm == "FusedCausalAttention";
+      saw_rope |= nm == "RotaryHeads";
+      saw_matmul |= nm == "MatMul";
+    }
+  EXPECT(saw_attn && saw_rope && saw_matmul);
+  check(deers_rocm_sync());
+  std::printf("ok module\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "graph";
   try {
@@ -256,8 +307,10 @@ int main(int argc, char** argv) {
       test_graph_of_attention_views();
     } else if (mode == "gpu" && argc > 2) {
       if (int rc = run_gpu(argv[2])) return rc;
+    } else if (mode == "module" && argc > 2) {
+      if (int rc = run_module(argv[2])) return rc;
     } else {
-      std::printf("usage: host_test graph | gpu <dir>\n");
+      std::printf("usage: host_test graph | gpu <dir> | module <dir>\n");
       return 2;
     }
   } catch (const std::exception& e) {

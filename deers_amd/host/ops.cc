@@ -109,7 +109,96 @@ void Compact::backward(GradientStore& grads, const Tensor& out_grad) const {
   grads.accumulate(arg_, out_grad);
 }
 
+// ---- Reshape ----
+Reshape::Reshape(Tensor arg, std::vector<int64_t> new_shape)
+    : arg_(arg.compact()), new_shape_(std::move(new_shape)) {
+  if (arg_.layout().size() != Layout(new_shape_).size())
+    throw std::logic_error("reshape: size " + std::to_string(arg_.layout().size()) +
+                           " cannot be reshaped to size " + std::to_string(Layout(new_shape_).size()));
+}
+Tensor Reshape::forward(std::unique_ptr<Reshape> self) {
+  auto storage = self->arg_.storage();
+  Layout layout(self->new_shape_);
+  return Tensor(std::move(storage), std::move(layout), false, std::move(self));
+}
+void Reshape::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(arg_, out_grad.reshape(arg_.shape()));
+}
+
+// ---- MatMul ----
+MatMul::MatMul(Tensor a, Tensor b) : a_(std::move(a)), b_(std::move(b)) {
+  const size_t nd = a_.layout().ndim();
+  if (nd < 2 || b_.layout().ndim() < 2)
+    throw std::logic_error("matmul requires ndim >= 2");
+  if (nd != b_.layout().ndim()) throw std::logic_error("matmul requires same number of dimensions");
+  if (a_.shape()[nd - 1] != b_.shape()[nd - 2]) throw std::logic_error("matmul inner dimensions must match");
+  for (size_t i = 0; i + 2 < nd; ++i)
+    if (a_.shape()[i] != b_.shape()[i]) throw std::logic_error("matmul batch dimension mismatch");
+  if (a_.dtype() != b_.dtype()) throw std::logic_error("matmul: dtypes differ");
+}
+
+namespace {
+// Describes the last two axes and the (collapsed) batch axes of `t` for the library:
+// returns false when the batch axes cannot be expressed by one stride or no matrix
+// stride is 1, in which case the caller compacts.
+bool gemm_view(const Tensor& t, int64_t* rs, int64_t* cs, int64_t* bs) {
+  const Layout& l = t.layout();
+  const size_t nd = l.ndim();
+  *rs = l.strides[nd - 2];
+  *cs = l.strides[nd - 1];
+  const int64_t rows = l.shape[nd - 2], cols = l.shape[nd - 1];
+  if (!((*cs == 1 && *rs >= cols) || (*rs == 1 && *cs >= rows) || rows == 1 || cols == 1)) return false;
+  // batch axes must walk memory like one axis: stride[i] == stride[i+1] * shape[i+1]
+  *bs = 0;
+  int64_t expect = -1;
+  for (int i = (int)nd - 3; i >= 0; --i) {
+    if (l.shape[i] == 1) continue;
+    if (expect >= 0 && l.strides[i] != expect) return false;
+    if (expect < 0) *bs = l.strides[i];
+    expect = l.strides[i] * l.shape[i];
+  }
+  return *bs >= 0;
+}
+}  // namespace
+
+Tensor MatMul::forward(std::unique_ptr<MatMul> self) {
+  Tensor a = self->a_, b = self->b_;
+  int64_t ars, acs, abs_, brs, bcs, bbs;
+  if (!gemm_view(a, &ars, &acs, &abs_)) { a = a.detach().compact(); gemm_view(a, &ars, &acs, &abs_); }
+  if (!gemm_view(b, &brs, &bcs, &bbs)) { b = b.detach().compact(); gemm_view(b, &brs, &bcs, &bbs); }
+  const size_t nd = a.layout().ndim();
+  const int64_t m = a.shape()[nd - 2], k = a.shape()[nd - 1], n = b.shape()[nd - 1];
+  std::vector<int64_t> out_shape(a.shape().begin(), a.shape().end() - 2);
+  int64_t batch = 1;
+  for (int64_t d : out_shape) batch *= d;
+  out_shape.push_back(m);
+  out_shape.push_back(n);
+  Tensor out = empty(out_shape, a.dtype(), backed(a));
+  if (backed(a))
+    check(deers_rocm_matmul((int)a.dtype(), a.data(), ars, acs, abs_, b.data(), brs, bcs, bbs,
+                            out.data(), batch, m, n, k));
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+
+void MatMul::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(a_, out_grad.matmul(b_.transpose()));
+  grads.accumulate(b_, a_.transpose().matmul(out_grad));
+}
+
 // ---- Tensor conveniences that build ops ----
+Tensor Tensor::transpose() const {
+  const size_t nd = layout().ndim();
+  std::vector<size_t> dims(nd);
+  for (size_t i = 0; i < nd; ++i) dims[i] = i;
+  std::swap(dims[nd - 1], dims[nd - 2]);
+  return permute(dims);
+}
+Tensor Tensor::reshape(const std::vector<int64_t>& shape) const {
+  return Reshape::forward(std::make_unique<Reshape>(*this, shape));
+}
+Tensor Tensor::matmul(const Tensor& other) const {
+  return MatMul::forward(std::make_unique<MatMul>(*this, other));
+}
 Tensor Tensor::permute(const std::vector<size_t>& dims) const {
   return Permute::forward(std::make_unique<Permute>(*this, dims));
 }
@@ -231,6 +320,33 @@ Tensor rotary_heads(const Tensor& x, const Tensor& cos, const Tensor& sin) {
 Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v) {
   const double scale = 1.0 / std::sqrt((double)q.shape().at(3));
   return FusedCausalAttention::forward(std::make_unique<FusedCausalAttention>(q, k, v, scale));
+}
+
+// ---- CausalSelfAttention module ----
+CausalSelfAttention::CausalSelfAttention(int64_t n_embd, int64_t n_head, Tensor wq, Tensor wk,
+                                         Tensor wv, Tensor wo)
+    : n_head_(n_head), head_dim_(n_embd / n_head), wq_(std::move(wq)), wk_(std::move(wk)),
+      wv_(std::move(wv)), wo_(std::move(wo)) {
+  if (n_embd % n_head) throw std::logic_error("n_embd must be divisible by n_head");
+  for (const Tensor* w : {&wq_, &wk_, &wv_, &wo_})
+    if (w->shape() != std::vector<int64_t>{n_embd, n_embd})
+      throw std::logic_error("projection weights must be [n_embd, n_embd]");
+}
+
+Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const {
+  if (x.layout().ndim() != 3) throw std::logic_error("attention expects input shape [B, T, C]");
+  const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
+  if (C != n_head_ * head_dim_) throw std::logic_error("input channel size must match attention width");
+  const Tensor x_flat = x.reshape({B * T, C});
+  const std::vector<int64_t> bthd{B, T, n_head_, head_dim_};
+  const Tensor q = x_flat.matmul(wq_).reshape(bthd);  // [B,T,H,D]
+  const Tensor k = x_flat.matmul(wk_).reshape(bthd);
+  const Tensor v = x_flat.matmul(wv_).reshape(bthd);
+  const Tensor qh = rotary_heads(q, cos, sin);         // [B,H,T,D], compact
+  const Tensor kh = rotary_heads(k, cos, sin);
+  const Tensor vh = v.permute({0, 2, 1, 3});           // a view; the kernels read it by stride
+  const Tensor y = causal_self_attention(qh, kh, vh).permute({0, 2, 1, 3}).reshape({B * T, C});
+  return y.matmul(wo_).reshape({B, T, C});
 }
 
 Tensor attention_decode(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache) {

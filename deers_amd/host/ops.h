@@ -61,6 +61,36 @@ class Compact : public TensorOp {
   Tensor arg_;
 };
 
+// Same storage under a new compact shape; the argument is compacted first, which is
+// where the reference's head merge copy happens (src/ops.rs:899-934).
+class Reshape : public TensorOp {
+ public:
+  Reshape(Tensor arg, std::vector<int64_t> new_shape);
+  static Tensor forward(std::unique_ptr<Reshape> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "Reshape"; }
+
+ private:
+  Tensor arg_;
+  std::vector<int64_t> new_shape_;
+};
+
+// Batched a[..,m,k] @ b[..,k,n] with equal batch dimensions (src/ops.rs:1012-1106);
+// operands go to the library by stride, so the transposed views of the backward
+// (dA = dC @ B^T, dB = A^T @ dC) cost no copy.
+class MatMul : public TensorOp {
+ public:
+  MatMul(Tensor a, Tensor b);
+  static Tensor forward(std::unique_ptr<MatMul> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&a_, &b_}; }
+  const char* name() const override { return "MatMul"; }
+
+ private:
+  Tensor a_, b_;
+};
+
 // y = softmax(q k^T * scale + causal mask) v for q, k, v logical [B,H,T,D] (views
 // welcome: any strides with a unit D stride go to the kernels as they are, other
 // views are compacted first, as FusedLogSoftmax::forward compacts its argument,
@@ -106,6 +136,21 @@ Tensor rotary_heads(const Tensor& x, const Tensor& cos, const Tensor& sin);
 // The call site of src/models/gpt.rs:139-144: scale = 1/sqrt(head_dim) computed in
 // f64 and narrowed to f32 (src/storage.rs:115-117).
 Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
+
+// The attention module of src/models/gpt.rs:76-148 on the ROCm device: bias-free
+// q/k/v/out projections with weights [in, out] (y = x @ W, src/nn.rs:183-190), RoPE on
+// queries and keys, the fused causal attention core, head merge, output projection.
+class CausalSelfAttention {
+ public:
+  CausalSelfAttention(int64_t n_embd, int64_t n_head, Tensor wq, Tensor wk, Tensor wv, Tensor wo);
+  // x [B,T,C] with the RoPE tables of precompute_rotary_embeddings -> [B,T,C]
+  Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
+  std::vector<Tensor> parameters() const { return {wq_, wk_, wv_, wo_}; }
+
+ private:
+  int64_t n_head_, head_dim_;
+  Tensor wq_, wk_, wv_, wo_;
+};
 
 // One query token per (b,h) against a KV cache: q [B,H,D], caches [B,H,L,D] compact;
 // not differentiable (inference only).

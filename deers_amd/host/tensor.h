@@ -127,6 +127,9 @@ class Tensor {
   // Differentiable views and copies (src/ops.rs:687-727, 1254-1287).
   Tensor permute(const std::vector<size_t>& dims) const;
   Tensor compact() const;  // returns *this when already compact
+  Tensor transpose() const;  // swaps the last two axes (a Permute)
+  Tensor reshape(const std::vector<int64_t>& shape) const;  // compacts first (src/ops.rs:913)
+  Tensor matmul(const Tensor& other) const;
   // Differentiable element-wise ops used by the contract tests.
   Tensor neg() const;
   Tensor add(const Tensor& other) const;

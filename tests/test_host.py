@@ -87,3 +87,55 @@ def test_host_fused_attention_matches_oracle(tmp_path, dtype, B, H, T, D, L, tol
         ref = oracle.attn_fwd(d["q"].astype(np.float32), d["k"].astype(np.float32),
                               d["v"].astype(np.float32))[:, :, 0]
         assert float(np.max(np.abs(got - ref))) <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,B,T,C,H,tol", [
+    (np.float32, 2, 70, 128, 4, 2e-4),
+    (np.float16, 2, 200, 256, 4, 2e-2),
+])
+def test_host_attention_module_matches_composed_oracle(tmp_path, dtype, B, T, C, H, tol):
+    """x -> q/k/v projections -> RoPE -> causal attention -> head merge -> out projection
+    (src/models/gpt.rs:101-147) and its backward, against the same chain on the CPU oracle.
+    f16 tolerance: four GEMMs with f16 outputs around the core (the reference's own f16
+    helper uses 1e-2, tests/utils.rs:14; gradients of the weights sum over B*T rows)."""
+    import oracle
+    rng = np.random.default_rng(41)
+    D = C // H
+    x = rng.standard_normal((B, T, C)).astype(dtype)
+    ws = [(rng.standard_normal((C, C)) / np.sqrt(C)).astype(dtype) for _ in range(4)]
+    dy = rng.standard_normal((B, T, C)).astype(dtype)
+    for name, a in zip(("x", "wq", "wk", "wv", "wo", "dy"), (x, *ws, dy)):
+        a.tofile(tmp_path / f"{name}.bin")
+    (tmp_path / "module.txt").write_text(f"{0 if dtype == np.float16 else 1} {B} {T} {C} {H}\n")
+    r = _run("module", str(tmp_path))
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ok module" in r.stdout and "all passed" in r.stdout
+
+    f = lambda a: a.astype(np.float32)
+    xf, (wq, wk, wv, wo), dyf = f(x).reshape(B * T, C), [f(w) for w in ws], f(dy).reshape(B * T, C)
+    mm = lambda a, b: oracle.matmul(a[None], b[None])[0]
+    rnd = (lambda a: a.astype(np.float16).astype(np.float32)) if dtype == np.float16 else (lambda a: a)
+    cos, sin = oracle.rope_tables(T, D, dtype=dtype)
+    c32, s32 = f(cos), f(sin)
+    hd = lambda a: np.ascontiguousarray(a.transpose(0, 2, 1, 3))
+    q, k, v = (rnd(mm(xf, w)).reshape(B, T, H, D) for w in (wq, wk, wv))
+    qh, kh, vh = hd(rnd(oracle.rope_apply(q, c32, s32))), hd(rnd(oracle.rope_apply(k, c32, s32))), hd(v)
+    o = rnd(oracle.attn_fwd(qh, kh, vh))
+    o_flat = hd(o).reshape(B * T, C)
+    want_y = mm(o_flat, wo)
+    # backward by hand, in the order the reverse sweep runs it
+    d_o_flat = rnd(mm(dyf, wo.T))
+    want_dwo = mm(o_flat.T, dyf)
+    gq, gk, gv = (rnd(g) for g in oracle.attn_bwd(qh, kh, vh, hd(d_o_flat.reshape(B, T, H, D))))
+    dq = rnd(oracle.rope_apply_bwd(hd(gq), c32, s32)).reshape(B * T, C)
+    dk = rnd(oracle.rope_apply_bwd(hd(gk), c32, s32)).reshape(B * T, C)
+    dv = hd(gv).reshape(B * T, C)
+    want = {"dwq": mm(xf.T, dq), "dwk": mm(xf.T, dk), "dwv": mm(xf.T, dv), "dwo": want_dwo,
+            "dx": mm(dq, wq.T) + mm(dk, wk.T) + mm(dv, wv.T)}
+    got = lambda name, shape: np.fromfile(tmp_path / f"{name}.bin", dtype=dtype).reshape(shape).astype(np.float64)
+    assert np.max(np.abs(got("y", (B * T, C)) - want_y)) <= tol
+    for name, ref in want.items():
+        g = got(name, ref.shape)
+        scale = max(1.0, float(np.max(np.abs(ref))))
+        assert np.max(np.abs(g - ref)) <= tol * scale, name
