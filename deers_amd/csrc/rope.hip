@@ -68,17 +68,19 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
 
 }  // namespace
 
-// x: logical [B,T,H,D] with element strides xs = {b,t,h} (D stride 1); y: compact
-// [B,H,T,D].  inverse: dy [B,H,T,D] with strides {b,h,t} -> dx compact [B,T,H,D].
+// x: logical [B,T,H,D] with element strides xs = {b,t,h} (D stride 1); y: [B,H,T,D],
+// compact or with element strides {b,h,t} (a row range of a KV cache).
+// inverse: dy [B,H,T,D] with strides {b,h,t} -> dx compact [B,T,H,D].
 void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
-                 const void* cos, const void* sin, void* dst, int B, int T, int H, int D,
-                 hipStream_t stream) {
+                 const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
+                 int T, int H, int D, hipStream_t stream) {
   RopeParams p{};
   p.src = src; p.dst = dst; p.cos = cos; p.sin = sin;
   p.B = B; p.T = T; p.H = H; p.D = D;
   if (!inverse) {
     p.s_b = src_strides[0]; p.s_t = src_strides[1]; p.s_h = src_strides[2];
     p.d_b = (int64_t)H * T * D; p.d_h = (int64_t)T * D; p.d_t = D;
+    if (dst_strides) { p.d_b = dst_strides[0]; p.d_h = dst_strides[1]; p.d_t = dst_strides[2]; }
   } else {
     p.s_b = src_strides[0]; p.s_h = src_strides[1]; p.s_t = src_strides[2];
     p.d_b = (int64_t)T * H * D; p.d_t = (int64_t)H * D; p.d_h = D;

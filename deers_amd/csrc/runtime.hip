@@ -32,8 +32,11 @@ void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t s
 void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
                          const int64_t* strides, int ndim, void* dst, hipStream_t stream);
 void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
-                 const void* cos, const void* sin, void* dst, int B, int T, int H, int D,
-                 hipStream_t stream);
+                 const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
+                 int T, int H, int D, hipStream_t stream);
+void launch_copy_view(int dtype_f16, const void* src, const int64_t* src_strides, void* dst,
+                      const int64_t* dst_strides, const int64_t* shape, int ndim,
+                      hipStream_t stream);
 }  // namespace deers
 
 namespace {
@@ -555,6 +558,23 @@ int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
   return DEERS_ROCM_OK;
 }
 
+int deers_rocm_copy_view(int dtype, const void* src, const int64_t* src_strides, void* dst,
+                         const int64_t* dst_strides, const int64_t* shape, int ndim) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (ndim < 1 || ndim > 6) return fail(DEERS_ROCM_ERR_ARG, "copy_view: ndim %d not in 1..6", ndim);
+  if (!src || !dst || !shape || !src_strides || !dst_strides)
+    return fail(DEERS_ROCM_ERR_ARG, "copy_view: null pointer");
+  for (int d = 0; d < ndim; ++d)
+    if (shape[d] < 0 || src_strides[d] < 0 || dst_strides[d] < 0)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "copy_view: negative extent or stride in dim %d", d);
+  deers::launch_copy_view(dtype == DEERS_ROCM_F16, src, src_strides, dst, dst_strides, shape, ndim,
+                          g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
 // ---- batched matrix product (library GEMM) ----
 
 int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
@@ -646,14 +666,24 @@ static int rope_common(const char* what, int dtype, const void* src, const int64
 }
 
 int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides, const void* cos,
-                        const void* sin, void* y, int64_t B, int64_t T, int64_t H, int64_t D) {
+                        const void* sin, void* y, const int64_t* y_strides, int64_t B, int64_t T,
+                        int64_t H, int64_t D) {
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   int64_t st[3];
   if (int rc = rope_common("rope_fwd", dtype, x, x_strides, cos, sin, y, B, T, H, D, st, false))
     return rc;
-  deers::launch_rope(dtype == DEERS_ROCM_F16, false, x, st, cos, sin, y, (int)B, (int)T, (int)H,
-                     (int)D, g_rt.stream);
+  if (y_strides) {
+    const int64_t per16 = dtype == DEERS_ROCM_F16 ? 8 : 4;
+    if (y_strides[3] != 1)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "rope_fwd: innermost output stride must be 1");
+    for (int d = 0; d < 3; ++d)
+      if (y_strides[d] < 0 || y_strides[d] % per16)
+        return fail(DEERS_ROCM_ERR_LAYOUT,
+                    "rope_fwd: output strides must be non-negative multiples of 16 bytes");
+  }
+  deers::launch_rope(dtype == DEERS_ROCM_F16, false, x, st, cos, sin, y, y_strides, (int)B, (int)T,
+                     (int)H, (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }
@@ -665,8 +695,8 @@ int deers_rocm_rope_bwd(int dtype, const void* dy, const int64_t* dy_strides, co
   int64_t st[3];
   if (int rc = rope_common("rope_bwd", dtype, dy, dy_strides, cos, sin, dx, B, T, H, D, st, true))
     return rc;
-  deers::launch_rope(dtype == DEERS_ROCM_F16, true, dy, st, cos, sin, dx, (int)B, (int)T, (int)H,
-                     (int)D, g_rt.stream);
+  deers::launch_rope(dtype == DEERS_ROCM_F16, true, dy, st, cos, sin, dx, nullptr, (int)B, (int)T,
+                     (int)H, (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -110,6 +110,46 @@ void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t s
                        (const float*)a, (float*)out, n);
 }
 
+// dst viewed through dst_strides <- src viewed through src_strides, same shape
+// (element-wise; used for small scatters such as a KV-cache append).
+template <typename T>
+__global__ __launch_bounds__(256) void copy_view_kernel(const T* src, T* dst, View6 v, View6 w,
+                                                        size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    size_t rem = i;
+    int64_t so = 0, dof = 0;
+#pragma unroll
+    for (int d = 5; d >= 0; --d) {
+      const size_t idx = rem % (size_t)v.shape[d];
+      rem /= (size_t)v.shape[d];
+      so += (int64_t)idx * v.stride[d];
+      dof += (int64_t)idx * w.stride[d];
+    }
+    dst[dof] = src[so];
+  }
+}
+
+void launch_copy_view(int dtype_f16, const void* src, const int64_t* src_strides, void* dst,
+                      const int64_t* dst_strides, const int64_t* shape, int ndim,
+                      hipStream_t stream) {
+  View6 v, w;
+  size_t n = 1;
+  for (int d = 0; d < 6; ++d) {
+    const int s = d - (6 - ndim);
+    v.shape[d] = w.shape[d] = s >= 0 ? shape[s] : 1;
+    v.stride[d] = s >= 0 ? src_strides[s] : 0;
+    w.stride[d] = s >= 0 ? dst_strides[s] : 0;
+    n *= (size_t)v.shape[d];
+  }
+  if (n == 0) return;
+  if (dtype_f16)
+    hipLaunchKernelGGL(copy_view_kernel<half_t>, dim3(grid_for(n)), dim3(256), 0, stream,
+                       (const half_t*)src, (half_t*)dst, v, w, n);
+  else
+    hipLaunchKernelGGL(copy_view_kernel<float>, dim3(grid_for(n)), dim3(256), 0, stream,
+                       (const float*)src, (float*)dst, v, w, n);
+}
+
 void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
                          const int64_t* strides, int ndim, void* dst, hipStream_t stream) {
   View6 v;

@@ -281,6 +281,25 @@ static int run_module(const std::string& dir) {
       dump(*g, dir + "/" + name);
     }
   }
+  // generation with a KV cache, teacher-forced with the same inputs: step t must give
+  // row t of the full causal forward (f16 only: the decode kernel is f16)
+  if (dtype == DType::F16 && (C / H == 64 || C / H == 128)) {
+    std::vector<char> xh((size_t)B * T * C * 2), step((size_t)B * C * 2), ys((size_t)B * T * C * 2);
+    x.to_host(xh.data());
+    KvCache cache = KvCache::create(B, H, T + 7, C / H, dtype);  // spare capacity on purpose
+    for (int t = 0; t < T; ++t) {
+      for (int b = 0; b < B; ++b)
+        std::memcpy(&step[(size_t)b * C * 2], &xh[((size_t)b * T + t) * C * 2], (size_t)C * 2);
+      Tensor xt = Tensor::from_host(step.data(), {B, 1, C}, dtype);
+      Tensor yt = attn.decode_step(xt, cache, cos, sin);
+      EXPECT(!yt.requires_grad());
+      yt.to_host(step.data());
+      for (int b = 0; b < B; ++b)
+        std::memcpy(&ys[((size_t)b * T + t) * C * 2], &step[(size_t)b * C * 2], (size_t)C * 2);
+    }
+    EXPECT(cache.len == T);
+    write_file(dir + "/y_decode.bin", ys.data(), ys.size());
+  }
   // op names along the graph, output first: the fused ops are really in it
   bool saw_attn = false, saw_rope = false, saw_matmul = false;
   for (const Tensor* n : y.sorted_nodes())

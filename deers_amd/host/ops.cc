@@ -274,7 +274,7 @@ Tensor RotaryHeads::forward(std::unique_ptr<RotaryHeads> self) {
   const int64_t B = x.shape()[0], T = x.shape()[1], H = x.shape()[2], D = x.shape()[3];
   Tensor y = empty({B, H, T, D}, x.dtype(), true);
   check(deers_rocm_rope_fwd((int)x.dtype(), x.data(), x.layout().strides.data(), cos.data(),
-                            sin.data(), y.data(), B, T, H, D));
+                            sin.data(), y.data(), nullptr, B, T, H, D));
   return Tensor(y.storage(), y.layout(), false, std::move(self));
 }
 
@@ -347,6 +347,48 @@ Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Te
   const Tensor vh = v.permute({0, 2, 1, 3});           // a view; the kernels read it by stride
   const Tensor y = causal_self_attention(qh, kh, vh).permute({0, 2, 1, 3}).reshape({B * T, C});
   return y.matmul(wo_).reshape({B, T, C});
+}
+
+KvCache KvCache::create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType dtype) {
+  KvCache c;
+  c.k = Tensor::zeros({B, H, capacity, D}, dtype);
+  c.v = Tensor::zeros({B, H, capacity, D}, dtype);
+  c.capacity = capacity;
+  return c;
+}
+
+Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos,
+                                        const Tensor& sin) const {
+  NoGradGuard no_grad;
+  if (x_t.layout().ndim() != 3 || x_t.shape()[1] != 1)
+    throw std::logic_error("decode_step expects input shape [B, 1, C]");
+  if (cache.len >= cache.capacity) throw std::logic_error("decode_step: KV cache is full");
+  const int64_t B = x_t.shape()[0], C = x_t.shape()[2], H = n_head_, D = head_dim_;
+  const int64_t pos = cache.len, cap = cache.capacity;
+  if (pos >= cos.shape()[1]) throw std::logic_error("decode_step: position beyond the RoPE tables");
+  const int dt = (int)x_t.dtype();
+  const size_t el = size_in_bytes(x_t.dtype());
+  const Tensor x_flat = x_t.reshape({B, C});
+  const Tensor q = x_flat.matmul(wq_), k = x_flat.matmul(wk_), v = x_flat.matmul(wv_);  // [B, H*D]
+  // row `pos` of the compact [1,T,1,D/2] tables
+  const Tensor cc = cos.compact(), sc = sin.compact();
+  const char* cos_t = (const char*)cc.data() + pos * (D / 2) * el;
+  const char* sin_t = (const char*)sc.data() + pos * (D / 2) * el;
+  const int64_t x_strides[4] = {H * D, H * D, D, 1};                 // [B,1,H,D] over [B, H*D]
+  const int64_t cache_strides[4] = {H * cap * D, cap * D, D, 1};     // [B,H,1,D] at one cache row
+  Tensor qh = empty({B, H, D}, x_t.dtype(), true);
+  check(deers_rocm_rope_fwd(dt, q.data(), x_strides, cos_t, sin_t, qh.data(), nullptr, B, 1, H, D));
+  check(deers_rocm_rope_fwd(dt, k.data(), x_strides, cos_t, sin_t,
+                            (char*)cache.k.data() + pos * D * el, cache_strides, B, 1, H, D));
+  const int64_t shape[3] = {B, H, D}, v_src[3] = {H * D, D, 1}, v_dst[3] = {H * cap * D, cap * D, 1};
+  check(deers_rocm_copy_view(dt, v.data(), v_src, (char*)cache.v.data() + pos * D * el, v_dst, shape, 3));
+  cache.len = pos + 1;
+  Tensor o = empty({B, H * D}, x_t.dtype(), true);
+  const int64_t kv_strides[3] = {H * cap * D, cap * D, D};
+  const double scale = 1.0 / std::sqrt((double)D);
+  check(deers_rocm_attn_decode(dt, qh.data(), cache.k.data(), cache.v.data(), kv_strides, o.data(), B,
+                               H, cache.len, D, (float)scale));
+  return o.matmul(wo_).reshape({B, 1, C});
 }
 
 Tensor attention_decode(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache) {

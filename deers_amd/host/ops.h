@@ -140,11 +140,25 @@ Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
 // The attention module of src/models/gpt.rs:76-148 on the ROCm device: bias-free
 // q/k/v/out projections with weights [in, out] (y = x @ W, src/nn.rs:183-190), RoPE on
 // queries and keys, the fused causal attention core, head merge, output projection.
+// Keys (rotated) and values of the tokens seen so far, [B,H,L_cap,D]; rows [0,len)
+// are valid.  The reference keeps no cache and re-runs the whole window per generated
+// token (examples/tinystories_train.rs:250-276).
+struct KvCache {
+  Tensor k, v;
+  int64_t len = 0, capacity = 0;
+  static KvCache create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType dtype);
+};
+
 class CausalSelfAttention {
  public:
   CausalSelfAttention(int64_t n_embd, int64_t n_head, Tensor wq, Tensor wk, Tensor wv, Tensor wo);
   // x [B,T,C] with the RoPE tables of precompute_rotary_embeddings -> [B,T,C]
   Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
+  // One generation step (inference, no autograd): x_t [B,1,C] is the token at position
+  // cache.len; its rotated key and its value are appended to the cache and the query
+  // attends to all cache.len+1 positions through the decode kernel.  Returns [B,1,C],
+  // equal to row cache.len of forward() on the whole prefix.
+  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
   std::vector<Tensor> parameters() const { return {wq_, wk_, wv_, wo_}; }
 
  private:

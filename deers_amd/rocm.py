@@ -216,11 +216,18 @@ def matmul_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
         i64(k)))
 
 
-def rope_fwd_raw(dtype, x, cos, sin, y, B, T, H, D, x_strides=None):
-    """deers_rocm_rope_fwd: x logical [B,T,H,D] -> y compact [B,H,T,D]."""
+def rope_fwd_raw(dtype, x, cos, sin, y, B, T, H, D, x_strides=None, y_strides=None):
+    """deers_rocm_rope_fwd: x logical [B,T,H,D] -> y [B,H,T,D] (compact unless y_strides)."""
     _check(load().deers_rocm_rope_fwd(
-        ctypes.c_int(dtype_code(dtype)), x, _strides(x_strides), cos, sin, y, ctypes.c_int64(B),
-        ctypes.c_int64(T), ctypes.c_int64(H), ctypes.c_int64(D)))
+        ctypes.c_int(dtype_code(dtype)), x, _strides(x_strides), cos, sin, y, _strides(y_strides),
+        ctypes.c_int64(B), ctypes.c_int64(T), ctypes.c_int64(H), ctypes.c_int64(D)))
+
+
+def copy_view_raw(dtype, src, src_strides, dst, dst_strides, shape):
+    nd = len(shape)
+    arr = lambda v: (ctypes.c_int64 * nd)(*[int(x) for x in v])  # noqa: E731
+    _check(load().deers_rocm_copy_view(ctypes.c_int(dtype_code(dtype)), src, arr(src_strides), dst,
+                                       arr(dst_strides), arr(shape), ctypes.c_int(nd)))
 
 
 def rope_bwd_raw(dtype, dy, cos, sin, dx, B, T, H, D, dy_strides=None):

@@ -192,6 +192,15 @@ int deers_rocm_neg(int dtype, const void* a, void* out, size_t n);
 int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
                             const int64_t* strides, int ndim, void* dst);
 
+/* dst viewed through dst_strides <- src viewed through src_strides, both of `shape`
+ * (ndim in 1..6, non-negative strides).  The scatter counterpart of copy_compact;
+ * used to append value rows to a KV cache.  The reference has no KV cache (it
+ * re-runs the window per token, examples/tinystories_train.rs:250-276); the closest
+ * reference routine is the strided copy of src/storage/cpu.rs:1063-1102. */
+int deers_rocm_copy_view(int dtype, const void* src, const int64_t* src_strides,
+                         void* dst, const int64_t* dst_strides,
+                         const int64_t* shape, int ndim);
+
 /* ---- batched matrix product ---------------------------------------------------
  * c[batch,m,n] (compact, row-major) = a[batch,m,k] @ b[batch,k,n].  Replaces
  * BackendStorage::matmul (src/storage.rs:270-279; CPU src/storage/cpu.rs:688-753,
@@ -216,10 +225,13 @@ int deers_rocm_matmul(int dtype,
  * precompute_rotary_embeddings (src/models/gpt.rs:12-47), compact, in the tensor's
  * dtype.  D/2 must be a multiple of 16 bytes; arithmetic is f32 with one rounding. */
 
-/* y (compact [B,H,T,D]) = permute(apply_rotary_emb(x)), x logical [B,T,H,D] with
- * element strides x_strides = {b,t,h,d} (NULL = compact, d must be 1). */
+/* y [B,H,T,D] = permute(apply_rotary_emb(x)), x logical [B,T,H,D] with element
+ * strides x_strides = {b,t,h,d} (NULL = compact, d must be 1).  y is compact, or has
+ * element strides y_strides = {b,h,t,d} (d must be 1): with T new positions and a
+ * pointer to row `pos` of a [B,H,L_cap,D] KV cache the rotated keys are appended in
+ * place (pass cos/sin advanced to row `pos` of the tables). */
 int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides,
-                        const void* cos, const void* sin, void* y,
+                        const void* cos, const void* sin, void* y, const int64_t* y_strides,
                         int64_t B, int64_t T, int64_t H, int64_t D);
 
 /* Backward of the above (Permute::backward then the element-wise backward bodies,

@@ -135,6 +135,10 @@ def test_host_attention_module_matches_composed_oracle(tmp_path, dtype, B, T, C,
             "dx": mm(dq, wq.T) + mm(dk, wk.T) + mm(dv, wv.T)}
     got = lambda name, shape: np.fromfile(tmp_path / f"{name}.bin", dtype=dtype).reshape(shape).astype(np.float64)
     assert np.max(np.abs(got("y", (B * T, C)) - want_y)) <= tol
+    if dtype == np.float16:
+        # token-by-token generation through the KV cache reproduces the full forward's rows
+        assert np.max(np.abs(got("y_decode", (B * T, C)) - want_y)) <= tol
+        assert np.max(np.abs(got("y_decode", (B * T, C)) - got("y", (B * T, C)))) <= tol
     for name, ref in want.items():
         g = got(name, ref.shape)
         scale = max(1.0, float(np.max(np.abs(ref))))

@@ -101,3 +101,39 @@ def test_rope_strided_views_and_errors():
                           x_strides=(T * H * D, H * D, D, 2))
     with pytest.raises(rocm.RocmError):
         rocm.rope_fwd_raw(np.float16, None, dc.ptr, ds.ptr, y.ptr, B, T, H, D)
+
+
+@pytest.mark.gpu
+def test_rope_appends_rotated_keys_into_a_cache_and_copy_view_scatters_values():
+    """The decode-time use: T_new rotated key rows written at row `pos` of a
+    [B,H,L_cap,D] cache through output strides, value rows through copy_view."""
+    import ctypes
+    B, H, D, cap, pos, tn = 2, 3, 64, 20, 5, 4
+    T = pos + tn
+    x, _, cos, sin = _inputs(B, T, H, D, np.float16, 24)
+    cache0 = synth.normal((B, H, cap, D), synth.tensor_seed(24, "rope", "cache"), 1.0).astype(np.float16)
+    dcache = rocm.DeviceBuffer.from_numpy(cache0)
+    dx = rocm.DeviceBuffer.from_numpy(np.ascontiguousarray(x[:, pos:]))
+    dc, ds = rocm.DeviceBuffer.from_numpy(cos), rocm.DeviceBuffer.from_numpy(sin)
+    el = 2
+    row = lambda buf, r, width: ctypes.c_void_p(buf.ptr.value + r * width * el)
+    rocm.rope_fwd_raw(np.float16, dx.ptr, row(dc, pos, D // 2), row(ds, pos, D // 2),
+                      row(dcache, pos, D), B, tn, H, D, y_strides=(H * cap * D, cap * D, D, 1))
+    ref = rocm.DeviceBuffer((B, H, T, D), np.float16)
+    dfull = rocm.DeviceBuffer.from_numpy(x)
+    rocm.rope_fwd_raw(np.float16, dfull.ptr, dc.ptr, ds.ptr, ref.ptr, B, T, H, D)
+    got = dcache.numpy()
+    assert np.array_equal(got[:, :, pos:pos + tn], ref.numpy()[:, :, pos:])  # same bits as the full pass
+    assert np.array_equal(got[:, :, :pos], cache0[:, :, :pos])              # nothing else touched
+    assert np.array_equal(got[:, :, pos + tn:], cache0[:, :, pos + tn:])
+    # values: [B,tn,H,D] rows scattered to cache rows pos..pos+tn
+    v = np.ascontiguousarray(x[:, pos:])
+    dv = rocm.DeviceBuffer.from_numpy(v)
+    dvc = rocm.DeviceBuffer.from_numpy(cache0)
+    rocm.copy_view_raw(np.float16, dv.ptr, (tn * H * D, D, H * D, 1), row(dvc, pos, D),
+                       (H * cap * D, cap * D, D, 1), (B, H, tn, D))
+    gotv = dvc.numpy()
+    assert np.array_equal(gotv[:, :, pos:pos + tn], v.transpose(0, 2, 1, 3))
+    assert np.array_equal(gotv[:, :, :pos], cache0[:, :, :pos])
+    with pytest.raises(rocm.RocmError):
+        rocm.copy_view_raw(np.float16, dv.ptr, (1,) * 7, dvc.ptr, (1,) * 7, (1,) * 7)
