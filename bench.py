@@ -246,8 +246,9 @@ def main():
     dom = max(kern, key=lambda n: kern[n]["avg_us"] * kern[n]["calls"])
     # tile GEMMs each kernel must execute (causal-halved, 2*B*H*T^2*D/2 FLOP each)
     gemm = 2.0 * B * H * T * T * D / 2.0
-    kernel_flops = {"attn_fwd_f16": 2 * gemm, "attn_bwd_dkdv_f16": 4 * gemm,
-                    "attn_bwd_dq_f16": 3 * gemm}
+    # (the backward is one launch: the dQ role recomputes S and dP, 3 GEMMs, the dK/dV
+    # role 4)
+    kernel_flops = {"attn_fwd_f16": 2 * gemm, "attn_bwd_f16": 7 * gemm}
     for n, st in kern.items():
         if n in kernel_flops:
             st["tflops"] = kernel_flops[n] / (st["avg_us"] * 1e-6) / 1e12
@@ -256,8 +257,7 @@ def main():
     # HBM bytes per launch at this shape from the FETCH_SIZE / WRITE_SIZE passes of
     # profiles/c2_c4_hbm_traffic_fetch_write.txt (scaled by what the same counters read
     # for a copy of known size); a profiler measurement, not taken in this run.
-    measured_traffic = {"attn_bwd_dkdv_f16": 80.5e6, "attn_bwd_dq_f16": 83.5e6,
-                        "attn_fwd_f16": 53.2e6}
+    measured_traffic = {"attn_bwd_f16": 164.0e6, "attn_fwd_f16": 53.2e6}
     roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": (achieved / PEAK_F16_TFLOPS) if achieved else None,
                 "traffic": measured_traffic.get(dom), "avg_launch_us": kern[dom]["avg_us"],

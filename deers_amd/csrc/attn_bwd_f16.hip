@@ -62,9 +62,8 @@ struct BwdCfg {
 // dK / dV
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_kernel(BwdParams p, int BH,
-                                                                   int n_blocks,
-                                                                   int heads_per_xcd) {
+__device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, int n_blocks,
+                                                  int heads_per_xcd, int block_id) {
   using Cfg = BwdCfg<D>;
   constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
   constexpr int VEC_B = Cfg::VEC_B, SLOT_B = Cfg::SLOT_B;
@@ -86,7 +85,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
   const int T = p.T;
 
   int bh, rank;
-  if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  if (!map_block(block_id, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
   const int kvblk = rank;  // key block 0 walks the most query tiles
   set_block_priority(rank, n_blocks);
   const int b = bh / p.H, h = bh % p.H;
@@ -123,8 +122,24 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
     ld_q_tail[i] = (uint32_t)(row_tail * sqt * 2 + col);
     ld_do_tail[i] = (uint32_t)(row_tail * sdot * 2 + col);
   }
+  // The row statistics of query block qb come from the dQ workgroup that owns it, which
+  // runs in the same launch on the same XCD (see the launch kernel below).
+  int ready_upto = -1;  // query blocks [0, ready_upto] are known to be published
+  auto wait_published = [&](int qb) {
+    if (qb <= ready_upto) return;
+    const int* flag = p.ready + (int64_t)bh * n_blocks + qb;
+    // Bounded: a producer cannot be held up by this workgroup (it was dispatched
+    // earlier and waits for nothing), so the bound is never reached in practice; it
+    // only guarantees that every wave leaves the loop.
+    for (int spins = 0; spins < (1 << 20); ++spins) {
+      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) break;
+      __builtin_amdgcn_s_sleep(8);
+    }
+    ready_upto = qb;
+  };
   auto request = [&](int t) {
     const int tc = min(t, n_tiles - 1);  // clamped repeats are never consumed
+    wait_published(tc * kBwdStep / kBwdBlk);
     const uint32_t slot = lds0 + (t % NS) * SLOT_B;
     const half_t* qbase = Q + (uint32_t)(tc * kBwdStep * sqt);
     const half_t* dobase = dO + (uint32_t)(tc * kBwdStep * sdot);
@@ -288,8 +303,8 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dkdv_f16_ker
 // dQ
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kernel(BwdParams p, int BH, int n_blocks,
-                                                                 int heads_per_xcd) {
+__device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int n_blocks,
+                                                int heads_per_xcd, int block_id) {
   using Cfg = BwdCfg<D>;
   constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
   constexpr int KS = D / 16;
@@ -308,7 +323,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   const int T = p.T;
 
   int bh, rank;
-  if (!map_block(n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  if (!map_block(block_id, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
   const int qtile = n_blocks - 1 - rank;  // the last query block walks the most key tiles
   set_block_priority(rank, n_blocks);
   const int b = bh / p.H, h = bh % p.H;
@@ -458,6 +473,12 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   for (int j = 0; j < n_tiles; ++j) {
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
+    if (j == 0 && tid == 0) {
+      // every wave drained its stores of lse2 / negdelta (wait_all_vmem above) before
+      // this barrier: the rows are in the XCD's L2, tell the dK/dV workgroups
+      __hip_atomic_store(p.ready + (int64_t)bh * n_blocks + qtile, p.epoch, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
     request(j + P);
     const char* slot = smem + (j % NS) * 2 * TILE_B;
     const int kv0 = j * kBwdStep;
@@ -488,35 +509,42 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_dq_f16_kerne
   DEERS_TRACE_POINT(30);
 }
 
+// One launch for the whole backward: the first half of the grid runs the dQ role, the
+// second half the dK/dV role, each longest block first.  Block ids of both halves map
+// to heads the same way (the first half is a multiple of 8 long), so the dK/dV
+// workgroups of a head share an XCD, and its L2, with the dQ workgroups that publish
+// the head's row statistics; they are dispatched after them and poll a per-block
+// flag before they first touch a query block's statistics.  Against two launches
+// this saves a dispatch and lets the heavy dK/dV blocks start while the light dQ
+// blocks drain.
+template <int D>
+__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(BwdParams p, int BH,
+                                                              int n_blocks,
+                                                              int heads_per_xcd) {
+  const int per_role = 8 * n_blocks * heads_per_xcd;
+  if ((int)blockIdx.x < per_role)
+    bwd_dq_f16_body<D>(p, BH, n_blocks, heads_per_xcd, blockIdx.x);
+  else
+    bwd_dkdv_f16_body<D>(p, BH, n_blocks, heads_per_xcd, blockIdx.x - per_role);
+}
+
 template <int D>
 static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
   const int BH = B * p.H;
   const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
   const int heads_per_xcd = (BH + 7) / 8;
-  const dim3 grid(8 * n_blocks * heads_per_xcd);
+  const dim3 grid(2 * 8 * n_blocks * heads_per_xcd);
+  constexpr size_t lds = BwdCfg<D>::kLdsDkdv > BwdCfg<D>::kLdsDq ? BwdCfg<D>::kLdsDkdv : BwdCfg<D>::kLdsDq;
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
-    if (BwdCfg<D>::kLdsDkdv > 64 * 1024)
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dkdv_f16_kernel<D>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)BwdCfg<D>::kLdsDkdv);
-    if (BwdCfg<D>::kLdsDq > 64 * 1024)
-      (void)hipFuncSetAttribute((const void*)attn_bwd_dq_f16_kernel<D>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)BwdCfg<D>::kLdsDq);
+    if (lds > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_bwd_f16_kernel<D>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     attr_set = true;
   }
-  // dQ first: it also publishes lse2 / negdelta for the dK/dV kernel
-  {
-    LaunchScope scope("attn_bwd_dq_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_dq_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDq, stream, p,
-                       BH, n_blocks, heads_per_xcd);
-  }
-  {
-    LaunchScope scope("attn_bwd_dkdv_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_dkdv_f16_kernel<D>, grid, dim3(256), BwdCfg<D>::kLdsDkdv, stream,
-                       p, BH, n_blocks, heads_per_xcd);
-  }
+  LaunchScope scope("attn_bwd_f16", stream);
+  hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, grid, dim3(256), lds, stream, p, BH, n_blocks,
+                     heads_per_xcd);
 }
 
 void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream) {

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
   const int T = p.T;
 
   int bh, rank;
-  if (!map_block(n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
+  if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
   const int qtile = n_qtiles - 1 - rank;  // longest rows first
   const int b = bh / p.H, h = bh % p.H;
 

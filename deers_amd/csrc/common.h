@@ -199,6 +199,9 @@ struct BwdParams {
   // f16 path workspace, rows padded to a multiple of 64 per head (t_pad):
   // lse2 = LSE*log2(e) (+inf in the padding), negdelta = -rowsum(dO o O) (0 in the padding)
   float* lse2; float* negdelta; int t_pad;
+  // ready[bh * n_blocks + q_block] == epoch once the dQ workgroup of that 128-row query
+  // block has published its lse2 / negdelta rows (f16 path, single-launch backward)
+  int* ready; int epoch;
   void* dq; void* dk; void* dv;
   Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
   int H, T;
@@ -213,8 +216,8 @@ struct DecodeParams {
   float scale_log2;
 };
 
-// Maps blockIdx.x to (head, block rank).  Workgroups are dealt round-robin to the 8
-// XCDs, so blockIdx.x % 8 is the XCD: every block of one head is given to one XCD
+// Maps a block id (blockIdx.x, or blockIdx.x minus a multiple of 8) to (head, block
+// rank).  Workgroups are dealt round-robin to the 8 XCDs, so id % 8 is the XCD: every block of one head is given to one XCD
 // (its operands stay in that XCD's L2) and each XCD's list is ordered longest
 // first (rank 0 = the block with the most iterations), which is what the
 // dispatcher's in-order hand-out to free slots needs for an even finish.
@@ -222,10 +225,10 @@ struct DecodeParams {
 // (The head and rank stay in vector registers on purpose: forcing them into scalar
 // registers with readfirstlane was measured and raises the kernels' vector register
 // count through the address arithmetic the compiler then hoists out of the loops.)
-__device__ __forceinline__ bool map_block(int n_blocks, int heads_per_xcd, int BH, int* bh,
-                                          int* rank) {
-  const int xcd = blockIdx.x & 7;
-  const int idx = blockIdx.x >> 3;
+__device__ __forceinline__ bool map_block(int block_id, int n_blocks, int heads_per_xcd, int BH,
+                                          int* bh, int* rank) {
+  const int xcd = block_id & 7;
+  const int idx = block_id >> 3;
   *bh = (idx % heads_per_xcd) * 8 + xcd;
   *rank = idx / heads_per_xcd;
   return *bh < BH;

@@ -48,6 +48,11 @@ struct Runtime {
   void* workspace = nullptr;  // grows on demand, freed never (process lifetime)
   size_t workspace_bytes = 0;
   rocblas_handle blas = nullptr;  // created by the first matmul, bound to `stream`
+  // per (head, 128-row query block) publication flags of the single-launch f16
+  // backward; a flag equals the current epoch once its rows are published
+  int* bwd_ready = nullptr;
+  size_t bwd_ready_len = 0;
+  int bwd_epoch = 0;
 };
 
 Runtime g_rt;
@@ -450,6 +455,23 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   if (int rc = workspace(ws_floats * sizeof(float), &ws)) return rc;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
   p.delta = static_cast<float*>(ws);
+  if (dtype == DEERS_ROCM_F16) {
+    const size_t n_flags = (size_t)(B * H) * (size_t)((T + 127) / 128);
+    if (n_flags > g_rt.bwd_ready_len || g_rt.bwd_epoch == INT32_MAX) {
+      if (g_rt.bwd_ready) {
+        HIP_TRY(hipStreamSynchronize(g_rt.stream));
+        HIP_TRY(hipFree(g_rt.bwd_ready));
+        g_rt.bwd_ready = nullptr;
+      }
+      const size_t want = n_flags > g_rt.bwd_ready_len ? n_flags : g_rt.bwd_ready_len;
+      HIP_TRY(hipMalloc(&g_rt.bwd_ready, want * sizeof(int)));
+      HIP_TRY(hipMemsetAsync(g_rt.bwd_ready, 0, want * sizeof(int), g_rt.stream));
+      g_rt.bwd_ready_len = want;
+      g_rt.bwd_epoch = 0;
+    }
+    p.ready = g_rt.bwd_ready;
+    p.epoch = ++g_rt.bwd_epoch;
+  }
   p.lse2 = static_cast<float*>(ws);
   p.negdelta = static_cast<float*>(ws) + B * H * t_pad;
   p.t_pad = (int)t_pad;
