@@ -7,10 +7,12 @@
 //     dP = dO V^T                           dS = P o (dP - delta),  delta = rowsum(dO o O)
 //     dQ = scale dS K                       dK = scale dS^T Q
 //
-// Two launches, no atomics, bit-reproducible (dQ runs first and publishes, for the
-// rows it owns, negdelta[b,h,t] = -sum_d dO*O and lse2 = LSE*log2(e) as f32 in a
-// workspace whose rows are padded to a multiple of 64 per head, with lse2 = +inf and
-// negdelta = 0 in the padding so padded query rows get probability exactly 0):
+// One launch with two roles, no atomics on data, bit-reproducible (the dQ role
+// publishes, for the rows it owns, negdelta[b,h,t] = -sum_d dO*O and
+// lse2 = LSE*log2(e) as f32 in a workspace whose rows are padded to a multiple of 64
+// per head, with lse2 = +inf and negdelta = 0 in the padding so padded query rows
+// get probability exactly 0; the dK/dV role waits for a block's rows through a flag,
+// see attn_bwd_f16_kernel):
 //   2. dK/dV   : a workgroup owns 128 key rows (32 per wave, K^T and V^T held in
 //                registers as B operands) and walks the 64-row query tiles at or
 //                below the diagonal.  Orientation S[q,kv] (one key column per lane)
@@ -22,7 +24,7 @@
 //                Orientation S^T[kv,q] (one query column per lane, LSE and delta are
 //                per-lane scalars); dS^T leaves the accumulators as the B operand of
 //                dQ^T += K^T dS^T with K^T fragments read transposed from LDS.
-// Recomputing S and dP in both kernels costs 7 tile GEMMs instead of 5 but
+// Recomputing S and dP in both roles costs 7 tile GEMMs instead of 5 but
 // keeps every product in registers and needs no dQ accumulation buffer.
 //
 // The "- delta" of dS is folded into the dP accumulator's initial value, so the
