@@ -18,6 +18,7 @@ materialised CPU path) timed on this box's host cores on a bounded sample.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import statistics
@@ -181,6 +182,45 @@ def bench_rope(steps: int, warmup: int):
     return out
 
 
+def bench_log_softmax(steps: int, warmup: int):
+    """Row-wise log-softmax forward and backward at config 5's logits, [8192, 50257] f32
+    (1.65 GB).  HBM-bound: the forward must read x and write y (2 x 1.65 GB), the
+    backward read grad and y and write dx (3 x 1.65 GB); the second sweep over each
+    201 KB row is served by L2."""
+    outer, inner = 8192, 50257
+    rows = synth.normal((256, inner), synth.tensor_seed(0, "lsm", "x"), 2.0).astype(np.float32)
+    x = rocm.DeviceBuffer((outer, inner), np.float32)
+    for r in range(0, outer, 256):  # the same 256 rows tiled: content does not change the work
+        rocm._check(rocm.load().deers_rocm_htod(
+            ctypes.c_void_p(x.ptr.value + r * inner * 4),
+            rows.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(rows.nbytes)))
+    y = rocm.DeviceBuffer((outer, inner), np.float32)
+    g = rocm.DeviceBuffer((outer, inner), np.float32, zeros=True)
+    d = rocm.DeviceBuffer((outer, inner), np.float32)
+
+    def step():
+        rocm.log_softmax_fwd_raw(np.float32, x.ptr, y.ptr, outer, inner)
+        rocm.log_softmax_bwd_raw(np.float32, g.ptr, y.ptr, d.ptr, outer, inner)
+
+    for _ in range(warmup):
+        step()
+    rocm.sync()
+    rocm.profile_enable(True)
+    for _ in range(steps):
+        step()
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    one = float(outer) * inner * 4
+    alg = {"log_softmax_fwd": 2 * one, "log_softmax_bwd": 3 * one}
+    out = {"shape": [outer, inner], "dtype": "f32"}
+    for name, (calls, ms) in prof.items():
+        us = 1e3 * ms / calls
+        out[name] = {"avg_us": us, "bytes_per_launch": alg[name],
+                     "GB/s": alg[name] / (us * 1e-6) / 1e9,
+                     "frac_hbm_peak": alg[name] / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -212,7 +252,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -228,6 +268,9 @@ def main():
             print(json.dumps({"only": "decode", **bench_decode(args.steps, args.warmup)}))
         elif args.only == "rope":
             print(json.dumps({"only": "rope", **bench_rope(args.steps, args.warmup)}))
+        elif args.only == "log_softmax":
+            print(json.dumps({"only": "log_softmax",
+                              **bench_log_softmax(min(args.steps, 20), min(args.warmup, 5))}))
         elif args.only == "copy":
             print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
         else:

@@ -34,6 +34,10 @@ void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
 void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
                  const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
                  int T, int H, int D, hipStream_t stream);
+void launch_log_softmax_fwd(int dtype_f16, const void* x, void* out, int64_t outer, int64_t inner,
+                            hipStream_t stream);
+void launch_log_softmax_bwd(int dtype_f16, const void* grad, const void* lsm, void* out,
+                            int64_t outer, int64_t inner, hipStream_t stream);
 void launch_copy_view(int dtype_f16, const void* src, const int64_t* src_strides, void* dst,
                       const int64_t* dst_strides, const int64_t* shape, int ndim,
                       hipStream_t stream);
@@ -593,6 +597,38 @@ int deers_rocm_copy_view(int dtype, const void* src, const int64_t* src_strides,
       return fail(DEERS_ROCM_ERR_LAYOUT, "copy_view: negative extent or stride in dim %d", d);
   deers::launch_copy_view(dtype == DEERS_ROCM_F16, src, src_strides, dst, dst_strides, shape, ndim,
                           g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- row-wise log-softmax ----
+
+static int lsm_check(const char* what, int dtype, int64_t outer, int64_t inner) {
+  if (int rc = check_dtype(dtype)) return rc;
+  if (outer < 0 || inner < 1 || outer > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "%s: need 0 <= outer < 2^31 rows of inner >= 1 elements", what);
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_log_softmax_fwd(int dtype, const void* x, void* out, int64_t outer, int64_t inner) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = lsm_check("log_softmax_fwd", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !out) return fail(DEERS_ROCM_ERR_ARG, "log_softmax_fwd: null pointer");
+  deers::launch_log_softmax_fwd(dtype == DEERS_ROCM_F16, x, out, outer, inner, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, void* out,
+                               int64_t outer, int64_t inner) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = lsm_check("log_softmax_bwd", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!grad || !lsm || !out) return fail(DEERS_ROCM_ERR_ARG, "log_softmax_bwd: null pointer");
+  deers::launch_log_softmax_bwd(dtype == DEERS_ROCM_F16, grad, lsm, out, outer, inner, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -207,6 +207,16 @@ def copy_compact_raw(dtype, src, shape, strides, dst):
                                           ctypes.c_int(nd), dst))
 
 
+def log_softmax_fwd_raw(dtype, x, out, outer, inner):
+    _check(load().deers_rocm_log_softmax_fwd(ctypes.c_int(dtype_code(dtype)), x, out,
+                                             ctypes.c_int64(outer), ctypes.c_int64(inner)))
+
+
+def log_softmax_bwd_raw(dtype, grad, lsm, out, outer, inner):
+    _check(load().deers_rocm_log_softmax_bwd(ctypes.c_int(dtype_code(dtype)), grad, lsm, out,
+                                             ctypes.c_int64(outer), ctypes.c_int64(inner)))
+
+
 def matmul_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
     """deers_rocm_matmul: c[batch,m,n] = a @ b; strides are (row, col, batch) in elements."""
     i64 = ctypes.c_int64

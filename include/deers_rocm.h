@@ -192,6 +192,17 @@ int deers_rocm_neg(int dtype, const void* a, void* out, size_t n);
 int deers_rocm_copy_compact(int dtype, const void* src, const int64_t* shape,
                             const int64_t* strides, int ndim, void* dst);
 
+/* ---- row-wise log-softmax --------------------------------------------------------
+ * The fused op of the loss (FusedLogSoftmax, src/ops.rs:1186-1251) over compact
+ * [outer, inner] data, innermost axis reduced; replaces
+ * BackendStorage::log_softmax_fwd / log_softmax_bwd (src/storage.rs:284-302; CPU
+ * src/storage/cpu.rs:793-888).  f16 computes in f32 and rounds once.  out may alias
+ * x (forward) or grad (backward). */
+int deers_rocm_log_softmax_fwd(int dtype, const void* x, void* out, int64_t outer, int64_t inner);
+/* out = grad - exp(lsm) * rowsum(grad), lsm = the forward's output. */
+int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, void* out,
+                               int64_t outer, int64_t inner);
+
 /* dst viewed through dst_strides <- src viewed through src_strides, both of `shape`
  * (ndim in 1..6, non-negative strides).  The scatter counterpart of copy_compact;
  * used to append value rows to a KV cache.  The reference has no KV cache (it

@@ -5,7 +5,8 @@ this package; the shipped library never does.  The arithmetic lives in
 ``attention_ref.cc`` (a restatement of the reference's CPU attention,
 src/models/gpt.rs:139-144 and its autograd backward); this module moves numpy
 arrays across the C boundary and restates the rotary embedding around the core
-(src/models/gpt.rs:12-73) directly in numpy.
+(src/models/gpt.rs:12-73) and the loss's row-wise log-softmax
+(src/storage/cpu.rs:793-888) directly in numpy.
 """
 from __future__ import annotations
 
@@ -221,3 +222,34 @@ def rope_apply_bwd(dy: np.ndarray, cos: np.ndarray, sin: np.ndarray, dtype=np.fl
     s = np.asarray(sin, dtype=dtype)[None, :, None, :]
     d1, d2 = dy[..., :half], dy[..., half:]
     return np.concatenate([d1 * c + d2 * (s * dtype(-1.0)), d1 * s + d2 * c], axis=3)
+
+
+# ---- row-wise log-softmax (numpy restatement) ----
+
+def _lsm_compute_type(dtype):
+    # f16 and f32 rows accumulate in f32 as the reference does; float64 is accepted so
+    # that tests can difference the same formula without rounding noise.
+    return np.float64 if np.dtype(dtype) == np.float64 else np.float32
+
+
+def log_softmax_fwd(x: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """log_softmax_fwd over the last axis of compact [outer, inner] data
+    (src/storage/cpu.rs:793-840): per row max, sum of exp(x - max) in f32,
+    lse = ln(sum) + max, out = x - lse; f16 rows convert each element to f32 and round
+    the result once."""
+    ct = _lsm_compute_type(dtype)
+    xf = np.asarray(x, dtype=dtype).astype(ct)
+    mx = xf.max(axis=-1, keepdims=True)
+    s = np.exp(xf - mx, dtype=ct).sum(axis=-1, keepdims=True, dtype=ct)
+    lse = np.log(s, dtype=ct) + mx
+    return (xf - lse).astype(dtype)
+
+
+def log_softmax_bwd(grad: np.ndarray, lsm: np.ndarray, dtype=np.float32) -> np.ndarray:
+    """log_softmax_bwd (src/storage/cpu.rs:842-888): per row s = sum(grad) in f32,
+    out = grad - exp(lsm) * s."""
+    ct = _lsm_compute_type(dtype)
+    g = np.asarray(grad, dtype=dtype).astype(ct)
+    l = np.asarray(lsm, dtype=dtype).astype(ct)
+    s = g.sum(axis=-1, keepdims=True, dtype=ct)
+    return (g - np.exp(l, dtype=ct) * s).astype(dtype)

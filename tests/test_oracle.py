@@ -302,3 +302,66 @@ def test_rope_backward_is_the_transpose():
     back = oracle.rope_apply_bwd(oracle.rope_apply(x, c64, s64, dtype=np.float64), c64, s64,
                                  dtype=np.float64)
     assert np.allclose(back, x, atol=1e-6)
+
+
+# ---- row-wise log-softmax (src/storage/cpu.rs:793-888) ----
+
+REF_LSM_INPUT = np.array([[1.0, 2.0, 3.0], [1.5, 0.5, -1.0]], dtype=np.float32)  # tests/tensor.rs:296
+
+
+def test_log_softmax_reference_literal_against_library_and_definition():
+    from scipy.special import log_softmax as scipy_lsm
+    y = oracle.log_softmax_fwd(REF_LSM_INPUT)
+    # the reference's own test compares with a library log-softmax on this input
+    assert np.abs(y - scipy_lsm(REF_LSM_INPUT.astype(np.float64), axis=1)).max() < 1e-6
+    # textbook definition, no max subtraction: x - ln(sum e^x)
+    naive = [[v - math.log(sum(math.exp(u) for u in row)) for v in row] for row in REF_LSM_INPUT.tolist()]
+    assert np.abs(y - np.array(naive)).max() < 1e-6
+    # row [1,2,3]: last entry is -ln(1 + e^-1 + e^-2)
+    assert abs(y[0, 2] + math.log(1 + math.exp(-1) + math.exp(-2))) < 1e-6
+
+
+def test_log_softmax_invariants():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((7, 333)) * 4).astype(np.float32)
+    y = oracle.log_softmax_fwd(x)
+    assert np.abs(np.exp(y.astype(np.float64)).sum(axis=1) - 1).max() < 1e-5
+    # shift invariance per row, and stability where the naive form overflows
+    assert np.abs(oracle.log_softmax_fwd(x + np.float32(3.0)) - y).max() < 1e-5
+    big = np.array([[1000.0, 1000.0, 999.0]], dtype=np.float32)
+    yb = oracle.log_softmax_fwd(big)
+    # lse = 1000.86 carries an f32 ulp of 6e-5
+    assert np.isfinite(yb).all() and abs(yb[0, 0] + math.log(2 + math.exp(-1))) < 1e-4
+    # a constant row is -ln(n); a single column is 0
+    assert np.abs(oracle.log_softmax_fwd(np.full((2, 10), 3.5, np.float32)) + math.log(10)).max() < 1e-6
+    assert (oracle.log_softmax_fwd(rng.standard_normal((4, 1)).astype(np.float32)) == 0).all()
+    # f16 rows: computed in f32, rounded once
+    xh = x.astype(np.float16)
+    yh = oracle.log_softmax_fwd(xh, dtype=np.float16)
+    assert yh.dtype == np.float16
+    assert (yh == oracle.log_softmax_fwd(xh.astype(np.float32)).astype(np.float16)).all()
+
+
+def test_log_softmax_backward_finite_differences_and_closed_form():
+    from scipy.special import log_softmax as scipy_lsm
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((3, 9))
+    g = rng.standard_normal((3, 9))
+    y = oracle.log_softmax_fwd(x, dtype=np.float64)
+    dx = oracle.log_softmax_bwd(g, y, dtype=np.float64)
+    # central differences of the library routine, not of the oracle
+    h = 1e-6
+    for (i, j) in [(0, 0), (1, 4), (2, 8), (0, 5)]:
+        xp, xm = x.copy(), x.copy()
+        xp[i, j] += h
+        xm[i, j] -= h
+        fd = (np.sum(scipy_lsm(xp, axis=1) * g) - np.sum(scipy_lsm(xm, axis=1) * g)) / (2 * h)
+        assert abs(fd - dx[i, j]) < 1e-6
+    # rows of dx sum to zero (softmax sums to one)
+    assert np.abs(dx.sum(axis=1)).max() < 1e-12
+    # the reference's backward test: loss = sum(log_softmax(x)) so g = 1 and
+    # dx = 1 - n * softmax(x)  (tests/tensor.rs:323-351)
+    yr = oracle.log_softmax_fwd(REF_LSM_INPUT)
+    dr = oracle.log_softmax_bwd(np.ones_like(yr), yr)
+    e = np.exp(REF_LSM_INPUT.astype(np.float64))
+    assert np.abs(dr - (1 - 3 * e / e.sum(axis=1, keepdims=True))).max() < 1e-6
