@@ -315,6 +315,55 @@ static int run_module(const std::string& dir) {
   return 0;
 }
 
+// Log-softmax through the graph: x [outer, inner] -> log_softmax(1), swept backward from
+// a given output gradient, and the reference's own case (loss = sum, tests/tensor.rs:323-351).
+static int run_log_softmax(const std::string& dir) {
+  check(deers_rocm_init(0));
+  int dt, outer, inner;
+  {
+    std::ifstream f(dir + "/case.txt");
+    if (!(f >> dt >> outer >> inner)) { std::printf("FAIL bad case.txt\n"); return 2; }
+  }
+  const DType dtype = dt == 0 ? DType::F16 : DType::F32;
+  const std::vector<int64_t> shape{outer, inner};
+  auto load = [&](const char* name) {
+    auto bytes = read_file(dir + "/" + name);
+    if (bytes.size() != (size_t)outer * inner * size_in_bytes(dtype)) { std::printf("FAIL size of %s\n", name); std::exit(2); }
+    return Tensor::from_host(bytes.data(), shape, dtype);
+  };
+  Tensor x = load("x.bin").attach();
+  Tensor seed = load("g.bin");
+  Tensor y = x.log_softmax(1);
+  EXPECT(y.requires_grad() && std::string(y.op()->name()) == "FusedLogSoftmax");
+  dump(y, dir + "/y.bin");
+  GradientStore grads = y.backward_from(seed);
+  const Tensor* gx = grads.get(x.id());
+  EXPECT(gx != nullptr);
+  if (gx) dump(*gx, dir + "/dx.bin");
+  // a transposed (non-compact) view is compacted first, as the op does in the reference
+  Tensor xt = load("x.bin").attach();
+  Tensor yt = xt.transpose().log_softmax(1);  // [inner, outer], rows = columns of x
+  EXPECT(yt.is_compact());
+  dump(yt, dir + "/yt.bin");
+  GradientStore gt = yt.backward();  // loss = sum(log_softmax)
+  const Tensor* gxt = gt.get(xt.id());
+  EXPECT(gxt != nullptr);
+  if (gxt) {
+    EXPECT(gxt->shape() == xt.shape());
+    dump(*gxt, dir + "/dxt.bin");
+  }
+  bool threw = false;
+  try { x.log_softmax(0); } catch (const std::logic_error&) { threw = true; }
+  EXPECT(threw);
+  {
+    NoGradGuard guard;
+    Tensor yn = x.log_softmax(1);
+    EXPECT(!yn.requires_grad() && yn.op() == nullptr);
+  }
+  std::printf("ok log_softmax\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "graph";
   try {
@@ -326,10 +375,12 @@ int main(int argc, char** argv) {
       test_graph_of_attention_views();
     } else if (mode == "gpu" && argc > 2) {
       if (int rc = run_gpu(argv[2])) return rc;
+    } else if (mode == "lsm" && argc > 2) {
+      if (int rc = run_log_softmax(argv[2])) return rc;
     } else if (mode == "module" && argc > 2) {
       if (int rc = run_module(argv[2])) return rc;
     } else {
-      std::printf("usage: host_test graph | gpu <dir> | module <dir>\n");
+      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | module <dir>\n");
       return 2;
     }
   } catch (const std::exception& e) {

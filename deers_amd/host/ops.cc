@@ -211,6 +211,35 @@ Tensor Tensor::add(const Tensor& other) const {
   return EWiseAdd::forward(std::make_unique<EWiseAdd>(*this, other));
 }
 
+// ---- FusedLogSoftmax ----
+FusedLogSoftmax::FusedLogSoftmax(Tensor arg, size_t axis) : arg_(std::move(arg)), axis_(axis) {
+  if (arg_.layout().ndim() == 0 || axis_ != arg_.layout().ndim() - 1)
+    throw std::logic_error("FusedLogSoftmax: the axis must be the last one");
+}
+Tensor FusedLogSoftmax::forward(std::unique_ptr<FusedLogSoftmax> self) {
+  const Tensor x = self->arg_.compact();
+  const int64_t inner = x.shape()[self->axis_];
+  const int64_t outer = inner ? (int64_t)x.layout().size() / inner : 0;
+  Tensor out = empty(x.shape(), x.dtype(), backed(x));
+  if (backed(x)) check(deers_rocm_log_softmax_fwd((int)x.dtype(), x.data(), out.data(), outer, inner));
+  self->lsm_output_ = out;
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void FusedLogSoftmax::backward(GradientStore& grads, const Tensor& out_grad) const {
+  if (!lsm_output_.defined()) throw std::logic_error("forward must run before backward");
+  const Tensor g = out_grad.compact();
+  const int64_t inner = g.shape()[axis_];
+  const int64_t outer = inner ? (int64_t)g.layout().size() / inner : 0;
+  Tensor dx = empty(g.shape(), g.dtype(), backed(g));
+  if (backed(g))
+    check(deers_rocm_log_softmax_bwd((int)g.dtype(), g.data(), lsm_output_.data(), dx.data(), outer,
+                                     inner));
+  grads.accumulate(arg_, dx);
+}
+Tensor Tensor::log_softmax(size_t axis) const {
+  return FusedLogSoftmax::forward(std::make_unique<FusedLogSoftmax>(*this, axis));
+}
+
 // ---- FusedCausalAttention ----
 FusedCausalAttention::FusedCausalAttention(Tensor q, Tensor k, Tensor v, double scale)
     : q_(std::move(q)), k_(std::move(k)), v_(std::move(v)), scale_(scale) {

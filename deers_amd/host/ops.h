@@ -115,6 +115,24 @@ class FusedCausalAttention : public TensorOp {
 // (src/models/gpt.rs:49-73, 135-136) as one op: returns the rotated heads as compact
 // [B,H,T,D]; the backward hands the [B,T,H,D] gradient to the projection.  cos and
 // sin are the tables of precompute_rotary_embeddings and carry no gradient.
+// src/ops.rs:1186-1251: log-softmax over the last axis in one kernel, its output saved
+// for the backward (out_grad - exp(lsm) * rowsum(out_grad)).  Tensor::log_softmax takes
+// this path when the axis is the last one (src/tensor.rs:408-427); other axes are not
+// part of this host.
+class FusedLogSoftmax : public TensorOp {
+ public:
+  FusedLogSoftmax(Tensor arg, size_t axis);  // std::logic_error unless axis is the last
+  static Tensor forward(std::unique_ptr<FusedLogSoftmax> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "FusedLogSoftmax"; }
+
+ private:
+  Tensor arg_;
+  size_t axis_;
+  Tensor lsm_output_;  // no op, no grad: saved like the reference's lsm_output
+};
+
 class RotaryHeads : public TensorOp {
  public:
   RotaryHeads(Tensor x, Tensor cos, Tensor sin);

@@ -130,6 +130,8 @@ class Tensor {
   Tensor transpose() const;  // swaps the last two axes (a Permute)
   Tensor reshape(const std::vector<int64_t>& shape) const;  // compacts first (src/ops.rs:913)
   Tensor matmul(const Tensor& other) const;
+  // Log-softmax over the last axis through the fused op (src/tensor.rs:408-427).
+  Tensor log_softmax(size_t axis) const;
   // Differentiable element-wise ops used by the contract tests.
   Tensor neg() const;
   Tensor add(const Tensor& other) const;

@@ -143,3 +143,38 @@ def test_host_attention_module_matches_composed_oracle(tmp_path, dtype, B, T, C,
         g = got(name, ref.shape)
         scale = max(1.0, float(np.max(np.abs(ref))))
         assert np.max(np.abs(g - ref)) <= tol * scale, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,outer,inner", [(np.float32, 6, 777), (np.float16, 5, 1000),
+                                               (np.float32, 2, 3)])
+def test_host_fused_log_softmax_matches_oracle(tmp_path, dtype, outer, inner):
+    import oracle
+    if (outer, inner) == (2, 3):  # the reference's literal, tests/tensor.rs:296
+        x = np.array([[1.0, 2.0, 3.0], [1.5, 0.5, -1.0]], dtype=dtype)
+    else:
+        x = synth.normal((outer, inner), synth.tensor_seed(41, "hostlsm", "x"), 3.0).astype(dtype)
+    g = synth.normal((outer, inner), synth.tensor_seed(41, "hostlsm", "g"), 1.0).astype(dtype)
+    x.tofile(tmp_path / "x.bin")
+    g.tofile(tmp_path / "g.bin")
+    (tmp_path / "case.txt").write_text(f"{0 if dtype == np.float16 else 1} {outer} {inner}\n")
+    r = _run("lsm", str(tmp_path))
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ok log_softmax" in r.stdout and "all passed" in r.stdout
+
+    def out(name, shape):
+        return np.fromfile(tmp_path / name, dtype=dtype).reshape(shape)
+
+    x32 = x.astype(np.float32)
+    tol = lambda want: (5e-3 + np.abs(want).max() * 2 ** -11) if dtype == np.float16 else 1e-4
+    y = out("y.bin", (outer, inner))
+    want = oracle.log_softmax_fwd(x32)
+    assert np.abs(y.astype(np.float32) - want).max() <= tol(want)
+    want_dx = oracle.log_softmax_bwd(g.astype(np.float32), y.astype(np.float32))
+    assert np.abs(out("dx.bin", (outer, inner)).astype(np.float32) - want_dx).max() <= tol(want_dx)
+    # transposed view: rows are the columns of x; loss = sum, so d = 1 - n * softmax
+    yt = out("yt.bin", (inner, outer))
+    want_t = oracle.log_softmax_fwd(np.ascontiguousarray(x32.T))
+    assert np.abs(yt.astype(np.float32) - want_t).max() <= tol(want_t)
+    want_dxt = oracle.log_softmax_bwd(np.ones_like(want_t), yt.astype(np.float32)).T
+    assert np.abs(out("dxt.bin", (outer, inner)).astype(np.float32) - want_dxt).max() <= tol(want_dxt)
