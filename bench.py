@@ -221,6 +221,44 @@ def bench_log_softmax(steps: int, warmup: int):
     return out
 
 
+def bench_adamw(steps: int, warmup: int):
+    """Fused AdamW step over 124,439,808 f32 parameters (GPT-2 small, as one tensor), and
+    the sum of squares of as many gradients.  HBM-bound: the step reads w, g, m, v and
+    writes w, m, v (28 B per parameter); the reduction reads g (4 B)."""
+    n = 124_439_808
+    w = rocm.DeviceBuffer((n,), np.float32)
+    rocm.fill_raw(np.float32, w.ptr, n, 0.02)
+    g = rocm.DeviceBuffer((n,), np.float32)
+    rocm.fill_raw(np.float32, g.ptr, n, 1e-3)
+    m = rocm.DeviceBuffer((n,), np.float32, zeros=True)
+    v = rocm.DeviceBuffer((n,), np.float32, zeros=True)
+    total = rocm.DeviceBuffer((1,), np.float32)
+    t = [0]
+
+    def step():
+        t[0] += 1
+        rocm.sum_squares_raw(np.float32, g.ptr, n, total.ptr)
+        rocm.adamw_step_raw(np.float32, w.ptr, g.ptr, m.ptr, v.ptr, n, 3e-4, 0.9, 0.95, 1e-8, 0.1,
+                            t[0], 0.5)
+
+    for _ in range(warmup):
+        step()
+    rocm.sync()
+    rocm.profile_enable(True)
+    for _ in range(steps):
+        step()
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    alg = {"adamw_step": 28.0 * n, "sumsq": 4.0 * n}
+    out = {"parameters": n, "dtype": "f32"}
+    for name, (calls, ms) in prof.items():
+        us = 1e3 * ms / calls
+        out[name] = {"avg_us": us, "bytes_per_launch": alg[name],
+                     "GB/s": alg[name] / (us * 1e-6) / 1e9,
+                     "frac_hbm_peak": alg[name] / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -252,7 +290,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -271,6 +309,9 @@ def main():
         elif args.only == "log_softmax":
             print(json.dumps({"only": "log_softmax",
                               **bench_log_softmax(min(args.steps, 20), min(args.warmup, 5))}))
+        elif args.only == "adamw":
+            print(json.dumps({"only": "adamw",
+                              **bench_adamw(min(args.steps, 20), min(args.warmup, 5))}))
         elif args.only == "copy":
             print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
         else:

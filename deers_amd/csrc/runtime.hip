@@ -38,6 +38,13 @@ void launch_log_softmax_fwd(int dtype_f16, const void* x, void* out, int64_t out
                             hipStream_t stream);
 void launch_log_softmax_bwd(int dtype_f16, const void* grad, const void* lsm, void* out,
                             int64_t outer, int64_t inner, hipStream_t stream);
+int sumsq_partial_count();
+void launch_adamw(int dtype_f16, void* w, const void* g, void* m, void* v, int64_t n, double lr,
+                  double beta1, double beta2, double eps, double weight_decay, int step,
+                  double grad_scale, hipStream_t stream);
+void launch_sumsq(int dtype_f16, const void* g, int64_t n, float* partial, float* out,
+                  int accumulate, hipStream_t stream);
+void launch_scale(int dtype_f16, void* x, int64_t n, double scale, hipStream_t stream);
 void launch_copy_view(int dtype_f16, const void* src, const int64_t* src_strides, void* dst,
                       const int64_t* dst_strides, const int64_t* shape, int ndim,
                       hipStream_t stream);
@@ -629,6 +636,50 @@ int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, voi
   if (outer == 0) return DEERS_ROCM_OK;
   if (!grad || !lsm || !out) return fail(DEERS_ROCM_ERR_ARG, "log_softmax_bwd: null pointer");
   deers::launch_log_softmax_bwd(dtype == DEERS_ROCM_F16, grad, lsm, out, outer, inner, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- optimizer step ----
+
+int deers_rocm_adamw_step(int dtype, void* w, const void* grad, void* m, void* v, int64_t n,
+                          double lr, double beta1, double beta2, double eps, double weight_decay,
+                          int64_t step, double grad_scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "adamw_step: negative element count");
+  if (step < 1 || step > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "adamw_step: step counts from 1 (got %lld)", (long long)step);
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!w || !grad || !m || !v) return fail(DEERS_ROCM_ERR_ARG, "adamw_step: null pointer");
+  deers::launch_adamw(dtype == DEERS_ROCM_F16, w, grad, m, v, n, lr, beta1, beta2, eps, weight_decay,
+                      (int)step, grad_scale, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_sum_squares(int dtype, const void* x, int64_t n, float* total, int accumulate) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "sum_squares: negative element count");
+  if (!total || (n > 0 && !x)) return fail(DEERS_ROCM_ERR_ARG, "sum_squares: null pointer");
+  void* ws = nullptr;
+  if (int rc = workspace(deers::sumsq_partial_count() * sizeof(float), &ws)) return rc;
+  deers::launch_sumsq(dtype == DEERS_ROCM_F16, x, n, (float*)ws, total, accumulate, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_scale(int dtype, void* x, int64_t n, double scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "scale: negative element count");
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!x) return fail(DEERS_ROCM_ERR_ARG, "scale: null pointer");
+  deers::launch_scale(dtype == DEERS_ROCM_F16, x, n, scale, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -217,6 +217,24 @@ def log_softmax_bwd_raw(dtype, grad, lsm, out, outer, inner):
                                              ctypes.c_int64(outer), ctypes.c_int64(inner)))
 
 
+def adamw_step_raw(dtype, w, grad, m, v, n, lr, beta1, beta2, eps, weight_decay, step,
+                   grad_scale=1.0):
+    _check(load().deers_rocm_adamw_step(
+        ctypes.c_int(dtype_code(dtype)), w, grad, m, v, ctypes.c_int64(n), ctypes.c_double(lr),
+        ctypes.c_double(beta1), ctypes.c_double(beta2), ctypes.c_double(eps),
+        ctypes.c_double(weight_decay), ctypes.c_int64(step), ctypes.c_double(grad_scale)))
+
+
+def sum_squares_raw(dtype, x, n, total, accumulate=False):
+    _check(load().deers_rocm_sum_squares(ctypes.c_int(dtype_code(dtype)), x, ctypes.c_int64(n),
+                                         total, ctypes.c_int(1 if accumulate else 0)))
+
+
+def scale_raw(dtype, x, n, scale):
+    _check(load().deers_rocm_scale(ctypes.c_int(dtype_code(dtype)), x, ctypes.c_int64(n),
+                                   ctypes.c_double(scale)))
+
+
 def matmul_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
     """deers_rocm_matmul: c[batch,m,n] = a @ b; strides are (row, col, batch) in elements."""
     i64 = ctypes.c_int64

@@ -203,6 +203,27 @@ int deers_rocm_log_softmax_fwd(int dtype, const void* x, void* out, int64_t oute
 int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, void* out,
                                int64_t outer, int64_t inner);
 
+/* ---- optimizer step ---------------------------------------------------------------
+ * One AdamW update of one parameter tensor in place, the body of the loop in
+ * AdamW::step_with_grads (src/optim.rs:214-251): w, m, v (n elements each, compact) are
+ * read and rewritten, grad is read.  `step` is the 1-based step count AFTER the
+ * increment at src/optim.rs:215; lr, betas, eps, weight_decay are the optimizer's f64
+ * fields.  The arithmetic follows the reference's chain of tensor ops, rounding to the
+ * tensor's type after each, so results are bit-identical to it for f32 and f16 alike
+ * (for f16 that includes eps = 1e-8 rounding to zero).  grad_scale != 1 first scales
+ * the gradient as clip_grad_norm would (src/optim.rs:288-293) without another pass
+ * over memory; grad itself is not modified. */
+int deers_rocm_adamw_step(int dtype, void* w, const void* grad, void* m, void* v, int64_t n,
+                          double lr, double beta1, double beta2, double eps, double weight_decay,
+                          int64_t step, double grad_scale);
+/* *total (a float in device memory) = or += sum of x[i]^2 in f32, the reduction of
+ * clip_grad_norm (src/optim.rs:270-277) for one gradient; the partition and the order
+ * of additions are fixed, so repeated calls give the same bits. */
+int deers_rocm_sum_squares(int dtype, const void* x, int64_t n, float* total, int accumulate);
+/* x *= scale in place, scale cast as the reference's scalar ops cast it
+ * (storage::ScalarMul, src/storage.rs:108-123): clip_grad_norm's rescaling. */
+int deers_rocm_scale(int dtype, void* x, int64_t n, double scale);
+
 /* dst viewed through dst_strides <- src viewed through src_strides, both of `shape`
  * (ndim in 1..6, non-negative strides).  The scatter counterpart of copy_compact;
  * used to append value rows to a KV cache.  The reference has no KV cache (it

@@ -5,8 +5,9 @@ this package; the shipped library never does.  The arithmetic lives in
 ``attention_ref.cc`` (a restatement of the reference's CPU attention,
 src/models/gpt.rs:139-144 and its autograd backward); this module moves numpy
 arrays across the C boundary and restates the rotary embedding around the core
-(src/models/gpt.rs:12-73) and the loss's row-wise log-softmax
-(src/storage/cpu.rs:793-888) directly in numpy.
+(src/models/gpt.rs:12-73), the loss's row-wise log-softmax
+(src/storage/cpu.rs:793-888) and the AdamW step with gradient clipping
+(src/optim.rs:214-296) directly in numpy.
 """
 from __future__ import annotations
 
@@ -253,3 +254,67 @@ def log_softmax_bwd(grad: np.ndarray, lsm: np.ndarray, dtype=np.float32) -> np.n
     l = np.asarray(lsm, dtype=dtype).astype(ct)
     s = g.sum(axis=-1, keepdims=True, dtype=ct)
     return (g - np.exp(l, dtype=ct) * s).astype(dtype)
+
+
+# ---- optimizer step (numpy restatement; every tensor op rounds to the tensor's dtype) ----
+
+def _powi(a: float, b: int) -> float:
+    """f64 power by repeated squaring, what Rust's f64::powi lowers to."""
+    recip = b < 0
+    b = abs(b)
+    r = 1.0
+    while True:
+        if b & 1:
+            r *= a
+        b //= 2
+        if b == 0:
+            break
+        a *= a
+    return 1.0 / r if recip else r
+
+
+def _scalar(x: float, dtype):
+    """A host f64 scalar as storage::ScalarMul / ScalarAdd see it (src/storage.rs:108-123):
+    cast to f32, then for f16 tensors to f16."""
+    return np.dtype(dtype).type(np.float32(x))
+
+
+def adamw_step(w, g, m, v, step: int, lr: float, betas=(0.9, 0.999), eps: float = 1e-8,
+               weight_decay: float = 0.0, dtype=np.float32):
+    """One AdamW::step_with_grads body for one parameter (src/optim.rs:214-251) as the
+    same chain of element-wise ops, each rounding to `dtype`; `step` is the count after
+    the increment at line 215.  Returns the new (w, m, v)."""
+    T = np.dtype(dtype).type
+    w, g, m, v = (np.asarray(a, dtype=dtype) for a in (w, g, m, v))
+    beta1, beta2 = betas
+    bc1 = 1.0 - _powi(beta1, step)
+    bc2 = 1.0 - _powi(beta2, step)
+    S = lambda x: _scalar(x, dtype)
+    with np.errstate(all="ignore"):
+        m = (m * S(beta1)).astype(T) + (g * S(1.0 - beta1)).astype(T)
+        v = (v * S(beta2)).astype(T) + ((g * g).astype(T) * S(1.0 - beta2)).astype(T)
+        m_hat = m * S(1.0 / bc1)
+        v_hat = v * S(1.0 / bc2)
+        decayed = w * S(1.0 - lr * weight_decay) if weight_decay > 0.0 else w
+        update = m_hat / (np.sqrt(v_hat) + S(eps))
+        w = decayed - update * S(lr)
+    return w.astype(T), m.astype(T), v.astype(T)
+
+
+def clip_grad_norm(grads, max_norm: float, dtype=np.float32):
+    """clip_grad_norm (src/optim.rs:258-296) over a list of gradient arrays: returns
+    (norm before clipping as f32, the list of possibly rescaled gradients)."""
+    assert max_norm > 0.0, "max_norm must be positive"
+    T = np.dtype(dtype).type
+    if not grads:
+        return np.float32(0.0), []
+    grads = [np.asarray(g, dtype=dtype) for g in grads]
+    total = T(0.0)
+    with np.errstate(all="ignore"):
+        for g in grads:
+            total = T(total + (g * g).astype(T).sum(dtype=T))
+        norm = np.float32(np.sqrt(total))
+    if not np.isfinite(norm) or norm <= np.float32(max_norm):
+        return norm, grads
+    scale = max_norm / (float(norm) + 1e-6)
+    return norm, [(g * _scalar(scale, dtype)).astype(T) for g in grads]

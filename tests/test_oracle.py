@@ -365,3 +365,85 @@ def test_log_softmax_backward_finite_differences_and_closed_form():
     dr = oracle.log_softmax_bwd(np.ones_like(yr), yr)
     e = np.exp(REF_LSM_INPUT.astype(np.float64))
     assert np.abs(dr - (1 - 3 * e / e.sum(axis=1, keepdims=True))).max() < 1e-6
+
+
+# ---- AdamW step and clip_grad_norm (src/optim.rs:214-296) ----
+
+def _adam_textbook(w, grads, lr, b1=0.9, b2=0.999, eps=1e-8, wd=0.0):
+    """Loshchilov & Hutter's AdamW in float64, written from the paper's update rule
+    (division by the bias corrections, decay folded into the update), not from the oracle."""
+    w = np.asarray(w, dtype=np.float64).copy()
+    m = np.zeros_like(w)
+    v = np.zeros_like(w)
+    for t, g in enumerate(grads, start=1):
+        g = np.asarray(g, dtype=np.float64)
+        m = b1 * m + (1 - b1) * g
+        v = b2 * v + (1 - b2) * g * g
+        w = w - lr * ((m / (1 - b1 ** t)) / (np.sqrt(v / (1 - b2 ** t)) + eps) + wd * w)
+    return w
+
+
+def test_adamw_reference_unit_tests():
+    z = np.zeros(1, np.float32)
+    # test_adamw_step (src/optim.rs:417-432): x = 0, loss (x-3)^2, lr 0.1 -> the first
+    # Adam step moves by lr * sign(-g) = +0.1
+    w, m, v = oracle.adamw_step(np.float32([0.0]), np.float32([-6.0]), z, z, 1, 0.1)
+    assert abs(w[0] - 0.1) < 1e-6 and abs(m[0] + 0.6) < 1e-6 and abs(v[0] - 0.036) < 1e-6
+    # test_adamw_weight_decay (459-471): zero gradient, only the decay acts: 5 * (1 - 0.1*0.1)
+    w, m, v = oracle.adamw_step(np.float32([5.0]), z, z, z, 1, 0.1, weight_decay=0.1)
+    assert abs(w[0] - 4.95) < 1e-6 and m[0] == 0 and v[0] == 0
+    # test_adamw_loss_decreases (435-456): 20 steps on (x-3)^2
+    x, m, v, losses = np.float32([0.0]), z, z, []
+    for t in range(1, 21):
+        losses.append(float((x[0] - 3) ** 2))
+        x, m, v = oracle.adamw_step(x, 2 * (x - np.float32(3.0)), m, v, t, 0.1)
+    assert losses[-1] < 0.2 * losses[0]
+    # test_adamw_converges_quadratic (536-553): 100 steps on x^2 + y^2 from (5, -3)
+    p, m, v = np.float32([5.0, -3.0]), np.zeros(2, np.float32), np.zeros(2, np.float32)
+    for t in range(1, 101):
+        p, m, v = oracle.adamw_step(p, 2 * p, m, v, t, 0.1)
+    assert np.abs(p).max() < 0.1
+
+
+def test_adamw_matches_textbook_rule_over_many_steps():
+    rng = np.random.default_rng(11)
+    w0 = rng.standard_normal(64).astype(np.float32)
+    grads = [rng.standard_normal(64).astype(np.float32) * 0.3 for _ in range(25)]
+    w, m, v = w0, np.zeros(64, np.float32), np.zeros(64, np.float32)
+    for t, g in enumerate(grads, start=1):
+        w, m, v = oracle.adamw_step(w, g, m, v, t, 3e-3, betas=(0.9, 0.95), weight_decay=0.1)
+    want = _adam_textbook(w0, grads, 3e-3, 0.9, 0.95, 1e-8, 0.1)
+    assert np.abs(w - want).max() < 2e-6
+    # first step in closed form: w(1 - lr*wd) - lr * g / (|g| + eps)
+    w1, _, _ = oracle.adamw_step(w0, grads[0], np.zeros(64, np.float32), np.zeros(64, np.float32), 1,
+                                 0.01, weight_decay=0.5)
+    g0 = grads[0].astype(np.float64)
+    assert np.abs(w1 - (w0 * (1 - 0.005) - 0.01 * g0 / (np.abs(g0) + 1e-8))).max() < 1e-6
+
+
+def test_adamw_f16_rounds_every_op_and_every_scalar():
+    # f16 tensors: eps = 1e-8 is below half the smallest f16 subnormal and becomes 0, so a
+    # zero gradient gives 0/0 = NaN in the reference's chain; a non-zero one is finite
+    h = np.float16
+    z = np.zeros(2, h)
+    w, m, v = oracle.adamw_step(h([1.0, 1.0]), h([0.0, 0.5]), z, z, 1, 0.1, dtype=h)
+    assert w.dtype == h and np.isnan(w[0]) and abs(float(w[1]) - 0.9) < 1e-3
+    assert oracle._scalar(1e-8, h) == 0 and oracle._scalar(0.999, h) == h(0.999)
+    assert abs(oracle._powi(0.999, 1000) - 0.999 ** 1000) < 1e-14
+    assert oracle._powi(2.0, 10) == 1024.0 and oracle._powi(2.0, -2) == 0.25 and oracle._powi(3.0, 0) == 1.0
+
+
+def test_clip_grad_norm_reference_cases():
+    # test_clip_grad_norm_scales_large_gradients (src/optim.rs:556-570)
+    norm, (g,) = oracle.clip_grad_norm([np.float32([3.0, 4.0])], 1.0)
+    assert abs(norm - 5.0) < 1e-5 and abs(g[0] - 0.6) < 1e-4 and abs(g[1] - 0.8) < 1e-4
+    # below the threshold nothing changes; several tensors share one norm
+    a, b = np.float32([1.0, 2.0]), np.float32([2.0])
+    norm, (ga, gb) = oracle.clip_grad_norm([a, b], 10.0)
+    assert abs(norm - 3.0) < 1e-6 and (ga == a).all() and (gb == b).all()
+    norm, (ga, gb) = oracle.clip_grad_norm([a, b], 1.5)
+    assert abs(np.sqrt((ga ** 2).sum() + (gb ** 2).sum()) - 1.5) < 1e-5
+    # a non-finite norm is returned and nothing is rescaled
+    norm, (gi,) = oracle.clip_grad_norm([np.float32([np.inf, 1.0])], 1.0)
+    assert np.isinf(norm) and gi[1] == 1.0
+    assert oracle.clip_grad_norm([], 1.0)[0] == 0.0
