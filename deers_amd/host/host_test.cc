@@ -15,6 +15,7 @@
 
 #include "../../include/deers_rocm.h"
 #include "ops.h"
+#include "optim.h"
 
 using namespace deers_host;
 
@@ -364,6 +365,75 @@ static int run_log_softmax(const std::string& dir) {
   return 0;
 }
 
+// K optimizer steps on two parameters with injected gradients, clipped to max_norm:
+// odd steps through clip_grad_norm (rescaled copies in the store), even steps through
+// clip_grad_scale folded into the step.  Writes the norms and the final w, m, v.
+static int run_optim(const std::string& dir) {
+  check(deers_rocm_init(0));
+  int dt, n0, n1, steps;
+  double lr, wd, max_norm;
+  {
+    std::ifstream f(dir + "/case.txt");
+    if (!(f >> dt >> n0 >> n1 >> steps >> lr >> wd >> max_norm)) { std::printf("FAIL bad case.txt\n"); return 2; }
+  }
+  const DType dtype = dt == 0 ? DType::F16 : DType::F32;
+  auto load = [&](const std::string& name, int64_t n) {
+    auto bytes = read_file(dir + "/" + name);
+    if (bytes.size() != (size_t)n * size_in_bytes(dtype)) { std::printf("FAIL size of %s\n", name.c_str()); std::exit(2); }
+    return Tensor::from_host(bytes.data(), {n}, dtype);
+  };
+  Tensor p0 = load("w0.bin", n0).attach(), p1 = load("w1.bin", n1).attach();
+  Tensor frozen = load("w1.bin", n1).attach();  // a parameter that never gets a gradient
+  const TensorId id0 = p0.id();
+  AdamW opt = AdamWConfig(lr).betas(0.9, 0.95).weight_decay(wd).build({p0, p1, frozen});
+  EXPECT(opt.step_count() == 0 && !opt.state_for(p0).has_value());
+  std::vector<float> norms;
+  for (int t = 1; t <= steps; ++t) {
+    GradientStore grads;
+    Tensor g0 = load("g0_" + std::to_string(t) + ".bin", n0);
+    grads.insert(p0.id(), g0);
+    grads.insert(p1.id(), load("g1_" + std::to_string(t) + ".bin", n1));
+    if (t % 2) {
+      norms.push_back(clip_grad_norm({p0, p1, frozen}, grads, max_norm));
+      EXPECT(norms.back() <= (float)max_norm || !(*grads.get(p0.id()) == g0));  // clipped => replaced
+      opt.step_with_grads(grads);
+    } else {
+      double scale = 1.0;
+      norms.push_back(clip_grad_scale({p0, p1, frozen}, grads, max_norm, &scale));
+      EXPECT(*grads.get(p0.id()) == g0);  // untouched
+      opt.step_with_grads(grads, scale);
+    }
+  }
+  EXPECT(opt.step_count() == (size_t)steps);
+  EXPECT(p0.id() == id0 && p0.requires_grad());
+  EXPECT(!opt.state_for(frozen).has_value());
+  write_file(dir + "/norms.bin", norms.data(), norms.size() * sizeof(float));
+  dump(p0, dir + "/w0_out.bin");
+  dump(p1, dir + "/w1_out.bin");
+  auto st = opt.state_for(p0);
+  EXPECT(st.has_value());
+  if (st) {
+    dump(st->first, dir + "/m0_out.bin");
+    dump(st->second, dir + "/v0_out.bin");
+  }
+  // moments can be loaded back (checkpoint resume, src/optim.rs:156-160)
+  if (st) {
+    AdamW resumed = AdamWConfig(lr).build({p0});
+    resumed.load_state_for(p0, st->first, st->second);
+    resumed.set_step_count(opt.step_count());
+    EXPECT(resumed.state_for(p0).has_value() && resumed.step_count() == (size_t)steps);
+  }
+  bool threw = false;
+  try { GradientStore g; clip_grad_norm({p0}, g, 0.0); } catch (const std::logic_error&) { threw = true; }
+  EXPECT(threw);
+  {
+    GradientStore g;
+    EXPECT(clip_grad_norm({}, g, 1.0) == 0.0f);
+  }
+  std::printf("ok optim\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "graph";
   try {
@@ -377,10 +447,12 @@ int main(int argc, char** argv) {
       if (int rc = run_gpu(argv[2])) return rc;
     } else if (mode == "lsm" && argc > 2) {
       if (int rc = run_log_softmax(argv[2])) return rc;
+    } else if (mode == "optim" && argc > 2) {
+      if (int rc = run_optim(argv[2])) return rc;
     } else if (mode == "module" && argc > 2) {
       if (int rc = run_module(argv[2])) return rc;
     } else {
-      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | module <dir>\n");
+      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | optim <dir> | module <dir>\n");
       return 2;
     }
   } catch (const std::exception& e) {

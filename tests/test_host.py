@@ -178,3 +178,49 @@ def test_host_fused_log_softmax_matches_oracle(tmp_path, dtype, outer, inner):
     assert np.abs(yt.astype(np.float32) - want_t).max() <= tol(want_t)
     want_dxt = oracle.log_softmax_bwd(np.ones_like(want_t), yt.astype(np.float32)).T
     assert np.abs(out("dxt.bin", (outer, inner)).astype(np.float32) - want_dxt).max() <= tol(want_dxt)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,max_norm", [(np.float32, 0.75), (np.float32, 1e9), (np.float16, 0.75)])
+def test_host_adamw_and_clip_grad_norm_match_oracle(tmp_path, dtype, max_norm):
+    import oracle
+    n0, n1, steps, lr, wd = 5003, 640, 6, 3e-3, 0.1
+    w0 = synth.normal((n0,), synth.tensor_seed(61, "hostopt", "w0"), 1.0).astype(dtype)
+    w1 = synth.normal((n1,), synth.tensor_seed(61, "hostopt", "w1"), 1.0).astype(dtype)
+    w0.tofile(tmp_path / "w0.bin")
+    w1.tofile(tmp_path / "w1.bin")
+    gs = []
+    for t in range(1, steps + 1):
+        g0 = synth.normal((n0,), synth.tensor_seed(61, "hostopt", f"g0_{t}"), 0.02).astype(dtype)
+        g1 = synth.normal((n1,), synth.tensor_seed(61, "hostopt", f"g1_{t}"), 0.02).astype(dtype)
+        g0.tofile(tmp_path / f"g0_{t}.bin")
+        g1.tofile(tmp_path / f"g1_{t}.bin")
+        gs.append((g0, g1))
+    dt = 0 if dtype == np.float16 else 1
+    (tmp_path / "case.txt").write_text(f"{dt} {n0} {n1} {steps} {lr} {wd} {max_norm}\n")
+    r = _run("optim", str(tmp_path))
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ok optim" in r.stdout and "all passed" in r.stdout
+
+    norms = np.fromfile(tmp_path / "norms.bin", dtype=np.float32)
+    assert norms.shape == (steps,)
+    m0 = np.zeros(n0, dtype)
+    v0 = np.zeros(n0, dtype)
+    m1 = np.zeros(n1, dtype)
+    v1 = np.zeros(n1, dtype)
+    eps = 1e-8
+    for t, (g0, g1) in enumerate(gs, start=1):
+        want_norm = np.sqrt((g0.astype(np.float64) ** 2).sum() + (g1.astype(np.float64) ** 2).sum())
+        assert abs(norms[t - 1] - want_norm) <= 1e-6 * want_norm
+        # rescale with the norm the device computed (summation order differs from numpy's
+        # in the last bit), exactly as src/optim.rs:285-293 does; the rest is bit for bit
+        if np.isfinite(norms[t - 1]) and norms[t - 1] > np.float32(max_norm):
+            s = oracle._scalar(max_norm / (float(norms[t - 1]) + 1e-6), dtype)
+            g0, g1 = (g0 * s).astype(dtype), (g1 * s).astype(dtype)
+        w0, m0, v0 = oracle.adamw_step(w0, g0, m0, v0, t, lr, (0.9, 0.95), eps, wd, dtype=dtype)
+        w1, m1, v1 = oracle.adamw_step(w1, g1, m1, v1, t, lr, (0.9, 0.95), eps, wd, dtype=dtype)
+    if max_norm < 1:
+        assert (norms > max_norm).all()  # the case does clip
+    out = lambda name: np.fromfile(tmp_path / name, dtype=dtype)
+    for name, want in (("w0_out.bin", w0), ("w1_out.bin", w1), ("m0_out.bin", m0), ("v0_out.bin", v0)):
+        assert np.array_equal(out(name), want, equal_nan=True), name
