@@ -118,15 +118,21 @@ __global__ __launch_bounds__(kLsmThreads) void log_softmax_bwd_kernel(const T* g
 
 // ---- rows held in registers ----
 // GROUP threads own one row; a workgroup of kRegBlock threads holds kRegBlock / GROUP
-// rows.  The row is cut into 16-byte chunks at 16-byte-ALIGNED addresses (rows start at
-// any element: 50257 is odd), so that every access is a full-width, cache-line-friendly
-// dwordx4: chunk c of the row starts `head` elements before the row when the row is
-// not aligned, and the first and last chunk may hold neighbours' elements, which are
-// replaced by the reduction's neutral element after the load and never stored.
+// rows.  The row is cut into 16-byte chunks counted from the 128-byte line its first
+// element lies in (rows start at any element: 50257 is odd), so that every access is a
+// full-width dwordx4 and every wavefront access covers whole cache lines.  Chunks
+// before the row are skipped; the chunks that straddle the row's ends hold neighbours'
+// elements, which are replaced by the reduction's neutral element after the load and
+// never stored.
 // Thread t of the group holds chunks t, t + GROUP, ... (NREG of them, packed as loaded,
 // so an f16 row takes half the registers of an f32 row).
 
 constexpr int kRegBlockOf(int group) { return group < 256 ? 256 : group; }
+// Waves per SIMD to compile the forward for.  A 1024-thread group is 4 waves per SIMD;
+// with up to 8 chunks per thread two such groups fit a CU (64 VGPRs each), and the
+// loads of one overlap the stores of the other.  (The backward streams lsm between
+// its stores and does not need it; capped at 64 VGPRs it would spill.)
+constexpr int kRegWavesOf(int group, int nreg) { return group == 1024 && nreg <= 8 ? 8 : 1; }
 
 template <int GROUP>
 __device__ __forceinline__ void group_reduce_ms(float& m, float& s, float* red_m, float* red_s,
@@ -211,18 +217,22 @@ __device__ __forceinline__ void chunk_store(u32x4 c, rsrc_t r, int byte_off) {
       r, byte_off, 0, kAuxNt);
 }
 
-// Where a row lies relative to its 16-byte chunks.
+// Where a row lies relative to its chunks.  Chunk 0 starts at the 128-byte line that
+// holds the row's first element, so that every wavefront access covers whole cache
+// lines; `head` elements (up to a line's worth) precede the row in chunks that are
+// never loaded or stored.  Operands that move with the row (the output, lsm) use the
+// same head, measured back from their own row start.
 template <typename T>
 struct RowGeom {
-  const char* base;  // 16-byte-aligned address of chunk 0
-  int head;          // elements of chunk 0 that precede the row
-  int n_chunks;      // chunks that overlap the row
+  int head;      // elements between the line start and the row
+  int n_chunks;  // chunks from the line start to the row's end
   __device__ __forceinline__ RowGeom(const T* row, int inner) {
     constexpr int kEpc = 16 / sizeof(T);
-    const uintptr_t a = (uintptr_t)row;
-    base = (const char*)(a & ~(uintptr_t)15);
-    head = (int)(a & 15) / (int)sizeof(T);
+    head = (int)((uintptr_t)row & 127) / (int)sizeof(T);
     n_chunks = (head + inner + kEpc - 1) / kEpc;
+  }
+  __device__ __forceinline__ const char* base_of(const T* row) const {
+    return (const char*)(row - head);
   }
 };
 
@@ -248,7 +258,7 @@ __device__ __forceinline__ void store_inside(const float (&f)[16 / sizeof(T)], T
 }
 
 template <typename T, int GROUP, int NREG>
-__global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_fwd_reg_kernel(
+__global__ __launch_bounds__(kRegBlockOf(GROUP), kRegWavesOf(GROUP, NREG)) void log_softmax_fwd_reg_kernel(
     const T* x, T* out, int64_t outer, int inner) {
   __shared__ float red_m[16], red_s[16];
   constexpr int kRows = kRegBlockOf(GROUP) / GROUP;
@@ -256,12 +266,18 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_fwd_reg_kernel
   const int t = threadIdx.x % GROUP;
   const int64_t r = (int64_t)blockIdx.x * kRows + threadIdx.x / GROUP;
   const bool live = r < outer;  // whole groups only: GROUP == 64 when kRows > 1
-  const RowGeom<T> geo(x + (live ? r : 0) * inner, inner);
+  const T* row = x + (live ? r : 0) * inner;
+  const RowGeom<T> geo(row, inner);
   const int n_chunks = live ? geo.n_chunks : 0;  // a dead group's descriptors cover nothing
+  const int lo0 = t * kEpc - geo.head;  // row position of this thread's chunk 0, element 0
   u32x4 c[NREG];
 #pragma unroll
-  for (int u = 0; u < NREG; ++u) c[u] = chunk_load(slice_rsrc(geo.base, n_chunks, u * GROUP), t * 16);
-  const int lo0 = t * kEpc - geo.head;  // row position of this thread's chunk 0, element 0
+  for (int u = 0; u < NREG; ++u) {
+    c[u] = u32x4{0u, 0u, 0u, 0u};
+    // chunks wholly before the row (slice 0 only) are not read
+    if (u > 0 || lo0 + kEpc > 0)
+      c[u] = chunk_load(slice_rsrc(geo.base_of(row), n_chunks, u * GROUP), t * 16);
+  }
 #pragma unroll
   for (int u = 0; u < NREG; ++u) {
     const int lo = lo0 + u * GROUP * kEpc;
@@ -290,7 +306,7 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_fwd_reg_kernel
   if (!live) return;
   const float lse = __logf(s) + m;
   T* orow = out + r * inner;
-  const RowGeom<T> ogeo(orow, inner);  // same head as the input row: checked by the launcher
+  const char* obase = geo.base_of(orow);  // 16-byte aligned: checked by the launcher
 #pragma unroll
   for (int u = 0; u < NREG; ++u) {
     const int lo = lo0 + u * GROUP * kEpc;
@@ -300,7 +316,7 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_fwd_reg_kernel
 #pragma unroll
     for (int e = 0; e < kEpc; ++e) f[e] -= lse;
     if (lo >= 0 && lo + kEpc <= inner)
-      chunk_store(pack<T>(f), slice_rsrc(ogeo.base, n_chunks, u * GROUP), t * 16);
+      chunk_store(pack<T>(f), slice_rsrc(obase, n_chunks, u * GROUP), t * 16);
     else
       store_inside<T>(f, orow, lo, inner);
   }
@@ -315,12 +331,17 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_bwd_reg_kernel
   const int t = threadIdx.x % GROUP;
   const int64_t r = (int64_t)blockIdx.x * kRows + threadIdx.x / GROUP;
   const bool live = r < outer;
-  const RowGeom<T> geo(grad + (live ? r : 0) * inner, inner);
+  const T* grow = grad + (live ? r : 0) * inner;
+  const RowGeom<T> geo(grow, inner);
   const int n_chunks = live ? geo.n_chunks : 0;
+  const int lo0 = t * kEpc - geo.head;
   u32x4 c[NREG];
 #pragma unroll
-  for (int u = 0; u < NREG; ++u) c[u] = chunk_load(slice_rsrc(geo.base, n_chunks, u * GROUP), t * 16);
-  const int lo0 = t * kEpc - geo.head;
+  for (int u = 0; u < NREG; ++u) {
+    c[u] = u32x4{0u, 0u, 0u, 0u};
+    if (u > 0 || lo0 + kEpc > 0)
+      c[u] = chunk_load(slice_rsrc(geo.base_of(grow), n_chunks, u * GROUP), t * 16);
+  }
 #pragma unroll
   for (int u = 0; u < NREG; ++u) {
     const int lo = lo0 + u * GROUP * kEpc;
@@ -337,15 +358,20 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_bwd_reg_kernel
   s = group_reduce_sum<GROUP>(s, red, t);
   if (!live) return;
   T* orow = out + r * inner;
-  const RowGeom<T> lgeo(lsm + r * inner, inner), ogeo(orow, inner);  // same head: see launcher
+  // 16-byte aligned like the gradient's chunks: checked by the launcher
+  const char* lbase = geo.base_of(lsm + r * inner);
+  const char* obase = geo.base_of(orow);
   constexpr int kBatch = NREG < 4 ? NREG : 4;  // lsm chunks in flight per thread
 #pragma unroll
   for (int u0 = 0; u0 < NREG; u0 += kBatch) {
     u32x4 lc[kBatch];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u)
-      if (u0 + u < NREG)
-        lc[u] = chunk_load(slice_rsrc(lgeo.base, n_chunks, (u0 + u) * GROUP), t * 16);
+      if (u0 + u < NREG) {
+        lc[u] = u32x4{0u, 0u, 0u, 0u};
+        if (u0 + u > 0 || lo0 + kEpc > 0)
+          lc[u] = chunk_load(slice_rsrc(lbase, n_chunks, (u0 + u) * GROUP), t * 16);
+      }
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       if (u0 + u >= NREG) continue;
@@ -358,7 +384,7 @@ __global__ __launch_bounds__(kRegBlockOf(GROUP)) void log_softmax_bwd_reg_kernel
 #pragma unroll
       for (int e = 0; e < kEpc; ++e) f[e] -= __expf(l[e]) * s;
       if (lo >= 0 && lo + kEpc <= inner)
-        chunk_store(pack<T>(f), slice_rsrc(ogeo.base, n_chunks, (u0 + u) * GROUP), t * 16);
+        chunk_store(pack<T>(f), slice_rsrc(obase, n_chunks, (u0 + u) * GROUP), t * 16);
       else
         store_inside<T>(f, orow, lo, inner);
     }
@@ -381,14 +407,16 @@ void launch_bwd_reg(const T* g, const T* l, T* out, int64_t outer, int inner, hi
                      dim3(kBlock), 0, stream, g, l, out, outer, inner);
 }
 
-// Chunks a row can overlap at worst.  When the first row is 16-byte aligned and the row
-// pitch is a multiple of 16 bytes every row starts a chunk; otherwise some row starts
-// on the last element of one.
+// Chunks from a row's line start to its end, at worst over all rows.  Row r starts
+// (first + r * pitch) mod 128 bytes into its line; those offsets step by gcd(pitch, 128).
 template <typename T>
 int64_t worst_chunks(const T* first_row, int64_t inner) {
   constexpr int kEpc = 16 / sizeof(T);
-  const bool aligned = ((uintptr_t)first_row & 15) == 0 && inner % kEpc == 0;
-  return ((aligned ? 0 : kEpc - 1) + inner + kEpc - 1) / kEpc;
+  const int64_t pitch = inner * (int64_t)sizeof(T);
+  int64_t g = 128;
+  while (pitch % g) g /= 2;
+  const int64_t max_head_bytes = (int64_t)((uintptr_t)first_row % (uintptr_t)g) + 128 - g;
+  return (max_head_bytes / (int64_t)sizeof(T) + inner + kEpc - 1) / kEpc;
 }
 inline bool same_phase(const void* a, const void* b) {
   return (((uintptr_t)a ^ (uintptr_t)b) & 15) == 0;
@@ -408,6 +436,8 @@ void dispatch_fwd(const T* x, T* out, int64_t outer, int64_t inner, hipStream_t 
   else if (n <= 64 * 1) launch_fwd_reg<T, 64, 1>(x, out, outer, (int)inner, stream);
   else if (n <= 64 * 4) launch_fwd_reg<T, 64, 4>(x, out, outer, (int)inner, stream);
   else if (n <= 256 * 4) launch_fwd_reg<T, 256, 4>(x, out, outer, (int)inner, stream);
+  else if (n <= 256 * 8) launch_fwd_reg<T, 256, 8>(x, out, outer, (int)inner, stream);
+  else if (n <= 256 * 13) launch_fwd_reg<T, 256, 13>(x, out, outer, (int)inner, stream);
   else if (n <= 1024 * 4) launch_fwd_reg<T, 1024, 4>(x, out, outer, (int)inner, stream);
   else if (n <= 1024 * 8) launch_fwd_reg<T, 1024, 8>(x, out, outer, (int)inner, stream);
   else if constexpr (sizeof(T) == 4) {
@@ -426,6 +456,8 @@ void dispatch_bwd(const T* g, const T* l, T* out, int64_t outer, int64_t inner,
   else if (n <= 64 * 1) launch_bwd_reg<T, 64, 1>(g, l, out, outer, (int)inner, stream);
   else if (n <= 64 * 4) launch_bwd_reg<T, 64, 4>(g, l, out, outer, (int)inner, stream);
   else if (n <= 256 * 4) launch_bwd_reg<T, 256, 4>(g, l, out, outer, (int)inner, stream);
+  else if (n <= 256 * 8) launch_bwd_reg<T, 256, 8>(g, l, out, outer, (int)inner, stream);
+  else if (n <= 256 * 13) launch_bwd_reg<T, 256, 13>(g, l, out, outer, (int)inner, stream);
   else if (n <= 1024 * 4) launch_bwd_reg<T, 1024, 4>(g, l, out, outer, (int)inner, stream);
   else if (n <= 1024 * 8) launch_bwd_reg<T, 1024, 8>(g, l, out, outer, (int)inner, stream);
   else if constexpr (sizeof(T) == 4) {
