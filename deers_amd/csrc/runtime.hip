@@ -38,6 +38,21 @@ void launch_log_softmax_fwd(int dtype_f16, const void* x, void* out, int64_t out
                             hipStream_t stream);
 void launch_log_softmax_bwd(int dtype_f16, const void* grad, const void* lsm, void* out,
                             int64_t outer, int64_t inner, hipStream_t stream);
+int index_add_max_indices();
+void launch_index_select(int dtype_f16, const void* table, const int64_t* idx, void* out,
+                         int64_t n_rows, int64_t n_idx, int width, int* flag, hipStream_t stream);
+void launch_index_add(int dtype_f16, const void* src, const int64_t* idx, void* dst, int64_t n_rows,
+                      int n_idx, int width, int* flag, hipStream_t stream);
+void launch_rms_norm(int dtype_f16, const void* x, const void* dy, void* out, int64_t outer, int width,
+                     float eps, int bwd, hipStream_t stream);
+void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int64_t n, int bwd,
+                    hipStream_t stream);
+void launch_cross_entropy_fwd(int dtype_f16, const void* logits, const int64_t* targets, float* row_lse,
+                              float* row_loss, float* loss, int64_t n_rows, int width, int* flag,
+                              hipStream_t stream);
+void launch_cross_entropy_bwd(int dtype_f16, const void* logits, const int64_t* targets,
+                              const float* row_lse, const float* upstream, void* dlogits,
+                              int64_t n_rows, int width, hipStream_t stream);
 int sumsq_partial_count();
 void launch_adamw(int dtype_f16, void* w, const void* g, void* m, void* v, int64_t n, double lr,
                   double beta1, double beta2, double eps, double weight_decay, int step,
@@ -64,6 +79,10 @@ struct Runtime {
   int* bwd_ready = nullptr;
   size_t bwd_ready_len = 0;
   int bwd_epoch = 0;
+  // sticky "an index was out of range" flag that index kernels raise; read back by the
+  // next synchronising call after one of them has been launched
+  int* index_flag = nullptr;
+  bool index_flag_armed = false;
 };
 
 Runtime g_rt;
@@ -251,11 +270,36 @@ int deers_rocm_init(int ordinal) {
   return DEERS_ROCM_OK;
 }
 
+// Device memory for the index flag, created by the first call that needs it.
+int index_flag(int** out) {
+  if (!g_rt.index_flag) {
+    HIP_TRY(hipMalloc((void**)&g_rt.index_flag, sizeof(int)));
+    HIP_TRY(hipMemsetAsync(g_rt.index_flag, 0, sizeof(int), g_rt.stream));
+  }
+  g_rt.index_flag_armed = true;
+  *out = g_rt.index_flag;
+  return DEERS_ROCM_OK;
+}
+
+// After the stream has drained: reports (once) an out-of-range index seen by any index
+// kernel since the last check.  Kernels skip such an index, they never follow it.
+int check_index_flag() {
+  if (!g_rt.index_flag_armed) return DEERS_ROCM_OK;
+  g_rt.index_flag_armed = false;
+  int seen = 0;
+  HIP_TRY(hipMemcpy(&seen, g_rt.index_flag, sizeof(int), hipMemcpyDeviceToHost));
+  if (!seen) return DEERS_ROCM_OK;
+  HIP_TRY(hipMemset(g_rt.index_flag, 0, sizeof(int)));
+  return fail(DEERS_ROCM_ERR_INDEX,
+              "an index was out of bounds in an index_select / index_add / cross_entropy call "
+              "since the last synchronisation (such rows were skipped)");
+}
+
 int deers_rocm_sync(void) {
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   HIP_TRY(hipStreamSynchronize(g_rt.stream));
-  return DEERS_ROCM_OK;
+  return check_index_flag();
 }
 
 const char* deers_rocm_last_error(void) { return t_err.c_str(); }
@@ -308,7 +352,7 @@ int deers_rocm_dtoh(void* dst_host, const void* src_device, size_t bytes) {
   if (!dst_host || !src_device) return fail(DEERS_ROCM_ERR_ARG, "dtoh: null pointer");
   HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, g_rt.stream));
   HIP_TRY(hipStreamSynchronize(g_rt.stream));
-  return DEERS_ROCM_OK;
+  return check_index_flag();
 }
 
 int deers_rocm_dtod(void* dst_device, const void* src_device, size_t bytes) {
@@ -636,6 +680,133 @@ int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, voi
   if (outer == 0) return DEERS_ROCM_OK;
   if (!grad || !lsm || !out) return fail(DEERS_ROCM_ERR_ARG, "log_softmax_bwd: null pointer");
   deers::launch_log_softmax_bwd(dtype == DEERS_ROCM_F16, grad, lsm, out, outer, inner, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- the other ops of a GPT training step ----
+
+static int rows_check(const char* what, int dtype, int64_t outer, int64_t inner) {
+  if (int rc = check_dtype(dtype)) return rc;
+  if (outer < 0 || inner < 1 || inner > INT32_MAX || outer > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "%s: need 0 <= rows < 2^31 of 1 <= width < 2^31 elements", what);
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_index_select(int dtype, const void* table, const int64_t* indices, void* out,
+                            int64_t n_rows, int64_t n_indices, int64_t width) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("index_select", dtype, n_indices, width)) return rc;
+  if (n_rows < 0) return fail(DEERS_ROCM_ERR_ARG, "index_select: negative table size");
+  if (n_indices == 0) return DEERS_ROCM_OK;
+  if (!table || !indices || !out) return fail(DEERS_ROCM_ERR_ARG, "index_select: null pointer");
+  int* flag = nullptr;
+  if (int rc = index_flag(&flag)) return rc;
+  deers::launch_index_select(dtype == DEERS_ROCM_F16, table, indices, out, n_rows, n_indices,
+                             (int)width, flag, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, void* dst,
+                         int64_t n_rows, int64_t n_indices, int64_t width) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("index_add", dtype, n_indices, width)) return rc;
+  if (n_rows < 0) return fail(DEERS_ROCM_ERR_ARG, "index_add: negative destination size");
+  if (n_indices > deers::index_add_max_indices())
+    return fail(DEERS_ROCM_ERR_ARG, "index_add: at most %d indices per call (got %lld)",
+                deers::index_add_max_indices(), (long long)n_indices);
+  if (n_indices == 0) return DEERS_ROCM_OK;
+  if (!src || !indices || !dst) return fail(DEERS_ROCM_ERR_ARG, "index_add: null pointer");
+  int* flag = nullptr;
+  if (int rc = index_flag(&flag)) return rc;
+  deers::launch_index_add(dtype == DEERS_ROCM_F16, src, indices, dst, n_rows, (int)n_indices,
+                          (int)width, flag, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_rms_norm_fwd(int dtype, const void* x, void* y, int64_t outer, int64_t inner,
+                            double eps) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("rms_norm_fwd", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !y) return fail(DEERS_ROCM_ERR_ARG, "rms_norm_fwd: null pointer");
+  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, nullptr, y, outer, (int)inner, (float)eps, 0,
+                         g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_rms_norm_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t outer,
+                            int64_t inner, double eps) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("rms_norm_bwd", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !dy || !dx) return fail(DEERS_ROCM_ERR_ARG, "rms_norm_bwd: null pointer");
+  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, dy, dx, outer, (int)inner, (float)eps, 1,
+                         g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_relu_sq_fwd(int dtype, const void* x, void* y, int64_t n) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "relu_sq_fwd: negative element count");
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!x || !y) return fail(DEERS_ROCM_ERR_ARG, "relu_sq_fwd: null pointer");
+  deers::launch_relu_sq(dtype == DEERS_ROCM_F16, x, nullptr, y, n, 0, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_relu_sq_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t n) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "relu_sq_bwd: negative element count");
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!x || !dy || !dx) return fail(DEERS_ROCM_ERR_ARG, "relu_sq_bwd: null pointer");
+  deers::launch_relu_sq(dtype == DEERS_ROCM_F16, x, dy, dx, n, 1, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_cross_entropy_fwd(int dtype, const void* logits, const int64_t* targets,
+                                 float* row_lse, float* loss, int64_t n_rows, int64_t n_classes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("cross_entropy_fwd", dtype, n_rows, n_classes)) return rc;
+  if (n_rows < 1) return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_fwd: needs at least one row");
+  if (!logits || !targets || !row_lse || !loss)
+    return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_fwd: null pointer");
+  void* ws = nullptr;  // per-row losses
+  if (int rc = workspace((size_t)n_rows * sizeof(float), &ws)) return rc;
+  int* flag = nullptr;
+  if (int rc = index_flag(&flag)) return rc;
+  deers::launch_cross_entropy_fwd(dtype == DEERS_ROCM_F16, logits, targets, row_lse, (float*)ws, loss,
+                                  n_rows, (int)n_classes, flag, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_cross_entropy_bwd(int dtype, const void* logits, const int64_t* targets,
+                                 const float* row_lse, const float* upstream, void* dlogits,
+                                 int64_t n_rows, int64_t n_classes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("cross_entropy_bwd", dtype, n_rows, n_classes)) return rc;
+  if (n_rows < 1) return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_bwd: needs at least one row");
+  if (!logits || !targets || !row_lse || !dlogits)
+    return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_bwd: null pointer");
+  deers::launch_cross_entropy_bwd(dtype == DEERS_ROCM_F16, logits, targets, row_lse, upstream, dlogits,
+                                  n_rows, (int)n_classes, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -217,6 +217,48 @@ def log_softmax_bwd_raw(dtype, grad, lsm, out, outer, inner):
                                              ctypes.c_int64(outer), ctypes.c_int64(inner)))
 
 
+def index_select_raw(dtype, table, indices, out, n_rows, n_indices, width):
+    _check(load().deers_rocm_index_select(ctypes.c_int(dtype_code(dtype)), table, indices, out,
+                                          ctypes.c_int64(n_rows), ctypes.c_int64(n_indices),
+                                          ctypes.c_int64(width)))
+
+
+def index_add_raw(dtype, src, indices, dst, n_rows, n_indices, width):
+    _check(load().deers_rocm_index_add(ctypes.c_int(dtype_code(dtype)), src, indices, dst,
+                                       ctypes.c_int64(n_rows), ctypes.c_int64(n_indices),
+                                       ctypes.c_int64(width)))
+
+
+def rms_norm_fwd_raw(dtype, x, y, outer, inner, eps):
+    _check(load().deers_rocm_rms_norm_fwd(ctypes.c_int(dtype_code(dtype)), x, y, ctypes.c_int64(outer),
+                                          ctypes.c_int64(inner), ctypes.c_double(eps)))
+
+
+def rms_norm_bwd_raw(dtype, x, dy, dx, outer, inner, eps):
+    _check(load().deers_rocm_rms_norm_bwd(ctypes.c_int(dtype_code(dtype)), x, dy, dx,
+                                          ctypes.c_int64(outer), ctypes.c_int64(inner),
+                                          ctypes.c_double(eps)))
+
+
+def relu_sq_fwd_raw(dtype, x, y, n):
+    _check(load().deers_rocm_relu_sq_fwd(ctypes.c_int(dtype_code(dtype)), x, y, ctypes.c_int64(n)))
+
+
+def relu_sq_bwd_raw(dtype, x, dy, dx, n):
+    _check(load().deers_rocm_relu_sq_bwd(ctypes.c_int(dtype_code(dtype)), x, dy, dx, ctypes.c_int64(n)))
+
+
+def cross_entropy_fwd_raw(dtype, logits, targets, row_lse, loss, n_rows, n_classes):
+    _check(load().deers_rocm_cross_entropy_fwd(ctypes.c_int(dtype_code(dtype)), logits, targets, row_lse,
+                                               loss, ctypes.c_int64(n_rows), ctypes.c_int64(n_classes)))
+
+
+def cross_entropy_bwd_raw(dtype, logits, targets, row_lse, upstream, dlogits, n_rows, n_classes):
+    _check(load().deers_rocm_cross_entropy_bwd(ctypes.c_int(dtype_code(dtype)), logits, targets, row_lse,
+                                               upstream, dlogits, ctypes.c_int64(n_rows),
+                                               ctypes.c_int64(n_classes)))
+
+
 def adamw_step_raw(dtype, w, grad, m, v, n, lr, beta1, beta2, eps, weight_decay, step,
                    grad_scale=1.0):
     _check(load().deers_rocm_adamw_step(

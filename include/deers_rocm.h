@@ -48,6 +48,8 @@ extern "C" {
 #define DEERS_ROCM_ERR_ARG 2         /* null pointer, bad dtype, unsupported size */
 #define DEERS_ROCM_ERR_LAYOUT 3      /* strides the kernels cannot consume */
 #define DEERS_ROCM_ERR_NOT_INIT 4    /* deers_rocm_init has not succeeded */
+#define DEERS_ROCM_ERR_INDEX 5       /* an index tensor held a value out of range; reported by
+                                        the next deers_rocm_sync / _dtoh (Error::IndexOutOfBounds) */
 
 /* ---- runtime ------------------------------------------------------------ */
 
@@ -202,6 +204,49 @@ int deers_rocm_log_softmax_fwd(int dtype, const void* x, void* out, int64_t oute
 /* out = grad - exp(lsm) * rowsum(grad), lsm = the forward's output. */
 int deers_rocm_log_softmax_bwd(int dtype, const void* grad, const void* lsm, void* out,
                                int64_t outer, int64_t inner);
+
+/* ---- the other ops of a GPT training step -------------------------------------------
+ * Indices and targets are int64 in device memory, as DType::I64 tensors are in the
+ * reference.  A value out of range cannot be seen by the host before the launch: the
+ * kernels skip it (they never follow it) and raise a flag that the next
+ * deers_rocm_sync / deers_rocm_dtoh returns as DEERS_ROCM_ERR_INDEX, the counterpart of
+ * Error::IndexOutOfBounds (src/storage/cpu.rs:591-597). */
+
+/* out[i, :] = table[indices[i], :]: BackendStorage::index_select along dim 0
+ * (src/storage.rs:263-270; CPU src/storage/cpu.rs:555-610), the embedding lookup of
+ * src/nn.rs:216-224.  table [n_rows, width], out [n_indices, width], compact. */
+int deers_rocm_index_select(int dtype, const void* table, const int64_t* indices, void* out,
+                            int64_t n_rows, int64_t n_indices, int64_t width);
+/* dst[indices[i], :] += src[i, :] for i ascending: BackendStorage::index_add along dim 0
+ * (src/storage.rs:272-280; CPU src/storage/cpu.rs:612-660, 954-975), the backward of
+ * index_select (src/ops.rs:1429-1447).  dst [n_rows, width] is accumulated into (zero
+ * it first for the reference's semantics); additions happen in the reference's order,
+ * so the result is the same bits and reproducible.  At most 2^19 indices per call. */
+int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, void* dst,
+                         int64_t n_rows, int64_t n_indices, int64_t width);
+/* y = x * (mean(x^2 over the last axis) + eps)^-0.5: RMSNorm::forward (src/nn.rs:244-251)
+ * in one pass over compact [outer, inner]; and its backward
+ * dx = inv * dy - x * inv^3 * sum(dy * x) / inner from x and dy. */
+int deers_rocm_rms_norm_fwd(int dtype, const void* x, void* y, int64_t outer, int64_t inner,
+                            double eps);
+int deers_rocm_rms_norm_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t outer,
+                            int64_t inner, double eps);
+/* y = relu(x)^2, the MLP activation `y.relu(); &y * &y` (src/models/gpt.rs:196-197), and
+ * its backward dx = dy * 2 * relu(x). */
+int deers_rocm_relu_sq_fwd(int dtype, const void* x, void* y, int64_t n);
+int deers_rocm_relu_sq_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t n);
+/* loss::cross_entropy (src/loss.rs:11-24): *loss (a float in device memory) =
+ * -mean_i log_softmax(logits)[i, targets[i]] over compact [n_rows, n_classes] logits,
+ * without writing the log-probabilities; row_lse [n_rows] (f32, device) receives each
+ * row's ln sum exp for the backward. */
+int deers_rocm_cross_entropy_fwd(int dtype, const void* logits, const int64_t* targets,
+                                 float* row_lse, float* loss, int64_t n_rows, int64_t n_classes);
+/* dlogits = (softmax(logits) - onehot(targets)) * upstream / n_rows, from the logits and
+ * the forward's row_lse; `upstream` is the gradient of the scalar loss in device memory
+ * (NULL = 1). */
+int deers_rocm_cross_entropy_bwd(int dtype, const void* logits, const int64_t* targets,
+                                 const float* row_lse, const float* upstream, void* dlogits,
+                                 int64_t n_rows, int64_t n_classes);
 
 /* ---- optimizer step ---------------------------------------------------------------
  * One AdamW update of one parameter tensor in place, the body of the loop in

@@ -318,3 +318,93 @@ def clip_grad_norm(grads, max_norm: float, dtype=np.float32):
         return norm, grads
     scale = max_norm / (float(norm) + 1e-6)
     return norm, [(g * _scalar(scale, dtype)).astype(T) for g in grads]
+
+
+# ---- the other ops of a GPT training step (numpy restatements) ----
+
+def index_select(table: np.ndarray, indices: np.ndarray) -> np.ndarray:
+    """index_select along dim 0 (src/storage/cpu.rs:555-610, 936-952): rows of `table`
+    picked by `indices`; an index out of range is an error there and here."""
+    indices = np.asarray(indices, dtype=np.int64)
+    if indices.size and (indices.min() < 0 or indices.max() >= table.shape[0]):
+        raise IndexError("index_select: index out of bounds")
+    return np.ascontiguousarray(table[indices])
+
+
+def index_add(n_rows: int, src: np.ndarray, indices: np.ndarray) -> np.ndarray:
+    """index_add along dim 0 into zeros [n_rows, width] (src/storage/cpu.rs:612-660,
+    954-975): out[indices[i]] += src[i] for i ascending, each `+=` in the storage type."""
+    indices = np.asarray(indices, dtype=np.int64)
+    if indices.size and (indices.min() < 0 or indices.max() >= n_rows):
+        raise IndexError("index_add: index out of bounds")
+    out = np.zeros((n_rows,) + src.shape[1:], dtype=src.dtype)
+    for i, r in enumerate(indices):  # the reference's loop order
+        out[r] = out[r] + src[i]
+    return out
+
+
+def rms_norm_fwd(x: np.ndarray, eps: float, dtype=np.float32) -> np.ndarray:
+    """RMSNorm::forward (src/nn.rs:244-251) as its chain of ops in `dtype`:
+    mean_sq = sum(x*x, last) * (1/n); inv = (mean_sq + eps)^-0.5; y = x * inv."""
+    T = np.dtype(dtype).type
+    x = np.asarray(x, dtype=dtype)
+    n = x.shape[-1]
+    sq = (x * x).astype(T)
+    mean_sq = (sq.sum(axis=-1, keepdims=True, dtype=T) * _scalar_any(1.0 / n, dtype)).astype(T)
+    inv = np.power((mean_sq + _scalar_any(eps, dtype)).astype(T), T(-0.5)).astype(T)
+    return (x * inv).astype(T)
+
+
+def rms_norm_bwd(x: np.ndarray, dy: np.ndarray, eps: float, dtype=np.float32) -> np.ndarray:
+    """Gradient of rms_norm_fwd w.r.t. x, what the reference's autograd yields through
+    mul / scalar_powf / scalar_add / mean / mul (src/ops.rs): with inv as above,
+    dx = dy*inv - x * inv^3 * sum(dy*x, last) / n."""
+    T = np.dtype(dtype).type
+    x = np.asarray(x, dtype=dtype)
+    dy = np.asarray(dy, dtype=dtype)
+    n = x.shape[-1]
+    inv = np.power((x * x).sum(axis=-1, keepdims=True, dtype=T) / T(n) + T(eps), T(-0.5))
+    dot = (dy * x).sum(axis=-1, keepdims=True, dtype=T)
+    return (dy * inv - x * (inv ** 3) * dot / T(n)).astype(T)
+
+
+def _scalar_any(x: float, dtype):
+    """Like _scalar, but passes float64 through for finite-difference checks."""
+    return np.float64(x) if np.dtype(dtype) == np.float64 else _scalar(x, dtype)
+
+
+def relu_sq_fwd(x: np.ndarray) -> np.ndarray:
+    """`y.relu(); &y * &y` (src/models/gpt.rs:196-197; Relu at src/storage.rs:77-88)."""
+    r = np.maximum(x, x.dtype.type(0))
+    return (r * r).astype(x.dtype)
+
+
+def relu_sq_bwd(x: np.ndarray, dy: np.ndarray) -> np.ndarray:
+    """Backward of relu_sq_fwd through EWiseMul (both operands are r = relu(x): the two
+    contributions dy*r are accumulated) and Relu (mask x > 0, src/storage.rs:90-102)."""
+    r = np.maximum(x, x.dtype.type(0))
+    g = (dy * r).astype(x.dtype)
+    return ((g + g) * (x > 0)).astype(x.dtype)
+
+
+def cross_entropy_fwd(logits: np.ndarray, targets: np.ndarray, dtype=np.float32):
+    """loss::cross_entropy (src/loss.rs:11-24): log_softmax(1), gather the target column,
+    sum, times -1/N.  Returns the scalar loss in `dtype`."""
+    T = np.dtype(dtype).type
+    lsm = log_softmax_fwd(logits, dtype=dtype)
+    targets = np.asarray(targets, dtype=np.int64)
+    n = lsm.shape[0]
+    picked = lsm[np.arange(n), targets]
+    return T(picked.sum(dtype=T) * _scalar_any(-1.0 / n, dtype))
+
+
+def cross_entropy_bwd(logits: np.ndarray, targets: np.ndarray, upstream: float = 1.0,
+                      dtype=np.float32) -> np.ndarray:
+    """Gradient of cross_entropy_fwd w.r.t. the logits through ScalarMul, Sum, Gather
+    (scatter of the upstream gradient into zeros) and log_softmax_bwd."""
+    T = np.dtype(dtype).type
+    lsm = log_softmax_fwd(logits, dtype=dtype)
+    n = lsm.shape[0]
+    g = np.zeros_like(lsm)
+    g[np.arange(n), np.asarray(targets, dtype=np.int64)] = T(upstream) * _scalar_any(-1.0 / n, dtype)
+    return log_softmax_bwd(g, lsm, dtype=dtype)

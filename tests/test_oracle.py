@@ -447,3 +447,87 @@ def test_clip_grad_norm_reference_cases():
     norm, (gi,) = oracle.clip_grad_norm([np.float32([np.inf, 1.0])], 1.0)
     assert np.isinf(norm) and gi[1] == 1.0
     assert oracle.clip_grad_norm([], 1.0)[0] == 0.0
+
+
+# ---- embedding, RMSNorm, relu^2, cross-entropy (src/nn.rs, src/models/gpt.rs, src/loss.rs) ----
+
+def test_index_select_and_add_reference_literals():
+    # tests/tensor.rs:2290-2320 and 2359-2385
+    data = np.float32([10, 11, 12, 20, 21, 22, 30, 31, 32, 40, 41, 42]).reshape(4, 3)
+    assert (oracle.index_select(data, [2, 0, 3]) == data[[2, 0, 3]]).all()
+    assert (oracle.index_select(data, [2, 0, 3])[0] == [30, 31, 32]).all()
+    grad = oracle.index_add(4, np.ones((3, 3), np.float32), [2, 0, 2])
+    assert (grad.ravel() == np.float32([1, 1, 1, 0, 0, 0, 2, 2, 2, 0, 0, 0])).all()
+    with pytest.raises(IndexError):
+        oracle.index_select(data, [4])
+    with pytest.raises(IndexError):
+        oracle.index_add(4, np.ones((1, 3), np.float32), [-1])
+    # accumulation order is ascending position: visible in f16, where addition is not associative
+    src = np.float16([[2048.0], [1.0], [1.0]])
+    assert oracle.index_add(1, src, [0, 0, 0])[0, 0] == np.float16(2048.0)      # (2048+1)+1 = 2048
+    assert oracle.index_add(1, src[::-1].copy(), [0, 0, 0])[0, 0] == np.float16(2050.0)  # (1+1)+2048
+
+
+def test_rms_norm_reference_case_library_and_differences():
+    import torch
+    # tests/nn.rs:171-185: [1,2,3] / sqrt(14/3)
+    y = oracle.rms_norm_fwd(np.float32([[1, 2, 3]]), 1e-5)
+    assert np.abs(y - np.float32([1, 2, 3]) / np.sqrt(14.0 / 3.0)).max() < 1e-4
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((5, 48)).astype(np.float32)
+    dy = rng.standard_normal((5, 48)).astype(np.float32)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    ty = torch.nn.functional.rms_norm(tx, (48,), eps=1e-5)
+    ty.backward(torch.tensor(dy, dtype=torch.float64))
+    assert np.abs(oracle.rms_norm_fwd(x, 1e-5) - ty.detach().numpy()).max() < 1e-6
+    assert np.abs(oracle.rms_norm_bwd(x, dy, 1e-5) - tx.grad.numpy()).max() < 1e-5
+    # every output row has mean square 1 (up to eps); the gradient is orthogonal to x
+    assert np.abs((oracle.rms_norm_fwd(x, 0.0).astype(np.float64) ** 2).mean(axis=1) - 1).max() < 1e-6
+    d64 = oracle.rms_norm_bwd(x.astype(np.float64), dy.astype(np.float64), 0.0, dtype=np.float64)
+    assert np.abs((d64 * x).sum(axis=1)).max() < 1e-12
+    # central differences of the forward
+    x64, h = x.astype(np.float64), 1e-6
+    d = oracle.rms_norm_bwd(x64, dy.astype(np.float64), 1e-5, dtype=np.float64)
+    for (i, j) in [(0, 0), (3, 17), (4, 47)]:
+        xp, xm = x64.copy(), x64.copy()
+        xp[i, j] += h
+        xm[i, j] -= h
+        fd = ((oracle.rms_norm_fwd(xp, 1e-5, dtype=np.float64) - oracle.rms_norm_fwd(xm, 1e-5, dtype=np.float64)) * dy).sum() / (2 * h)
+        assert abs(fd - d[i, j]) < 1e-6
+
+
+def test_relu_sq_closed_forms():
+    x = np.float32([-2.0, -0.0, 0.0, 0.5, 3.0])
+    dy = np.float32([1.0, 1.0, 1.0, 2.0, -1.0])
+    assert (oracle.relu_sq_fwd(x) == np.float32([0, 0, 0, 0.25, 9.0])).all()
+    assert (oracle.relu_sq_bwd(x, dy) == np.float32([0, 0, 0, 2.0, -6.0])).all()
+    xh = np.float16([0.1, 1.7, -3.0])
+    assert oracle.relu_sq_fwd(xh).dtype == np.float16
+    assert (oracle.relu_sq_fwd(xh) == (np.maximum(xh, 0) * np.maximum(xh, 0))).all()
+
+
+def test_cross_entropy_reference_cases_and_library():
+    import torch
+    # log_softmax([1,2,3]) = [-2.4076, -1.4076, -0.4076] (the literals of src/loss.rs:34-36):
+    # targets 2 and 0 on two such rows give (0.4076 + 2.4076) / 2
+    row = np.float32([[1, 2, 3], [1, 2, 3]])
+    assert abs(float(oracle.cross_entropy_fwd(row, [2, 0])) - 1.4076) < 1e-4
+    assert abs(float(oracle.cross_entropy_fwd(np.zeros((3, 10), np.float32), [1, 5, 9])) - math.log(10)) < 1e-6
+    # src/loss.rs:66-86: gradient rows sum to zero
+    logits = np.float32([[1, 2, 3], [1, -1, 0]])
+    g = oracle.cross_entropy_bwd(logits, [2, 0])
+    assert np.abs(g.sum(axis=1)).max() < 1e-6
+    # library: torch's cross_entropy and autograd in f64
+    rng = np.random.default_rng(22)
+    x = (rng.standard_normal((7, 33)) * 3).astype(np.float32)
+    t = rng.integers(0, 33, 7)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tl = torch.nn.functional.cross_entropy(tx, torch.tensor(t))
+    (tl * 0.7).backward()
+    assert abs(float(oracle.cross_entropy_fwd(x, t)) - float(tl)) < 1e-6
+    assert np.abs(oracle.cross_entropy_bwd(x, t, upstream=0.7) - tx.grad.numpy()).max() < 1e-7
+    # closed form: (softmax - onehot) / N
+    p = np.exp(x.astype(np.float64))
+    p /= p.sum(axis=1, keepdims=True)
+    p[np.arange(7), t] -= 1
+    assert np.abs(oracle.cross_entropy_bwd(x, t) - p / 7).max() < 1e-7
