@@ -1,0 +1,124 @@
+#include "gpt.h"
+
+#include <cmath>
+#include <random>
+
+namespace deers_host {
+
+Embedding::Embedding(Tensor weight) : weight_(std::move(weight)) {
+  if (weight_.layout().ndim() != 2) throw std::logic_error("embedding weight must be [vocab, hidden]");
+}
+
+Tensor Embedding::forward(const Tensor& indices) const {
+  const int64_t hidden = weight_.shape()[1];
+  std::vector<int64_t> final_dims = indices.shape();
+  final_dims.push_back(hidden);
+  // indices.reshape([size]): an index tensor carries no gradient, so a plain view of the
+  // compact data under the flat shape serves
+  const Tensor ic = indices.compact();
+  const Tensor flat(ic.storage(), Layout({(int64_t)ic.layout().size()}), false, nullptr);
+  return weight_.index_select(0, flat).reshape(final_dims);
+}
+
+MLP::MLP(Tensor up_proj, Tensor down_proj) : up_(std::move(up_proj)), down_(std::move(down_proj)) {
+  if (up_.layout().ndim() != 2 || down_.layout().ndim() != 2 || up_.shape()[1] != down_.shape()[0] ||
+      up_.shape()[0] != down_.shape()[1])
+    throw std::logic_error("MLP weights must be [n_embd, hidden] and [hidden, n_embd]");
+}
+
+Tensor MLP::forward(const Tensor& x) const {
+  if (x.layout().ndim() != 3) throw std::logic_error("MLP expects input shape [B, T, C]");
+  const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
+  const Tensor y = relu_sq(x.reshape({B * T, C}).matmul(up_));  // [B*T, H]
+  return y.matmul(down_).reshape({B, T, C});
+}
+
+Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
+    : attn_(std::move(attn)), mlp_(std::move(mlp)), eps_(eps) {}
+
+Tensor Block::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const {
+  const Tensor h = x.add(attn_.forward(rms_norm(x, eps_), cos, sin));
+  return h.add(mlp_.forward(rms_norm(h, eps_)));
+}
+
+std::vector<Tensor> Block::parameters() const {
+  std::vector<Tensor> p = attn_.parameters();
+  for (const Tensor& t : mlp_.parameters()) p.push_back(t);
+  return p;
+}
+
+// Attaches every weight as a trainable leaf (once: a leaf's id is what the gradient
+// store and the optimizer key on) after checking count and the embedding's shape.
+static std::vector<Tensor> checked_attach(const GPTConfig& c, const std::vector<Tensor>& ws) {
+  if (c.n_embd % c.n_head) throw std::logic_error("n_embd must be divisible by n_head");
+  if ((int64_t)ws.size() != 2 + 6 * c.n_layer)
+    throw std::logic_error("GPT: expected " + std::to_string(2 + 6 * c.n_layer) + " weight tensors");
+  if (ws[0].shape() != std::vector<int64_t>{c.vocab_size, c.n_embd})
+    throw std::logic_error("GPT: wte must be [vocab_size, n_embd]");
+  if (ws.back().shape() != std::vector<int64_t>{c.n_embd, c.vocab_size})
+    throw std::logic_error("GPT: lm_head must be [n_embd, vocab_size]");
+  std::vector<Tensor> out;
+  out.reserve(ws.size());
+  for (const Tensor& w : ws) out.push_back(w.requires_grad() && !w.op() ? w : w.attach());
+  return out;
+}
+
+GPT::GPT(const GPTConfig& config, const std::vector<Tensor>& weights)
+    : config_(config), params_(checked_attach(config, weights)), wte_(params_[0]) {
+  for (int64_t l = 0; l < config.n_layer; ++l) {
+    const Tensor* b = &params_[1 + 6 * l];
+    blocks_.emplace_back(CausalSelfAttention(config.n_embd, config.n_head, b[0], b[1], b[2], b[3]),
+                         MLP(b[4], b[5]), config.rms_norm_eps);
+  }
+  lm_head_ = params_.back();
+  auto tables = precompute_rotary_embeddings(config.sequence_len, config.head_dim(), config.rope_base,
+                                             params_[0].dtype());
+  cos_ = tables.first;
+  sin_ = tables.second;
+}
+
+GPT GPT::init_random(const GPTConfig& c, uint64_t seed, DType dtype) {
+  if (dtype != DType::F32 && dtype != DType::F16) throw std::logic_error("GPT: f16 or f32 weights");
+  std::mt19937_64 gen(seed);
+  auto make = [&](int64_t rows, int64_t cols, bool normal) {
+    std::vector<float> host((size_t)rows * cols);
+    if (normal) {
+      std::normal_distribution<float> d(0.f, 1.f);
+      for (float& x : host) x = d(gen);
+    } else {
+      const float k = 1.0f / std::sqrt((float)rows);
+      std::uniform_real_distribution<float> d(-k, k);
+      for (float& x : host) x = d(gen);
+    }
+    Tensor t = Tensor::from_host(host.data(), {rows, cols}, DType::F32);
+    if (dtype == DType::F16) throw std::logic_error("GPT::init_random: f16 initialisation is not built");
+    return t;
+  };
+  std::vector<Tensor> w;
+  w.push_back(make(c.vocab_size, c.n_embd, true));
+  for (int64_t l = 0; l < c.n_layer; ++l) {
+    for (int i = 0; i < 4; ++i) w.push_back(make(c.n_embd, c.n_embd, false));
+    w.push_back(make(c.n_embd, c.mlp_hidden_dim, false));
+    w.push_back(make(c.mlp_hidden_dim, c.n_embd, false));
+  }
+  w.push_back(make(c.n_embd, c.vocab_size, false));
+  return GPT(c, w);
+}
+
+Tensor GPT::forward(const Tensor& idx) const {
+  if (idx.layout().ndim() != 2) throw std::logic_error("GPT expects token ids with shape [B, T]");
+  const int64_t B = idx.shape()[0], T = idx.shape()[1];
+  if (T > cos_.shape()[1]) throw std::logic_error("sequence length exceeds rotary cache");
+  // cos.narrow(1, 0, T): the first T rows of the compact [1, L, 1, D/2] tables
+  const Layout rows({1, T, 1, cos_.shape()[3]});
+  const Tensor cos(cos_.storage(), rows, false, nullptr), sin(sin_.storage(), rows, false, nullptr);
+  Tensor x = wte_.forward(idx);  // [B, T, C]
+  for (const Block& block : blocks_) x = block.forward(x, cos, sin);
+  x = rms_norm(x, config_.rms_norm_eps);
+  const Tensor logits = x.reshape({B * T, config_.n_embd}).matmul(lm_head_);  // [B*T, V]
+  return logits.reshape({B, T, config_.vocab_size});
+}
+
+std::vector<Tensor> GPT::parameters() const { return params_; }
+
+}  // namespace deers_host

@@ -1,0 +1,82 @@
+// The GPT model of src/models/gpt.rs on the ROCm device, in the C++ host: token
+// embedding, pre-norm residual blocks (RMSNorm, causal self-attention with RoPE, RMSNorm,
+// relu^2 MLP), final RMSNorm and a bias-free LM head.  Same structure, parameter order
+// and shapes as the reference; each module runs on the fused device ops of ops.h.
+#ifndef DEERS_HOST_GPT_H
+#define DEERS_HOST_GPT_H
+
+#include <cstdint>
+#include <vector>
+
+#include "ops.h"
+
+namespace deers_host {
+
+// src/nn.rs:203-229: weight [vocab, hidden]; indices of any shape -> [..., hidden].
+class Embedding {
+ public:
+  explicit Embedding(Tensor weight);
+  Tensor forward(const Tensor& indices) const;
+  std::vector<Tensor> parameters() const { return {weight_}; }
+
+ private:
+  Tensor weight_;
+};
+
+// src/models/gpt.rs:168-207: down(relu(up(x))^2), weights [in, out], no bias.
+class MLP {
+ public:
+  MLP(Tensor up_proj, Tensor down_proj);
+  Tensor forward(const Tensor& x) const;  // [B,T,C] -> [B,T,C]
+  std::vector<Tensor> parameters() const { return {up_, down_}; }
+
+ private:
+  Tensor up_, down_;
+};
+
+// src/models/gpt.rs:209-257
+class Block {
+ public:
+  Block(CausalSelfAttention attn, MLP mlp, double eps);
+  Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
+  std::vector<Tensor> parameters() const;  // attention, then MLP
+
+ private:
+  CausalSelfAttention attn_;
+  MLP mlp_;
+  double eps_;
+};
+
+// src/models/gpt.rs:259-284
+struct GPTConfig {
+  int64_t vocab_size, sequence_len, n_layer, n_head, n_embd, mlp_hidden_dim;
+  double rms_norm_eps;
+  float rope_base;
+  int64_t head_dim() const { return n_embd / n_head; }
+};
+
+// src/models/gpt.rs:286-377
+class GPT {
+ public:
+  // `weights` in parameters() order: wte [V,C]; per block q, k, v, out [C,C], up [C,H],
+  // down [H,C]; lm_head [C,V].  Each is attached as a trainable leaf.
+  GPT(const GPTConfig& config, const std::vector<Tensor>& weights);
+  // Reference initialisation: standard normal embedding (src/nn.rs:209-212), uniform
+  // [-1/sqrt(in), 1/sqrt(in)] projections (src/nn.rs:150-170), from a host generator.
+  static GPT init_random(const GPTConfig& config, uint64_t seed, DType dtype);
+
+  Tensor forward(const Tensor& idx) const;  // I64 [B,T] -> logits [B,T,V]
+  std::vector<Tensor> parameters() const;
+  const GPTConfig& config() const { return config_; }
+
+ private:
+  GPTConfig config_;
+  std::vector<Tensor> params_;  // the attached leaves, in parameters() order
+  Embedding wte_;
+  std::vector<Block> blocks_;
+  Tensor lm_head_;
+  Tensor cos_, sin_;  // [1, sequence_len, 1, head_dim/2]
+};
+
+}  // namespace deers_host
+#endif

@@ -15,6 +15,7 @@
 
 #include "../../include/deers_rocm.h"
 #include "ops.h"
+#include "gpt.h"
 #include "optim.h"
 
 using namespace deers_host;
@@ -434,6 +435,100 @@ static int run_optim(const std::string& dir) {
   return 0;
 }
 
+// The whole model: GPT forward, cross-entropy, reverse sweep, then `steps` training steps
+// (clip_grad_scale folded into AdamW), the way examples/tinystories_train.rs drives the
+// reference.  Writes logits, loss, every parameter's gradient, the per-step losses and
+// norms, and the final parameters.
+static int run_gpt(const std::string& dir) {
+  check(deers_rocm_init(0));
+  GPTConfig cfg;
+  int64_t B, T;
+  int steps;
+  double lr, wd, max_norm;
+  {
+    std::ifstream f(dir + "/case.txt");
+    if (!(f >> cfg.vocab_size >> cfg.sequence_len >> cfg.n_layer >> cfg.n_head >> cfg.n_embd >>
+          cfg.mlp_hidden_dim >> cfg.rms_norm_eps >> cfg.rope_base >> B >> T >> steps >> lr >> wd >> max_norm)) {
+      std::printf("FAIL bad case.txt\n");
+      return 2;
+    }
+  }
+  const int64_t C = cfg.n_embd, Hd = cfg.mlp_hidden_dim, V = cfg.vocab_size;
+  std::vector<std::vector<int64_t>> shapes{{V, C}};
+  for (int64_t l = 0; l < cfg.n_layer; ++l)
+    for (auto s : std::vector<std::vector<int64_t>>{{C, C}, {C, C}, {C, C}, {C, C}, {C, Hd}, {Hd, C}}) shapes.push_back(s);
+  shapes.push_back({C, V});
+  std::vector<Tensor> weights;
+  for (size_t i = 0; i < shapes.size(); ++i) {
+    auto bytes = read_file(dir + "/w" + std::to_string(i) + ".bin");
+    if (bytes.size() != (size_t)(shapes[i][0] * shapes[i][1]) * 4) { std::printf("FAIL size of w%zu\n", i); return 2; }
+    weights.push_back(Tensor::from_host(bytes.data(), shapes[i], DType::F32));
+  }
+  auto ids_b = read_file(dir + "/ids.bin"), tg_b = read_file(dir + "/targets.bin");
+  if (ids_b.size() != (size_t)(B * T) * 8 || tg_b.size() != (size_t)(B * T) * 8) { std::printf("FAIL ids/targets size\n"); return 2; }
+  Tensor ids = Tensor::from_host(ids_b.data(), {B, T}, DType::I64);
+  Tensor targets = Tensor::from_host(tg_b.data(), {B * T}, DType::I64);
+
+  GPT model(cfg, weights);
+  std::vector<Tensor> params = model.parameters();
+  EXPECT(params.size() == shapes.size());
+  for (const Tensor& p : params) EXPECT(p.requires_grad() && p.op() == nullptr);
+
+  Tensor logits = model.forward(ids);
+  EXPECT((logits.shape() == std::vector<int64_t>{B, T, V}));
+  dump(logits, dir + "/logits.bin");
+  Tensor loss = cross_entropy(logits.reshape({B * T, V}), targets);
+  EXPECT(loss.requires_grad() && std::string(loss.op()->name()) == "CrossEntropy");
+  dump(loss, dir + "/loss.bin");
+  {
+    GradientStore grads = loss.backward();
+    for (size_t i = 0; i < params.size(); ++i) {
+      const Tensor* g = grads.get(params[i].id());
+      EXPECT(g != nullptr);
+      if (g) {
+        EXPECT(g->shape() == params[i].shape());
+        dump(*g, dir + "/g" + std::to_string(i) + ".bin");
+      }
+    }
+  }
+  // inference under NoGradGuard builds no graph
+  {
+    NoGradGuard guard;
+    Tensor l2 = model.forward(ids);
+    EXPECT(!l2.requires_grad() && l2.op() == nullptr);
+  }
+  AdamW opt = AdamWConfig(lr).betas(0.9, 0.95).weight_decay(wd).build(params);
+  std::vector<float> losses, norms;
+  for (int t = 0; t < steps; ++t) {
+    Tensor l = cross_entropy(model.forward(ids).reshape({B * T, V}), targets);
+    float lv = 0;
+    l.to_host(&lv);
+    losses.push_back(lv);
+    GradientStore grads = l.backward();
+    double scale = 1.0;
+    norms.push_back(clip_grad_scale(params, grads, max_norm, &scale));
+    opt.step_with_grads(grads, scale);
+  }
+  write_file(dir + "/losses.bin", losses.data(), losses.size() * sizeof(float));
+  write_file(dir + "/norms.bin", norms.data(), norms.size() * sizeof(float));
+  for (size_t i = 0; i < params.size(); ++i) dump(params[i], dir + "/w" + std::to_string(i) + "_out.bin");
+  // a token id outside the vocabulary is reported, not followed
+  {
+    std::vector<int64_t> bad((size_t)(B * T), 0);
+    bad[0] = V;
+    Tensor bad_ids = Tensor::from_host(bad.data(), {B, T}, DType::I64);
+    bool threw = false;
+    try {
+      NoGradGuard guard;
+      Tensor l = model.forward(bad_ids);
+      check(deers_rocm_sync());  // the next synchronising call reports it
+    } catch (const RocmError&) { threw = true; }
+    EXPECT(threw);
+  }
+  std::printf("ok gpt\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "graph";
   try {
@@ -449,10 +544,12 @@ int main(int argc, char** argv) {
       if (int rc = run_log_softmax(argv[2])) return rc;
     } else if (mode == "optim" && argc > 2) {
       if (int rc = run_optim(argv[2])) return rc;
+    } else if (mode == "gpt" && argc > 2) {
+      if (int rc = run_gpt(argv[2])) return rc;
     } else if (mode == "module" && argc > 2) {
       if (int rc = run_module(argv[2])) return rc;
     } else {
-      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | optim <dir> | module <dir>\n");
+      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | optim <dir> | gpt <dir> | module <dir>\n");
       return 2;
     }
   } catch (const std::exception& e) {

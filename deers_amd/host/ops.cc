@@ -240,6 +240,124 @@ Tensor Tensor::log_softmax(size_t axis) const {
   return FusedLogSoftmax::forward(std::make_unique<FusedLogSoftmax>(*this, axis));
 }
 
+// ---- IndexSelect ----
+IndexSelect::IndexSelect(Tensor arg, size_t dim, Tensor indices)
+    : arg_(std::move(arg)), indices_(std::move(indices)) {
+  if (dim >= arg_.layout().ndim())
+    throw std::logic_error("index_select: dim " + std::to_string(dim) + " out of bounds for " +
+                           std::to_string(arg_.layout().ndim()) + " dims");
+  if (dim != 0 || arg_.layout().ndim() != 2)
+    throw std::logic_error("index_select: only dim 0 of a 2-D tensor is built on this device");
+  if (indices_.layout().ndim() != 1) throw std::logic_error("index_select requires 1D indices");
+  if (indices_.dtype() != DType::I64) throw std::logic_error("index_select indices must be i64");
+  arg_ = arg_.compact();  // src/ops.rs:1405
+  indices_ = indices_.compact();
+}
+Tensor IndexSelect::forward(std::unique_ptr<IndexSelect> self) {
+  const Tensor& w = self->arg_;
+  const int64_t n = self->indices_.shape()[0], rows = w.shape()[0], width = w.shape()[1];
+  Tensor out = empty({n, width}, w.dtype(), backed(w));
+  if (backed(w))
+    check(deers_rocm_index_select((int)w.dtype(), w.data(), (const int64_t*)self->indices_.data(),
+                                  out.data(), rows, n, width));
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void IndexSelect::backward(GradientStore& grads, const Tensor& out_grad) const {
+  const Tensor g = out_grad.compact();
+  Tensor dw = arg_.zeros_like();
+  if (backed(g))
+    check(deers_rocm_index_add((int)g.dtype(), g.data(), (const int64_t*)indices_.data(), dw.data(),
+                               arg_.shape()[0], indices_.shape()[0], arg_.shape()[1]));
+  grads.accumulate(arg_, dw);
+}
+Tensor Tensor::index_select(size_t dim, const Tensor& indices) const {
+  return IndexSelect::forward(std::make_unique<IndexSelect>(*this, dim, indices));
+}
+
+// ---- RmsNorm ----
+static void rows_of(const Tensor& t, int64_t* outer, int64_t* inner) {
+  if (t.layout().ndim() == 0) throw std::logic_error("a row-wise op needs at least one axis");
+  *inner = t.shape().back();
+  *outer = *inner ? (int64_t)t.layout().size() / *inner : 0;
+}
+Tensor RmsNorm::forward(std::unique_ptr<RmsNorm> self) {
+  self->arg_ = self->arg_.compact();
+  const Tensor& x = self->arg_;
+  int64_t outer, inner;
+  rows_of(x, &outer, &inner);
+  Tensor y = empty(x.shape(), x.dtype(), backed(x));
+  if (backed(x)) check(deers_rocm_rms_norm_fwd((int)x.dtype(), x.data(), y.data(), outer, inner, self->eps_));
+  return Tensor(y.storage(), y.layout(), false, std::move(self));
+}
+void RmsNorm::backward(GradientStore& grads, const Tensor& out_grad) const {
+  const Tensor g = out_grad.compact();
+  int64_t outer, inner;
+  rows_of(arg_, &outer, &inner);
+  Tensor dx = empty(arg_.shape(), arg_.dtype(), backed(arg_));
+  if (backed(arg_))
+    check(deers_rocm_rms_norm_bwd((int)arg_.dtype(), arg_.data(), g.data(), dx.data(), outer, inner, eps_));
+  grads.accumulate(arg_, dx);
+}
+Tensor rms_norm(const Tensor& x, double eps) {
+  return RmsNorm::forward(std::make_unique<RmsNorm>(x, eps));
+}
+
+// ---- ReluSq ----
+Tensor ReluSq::forward(std::unique_ptr<ReluSq> self) {
+  self->arg_ = self->arg_.compact();
+  const Tensor& x = self->arg_;
+  Tensor y = empty(x.shape(), x.dtype(), backed(x));
+  if (backed(x)) check(deers_rocm_relu_sq_fwd((int)x.dtype(), x.data(), y.data(), (int64_t)x.layout().size()));
+  return Tensor(y.storage(), y.layout(), false, std::move(self));
+}
+void ReluSq::backward(GradientStore& grads, const Tensor& out_grad) const {
+  const Tensor g = out_grad.compact();
+  Tensor dx = empty(arg_.shape(), arg_.dtype(), backed(arg_));
+  if (backed(arg_))
+    check(deers_rocm_relu_sq_bwd((int)arg_.dtype(), arg_.data(), g.data(), dx.data(),
+                                 (int64_t)arg_.layout().size()));
+  grads.accumulate(arg_, dx);
+}
+Tensor relu_sq(const Tensor& x) { return ReluSq::forward(std::make_unique<ReluSq>(x)); }
+
+// ---- CrossEntropy ----
+CrossEntropy::CrossEntropy(Tensor logits, Tensor targets)
+    : logits_(std::move(logits)), targets_(std::move(targets)) {
+  if (logits_.layout().ndim() != 2) throw std::logic_error("cross_entropy: logits must be [N, classes]");
+  if (targets_.layout().ndim() != 1 || targets_.shape()[0] != logits_.shape()[0])
+    throw std::logic_error("cross_entropy: targets must be [N]");
+  if (targets_.dtype() != DType::I64) throw std::logic_error("cross_entropy: targets must be i64");
+  if (logits_.shape()[0] < 1) throw std::logic_error("cross_entropy: empty batch");
+  logits_ = logits_.compact();
+  targets_ = targets_.compact();
+}
+Tensor CrossEntropy::forward(std::unique_ptr<CrossEntropy> self) {
+  const Tensor& x = self->logits_;
+  const int64_t n = x.shape()[0], v = x.shape()[1];
+  Tensor loss = empty({1}, DType::F32, backed(x));
+  self->row_lse_ = empty({n}, DType::F32, backed(x));
+  if (backed(x))
+    check(deers_rocm_cross_entropy_fwd((int)x.dtype(), x.data(), (const int64_t*)self->targets_.data(),
+                                       (float*)self->row_lse_.data(), (float*)loss.data(), n, v));
+  return Tensor(loss.storage(), loss.layout(), false, std::move(self));
+}
+void CrossEntropy::backward(GradientStore& grads, const Tensor& out_grad) const {
+  if (!row_lse_.defined()) throw std::logic_error("forward must run before backward");
+  if (out_grad.dtype() != DType::F32 || out_grad.layout().size() != 1)
+    throw std::logic_error("cross_entropy: the upstream gradient is one f32 value");
+  const Tensor up = out_grad.compact();
+  const Tensor& x = logits_;
+  Tensor dx = empty(x.shape(), x.dtype(), backed(x));
+  if (backed(x))
+    check(deers_rocm_cross_entropy_bwd((int)x.dtype(), x.data(), (const int64_t*)targets_.data(),
+                                       (const float*)row_lse_.data(), (const float*)up.data(), dx.data(),
+                                       x.shape()[0], x.shape()[1]));
+  grads.accumulate(logits_, dx);
+}
+Tensor cross_entropy(const Tensor& logits, const Tensor& targets) {
+  return CrossEntropy::forward(std::make_unique<CrossEntropy>(logits, targets));
+}
+
 // ---- FusedCausalAttention ----
 FusedCausalAttention::FusedCausalAttention(Tensor q, Tensor k, Tensor v, double scale)
     : q_(std::move(q)), k_(std::move(k)), v_(std::move(v)), scale_(scale) {

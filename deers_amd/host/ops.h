@@ -111,10 +111,6 @@ class FusedCausalAttention : public TensorOp {
   Tensor saved_o_, saved_lse_;  // set by forward, created with no op
 };
 
-// apply_rotary_emb on a [B,T,H,D] projection followed by permute([0,2,1,3])
-// (src/models/gpt.rs:49-73, 135-136) as one op: returns the rotated heads as compact
-// [B,H,T,D]; the backward hands the [B,T,H,D] gradient to the projection.  cos and
-// sin are the tables of precompute_rotary_embeddings and carry no gradient.
 // src/ops.rs:1186-1251: log-softmax over the last axis in one kernel, its output saved
 // for the backward (out_grad - exp(lsm) * rowsum(out_grad)).  Tensor::log_softmax takes
 // this path when the axis is the last one (src/tensor.rs:408-427); other axes are not
@@ -133,6 +129,75 @@ class FusedLogSoftmax : public TensorOp {
   Tensor lsm_output_;  // no op, no grad: saved like the reference's lsm_output
 };
 
+// Rows of a [n, width] table picked by 1-D I64 indices (IndexSelect, src/ops.rs:1383-1447,
+// dim 0 only: the embedding lookup of src/nn.rs:216-224).  The backward scatters the
+// output gradient into zeros of the table's shape in ascending position order
+// (index_add), so repeated tokens accumulate exactly as on the reference's CPU path.
+class IndexSelect : public TensorOp {
+ public:
+  IndexSelect(Tensor arg, size_t dim, Tensor indices);
+  static Tensor forward(std::unique_ptr<IndexSelect> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "IndexSelect"; }
+
+ private:
+  Tensor arg_, indices_;
+};
+
+// RMSNorm::forward (src/nn.rs:244-251), x * (mean(x^2, last) + eps)^-0.5, as one op with
+// one kernel each way instead of the reference's chain of five ops.
+class RmsNorm : public TensorOp {
+ public:
+  RmsNorm(Tensor arg, double eps) : arg_(std::move(arg)), eps_(eps) {}
+  static Tensor forward(std::unique_ptr<RmsNorm> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "RmsNorm"; }
+
+ private:
+  Tensor arg_;  // compacted by forward
+  double eps_;
+};
+Tensor rms_norm(const Tensor& x, double eps);
+
+// relu(x)^2, the MLP activation `y.relu(); &y * &y` (src/models/gpt.rs:196-197), as one op.
+class ReluSq : public TensorOp {
+ public:
+  explicit ReluSq(Tensor arg) : arg_(std::move(arg)) {}
+  static Tensor forward(std::unique_ptr<ReluSq> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&arg_}; }
+  const char* name() const override { return "ReluSq"; }
+
+ private:
+  Tensor arg_;
+};
+Tensor relu_sq(const Tensor& x);
+
+// loss::cross_entropy (src/loss.rs:21-24) on logits [N, V] and I64 targets [N] as one op:
+// the forward streams the logits once and keeps each row's ln-sum-exp, the backward
+// writes (softmax - onehot) * upstream / N; the [N, V] log-probabilities of the
+// reference's log_softmax + gather + sum chain are never materialised.  The loss is an
+// F32 tensor of shape [1] whatever the logits' type.
+class CrossEntropy : public TensorOp {
+ public:
+  CrossEntropy(Tensor logits, Tensor targets);
+  static Tensor forward(std::unique_ptr<CrossEntropy> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&logits_}; }
+  const char* name() const override { return "CrossEntropy"; }
+
+ private:
+  Tensor logits_, targets_;
+  Tensor row_lse_;  // [N] f32, set by forward
+};
+Tensor cross_entropy(const Tensor& logits, const Tensor& targets);
+
+// apply_rotary_emb on a [B,T,H,D] projection followed by permute([0,2,1,3])
+// (src/models/gpt.rs:49-73, 135-136) as one op: returns the rotated heads as compact
+// [B,H,T,D]; the backward hands the [B,T,H,D] gradient to the projection.  cos and
+// sin are the tables of precompute_rotary_embeddings and carry no gradient.
 class RotaryHeads : public TensorOp {
  public:
   RotaryHeads(Tensor x, Tensor cos, Tensor sin);

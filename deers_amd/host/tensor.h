@@ -32,8 +32,10 @@ struct RocmError : std::runtime_error {
 };
 void check(int rc);  // throws RocmError with deers_rocm_last_error() if rc != 0
 
-enum class DType { F16 = 0, F32 = 1 };
-inline size_t size_in_bytes(DType d) { return d == DType::F16 ? 2 : 4; }
+// F16 / F32 carry the library's dtype codes; I64 exists for index tensors only (token
+// ids, class targets: DType::I64 in the reference) and no arithmetic kernel takes it.
+enum class DType { F16 = 0, F32 = 1, I64 = 2 };
+inline size_t size_in_bytes(DType d) { return d == DType::F16 ? 2 : (d == DType::F32 ? 4 : 8); }
 
 // src/layout.rs: shape, strides in elements, offset in elements.
 struct Layout {
@@ -130,6 +132,8 @@ class Tensor {
   Tensor transpose() const;  // swaps the last two axes (a Permute)
   Tensor reshape(const std::vector<int64_t>& shape) const;  // compacts first (src/ops.rs:913)
   Tensor matmul(const Tensor& other) const;
+  // Rows of a 2-D tensor picked by a 1-D I64 index tensor (src/ops.rs:1383-1447, dim 0).
+  Tensor index_select(size_t dim, const Tensor& indices) const;
   // Log-softmax over the last axis through the fused op (src/tensor.rs:408-427).
   Tensor log_softmax(size_t axis) const;
   // Differentiable element-wise ops used by the contract tests.
