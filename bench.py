@@ -259,6 +259,43 @@ def bench_adamw(steps: int, warmup: int):
     return out
 
 
+def bench_gpt(steps: int, warmup: int):
+    """End-to-end GPT training step (BASELINE configs[4]): f32 parameters, 12 layers,
+    12 heads, n_embd 768, MLP 3072, vocabulary 50257, sequence 1024, batch 8; forward,
+    cross-entropy, backward, gradient-norm clipping, AdamW, all on the device through the
+    C++ host (deers_amd/host/gpt_step), with the library's GEMM kernel picked per problem by
+    timing during the untimed warm-up steps.  Reports the step time and tokens per second
+    and the time per kernel family from a profiled pass."""
+    import subprocess
+    exe = os.path.join(ROOT, "deers_amd", "host", "gpt_step")
+    if not os.path.exists(exe):
+        raise RuntimeError("deers_amd/host/gpt_step is not built (run __graft_entry__.build())")
+    cfg = {"vocab_size": 50257, "seq_len": 1024, "n_layer": 12, "n_head": 12, "n_embd": 768,
+           "mlp_hidden": 3072, "batch": 8}
+    r = subprocess.run([exe] + [str(cfg[k]) for k in ("vocab_size", "seq_len", "n_layer", "n_head",
+                                                      "n_embd", "mlp_hidden", "batch")]
+                       + [str(steps), str(warmup), "tune"], capture_output=True, text=True, timeout=600)
+    if r.returncode != 0:
+        raise RuntimeError("gpt_step failed: " + r.stderr.strip())
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    tokens = cfg["batch"] * cfg["seq_len"]
+    # matrix-product work: every Linear (blocks + LM head) forward and both backward products
+    linear_params = cfg["n_layer"] * (4 * cfg["n_embd"] ** 2 + 2 * cfg["n_embd"] * cfg["mlp_hidden"]) \
+        + cfg["n_embd"] * cfg["vocab_size"]
+    gemm_flops = 6.0 * linear_params * tokens
+    fwd_f, bwd_f = attn_flops(cfg["batch"], cfg["n_head"], cfg["seq_len"], cfg["n_embd"] // cfg["n_head"])
+    attn = cfg["n_layer"] * (fwd_f + bwd_f)
+    out["workload"] = ("GPT training step, f32, 12 layers x 12 heads x 768, MLP 3072, vocab 50257, "
+                       "seq 1024, batch 8 (BASELINE configs[4]); synthetic token ids, random-init weights")
+    out["flops_per_step"] = {"matmul": gemm_flops, "attention": attn}
+    out["model_tflops"] = (gemm_flops + attn) / (out["ms_per_step"] * 1e-3) / 1e12
+    mm = out["kernels"].get("matmul")
+    if mm:
+        mm["tflops"] = gemm_flops / (mm["ms_per_step"] * 1e-3) / 1e12
+        mm["frac_f32_matrix_peak"] = mm["tflops"] / 157.3
+    return out
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -290,7 +327,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw"], default="all",
+    ap.add_argument("--no-gpt", action="store_true",
+                    help="skip the end-to-end GPT training step reported beside the headline")
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw", "gpt"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -312,6 +351,8 @@ def main():
         elif args.only == "adamw":
             print(json.dumps({"only": "adamw",
                               **bench_adamw(min(args.steps, 20), min(args.warmup, 5))}))
+        elif args.only == "gpt":
+            print(json.dumps({"only": "gpt", **bench_gpt(min(args.steps, 10), min(args.warmup, 3))}))
         elif args.only == "copy":
             print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
         else:
@@ -369,6 +410,14 @@ def main():
                    "GB/s_whole_call": dec["gbs_call"], "peak_GB/s": PEAK_HBM_GBS,
                    "frac_hbm_peak": dec["gbs_kernel"] / PEAK_HBM_GBS},
     }
+    if not args.no_gpt:
+        # BASELINE configs[4], reported beside the headline (never part of `value`)
+        try:
+            g = bench_gpt(5, 2)
+            out["gpt_train_step"] = {k: g[k] for k in ("workload", "ms_per_step", "tokens_per_s",
+                                                       "parameters", "model_tflops", "kernels")}
+        except Exception as e:  # the headline line must not depend on it
+            out["gpt_train_step"] = {"error": str(e)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

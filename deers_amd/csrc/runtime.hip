@@ -3,6 +3,7 @@
 // checks in front of every kernel launch.  The shape of the runtime follows what
 // the reference's CUDA backend keeps in its OnceLock (one context, one stream,
 // device ordinal fixed at init: src/storage/cuda.rs:462-528).
+#define ROCBLAS_BETA_FEATURES_API 1  // solution enumeration for the GEMM tuner
 #include <rocblas/rocblas.h>
 #include "../../include/deers_rocm.h"
 
@@ -12,6 +13,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <map>
+#include <unordered_map>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -83,6 +85,19 @@ struct Runtime {
   // next synchronising call after one of them has been launched
   int* index_flag = nullptr;
   bool index_flag_armed = false;
+  // Block cache behind deers_rocm_alloc / _free.  Every kernel and copy of this library
+  // runs on `stream`, in order, so a block handed back by free can be handed out again
+  // without waiting for the device: whatever still reads it was enqueued earlier than
+  // whatever will write it.  A training step allocates the same sizes every iteration;
+  // going to hipMalloc / hipFree each time would serialise the host with the device.
+  // GEMM tuner (off by default): the library's own choice of kernel for a problem is a
+  // heuristic; with tuning on, the first call of each distinct problem times every
+  // kernel the library offers for it and later calls use the fastest.
+  bool tune_gemm = false;
+  std::map<std::vector<int64_t>, int> gemm_choice;  // problem -> solution index (0 = library default)
+  std::unordered_map<size_t, std::vector<void*>> free_blocks;  // by rounded size
+  std::unordered_map<void*, size_t> block_size;                // every block handed out
+  size_t cached_bytes = 0;
 };
 
 Runtime g_rt;
@@ -306,14 +321,46 @@ const char* deers_rocm_last_error(void) { return t_err.c_str(); }
 
 void* deers_rocm_stream(void) { return g_rt.ready ? (void*)g_rt.stream : nullptr; }
 
+// Returns every cached block to the driver (after the stream has drained).
+static int release_cached_blocks() {
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  for (auto& kv : g_rt.free_blocks)
+    for (void* p : kv.second) HIP_TRY(hipFree(p));
+  g_rt.free_blocks.clear();
+  g_rt.cached_bytes = 0;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_empty_cache(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  return release_cached_blocks();
+}
+
 int deers_rocm_alloc(size_t bytes, void** out_ptr) {
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   if (!out_ptr) return fail(DEERS_ROCM_ERR_ARG, "alloc: null out_ptr");
   *out_ptr = nullptr;
   if (bytes == 0) return DEERS_ROCM_OK;
+  const size_t size = (bytes + 255) & ~(size_t)255;
+  auto hit = g_rt.free_blocks.find(size);
+  if (hit != g_rt.free_blocks.end() && !hit->second.empty()) {
+    *out_ptr = hit->second.back();
+    hit->second.pop_back();
+    g_rt.cached_bytes -= size;
+    g_rt.block_size[*out_ptr] = size;
+    return DEERS_ROCM_OK;
+  }
   HIP_TRY(hipSetDevice(g_rt.ordinal));
-  HIP_TRY(hipMalloc(out_ptr, bytes));
+  hipError_t e = hipMalloc(out_ptr, size);
+  if (e == hipErrorOutOfMemory) {
+    (void)hipGetLastError();
+    if (int rc = release_cached_blocks()) return rc;
+    e = hipMalloc(out_ptr, size);
+  }
+  HIP_TRY(e);
+  g_rt.block_size[*out_ptr] = size;
   return DEERS_ROCM_OK;
 }
 
@@ -329,9 +376,15 @@ int deers_rocm_free(void* ptr) {
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   if (!ptr) return DEERS_ROCM_OK;
-  // Work already enqueued may still read the buffer.
-  HIP_TRY(hipStreamSynchronize(g_rt.stream));
-  HIP_TRY(hipFree(ptr));
+  auto it = g_rt.block_size.find(ptr);
+  if (it == g_rt.block_size.end())
+    return fail(DEERS_ROCM_ERR_ARG, "free: %p was not allocated by deers_rocm_alloc (or freed twice)", ptr);
+  // Work already enqueued may still read the buffer: it stays allocated and goes back
+  // to the cache, to be reused by later work on the same stream.
+  const size_t size = it->second;
+  g_rt.block_size.erase(it);
+  g_rt.free_blocks[size].push_back(ptr);
+  g_rt.cached_bytes += size;
   return DEERS_ROCM_OK;
 }
 
@@ -857,6 +910,25 @@ int deers_rocm_scale(int dtype, void* x, int64_t n, double scale) {
 
 // ---- batched matrix product (library GEMM) ----
 
+// the solution-enumeration calls are tagged "beta, subject to change" by their header
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wdeprecated-declarations"
+
+#define HIP_TRY_BOOL(expr)              \
+  do {                                  \
+    if ((expr) != hipSuccess) {         \
+      (void)hipGetLastError();          \
+      return false;                     \
+    }                                   \
+  } while (0)
+
+int deers_rocm_matmul_tune(int on) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  g_rt.tune_gemm = on != 0;
+  return DEERS_ROCM_OK;
+}
+
 int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
                       const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
                       int64_t batch, int64_t m, int64_t n, int64_t k) {
@@ -900,17 +972,81 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
   // own transpose with leading dimension = row stride.
   const rocblas_datatype ty = dtype == DEERS_ROCM_F16 ? rocblas_datatype_f16_r : rocblas_datatype_f32_r;
   const float alpha = 1.f, beta = 0.f;
-  const rocblas_status st = rocblas_gemm_strided_batched_ex(
-      g_rt.blas, b_t ? rocblas_operation_transpose : rocblas_operation_none,
-      a_t ? rocblas_operation_transpose : rocblas_operation_none, (rocblas_int)n, (rocblas_int)m,
-      (rocblas_int)k, &alpha, b, ty, (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c,
-      ty, (rocblas_int)n, m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch,
-      rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+  const rocblas_operation op_b = b_t ? rocblas_operation_transpose : rocblas_operation_none;
+  const rocblas_operation op_a = a_t ? rocblas_operation_transpose : rocblas_operation_none;
+  auto run = [&](int solution) {
+    return rocblas_gemm_strided_batched_ex(
+        g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
+        (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n, m * n, c,
+        ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
+        solution ? rocblas_gemm_algo_solution_index : rocblas_gemm_algo_standard, solution, 0);
+  };
+  int solution = 0;
+  if (g_rt.tune_gemm) {
+    const std::vector<int64_t> key{dtype, (int64_t)b_t, (int64_t)a_t, n, m, k, ldb, lda, b_bs, a_bs, batch};
+    auto hit = g_rt.gemm_choice.find(key);
+    if (hit != g_rt.gemm_choice.end()) {
+      solution = hit->second;
+    } else {
+      // Times the default and every listed kernel on the caller's own operands (the
+      // output is overwritten by the real call below): one warm-up and one timed run
+      // each, a second timed run for those within 20 % of the best so far.
+      rocblas_int count = 0;
+      std::vector<rocblas_int> list;
+      if (rocblas_gemm_strided_batched_ex_get_solutions(
+              g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
+              (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n,
+              m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
+              rocblas_gemm_algo_solution_index, 0, nullptr, &count) == rocblas_status_success &&
+          count > 0) {
+        list.resize(count);
+        if (rocblas_gemm_strided_batched_ex_get_solutions(
+                g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
+                (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n,
+                m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
+                rocblas_gemm_algo_solution_index, 0, list.data(), &count) != rocblas_status_success)
+          list.clear();
+      }
+      hipEvent_t e0, e1;
+      HIP_TRY(hipEventCreate(&e0));
+      HIP_TRY(hipEventCreate(&e1));
+      auto time_one = [&](int sol, float* ms) -> bool {
+        HIP_TRY_BOOL(hipEventRecord(e0, g_rt.stream));
+        if (run(sol) != rocblas_status_success) return false;
+        HIP_TRY_BOOL(hipEventRecord(e1, g_rt.stream));
+        HIP_TRY_BOOL(hipEventSynchronize(e1));
+        HIP_TRY_BOOL(hipEventElapsedTime(ms, e0, e1));
+        return true;
+      };
+      float best = 0.f;
+      float t = 0.f;
+      if (!time_one(0, &t) || !time_one(0, &best)) best = 1e30f;  // warm-up, then the default
+      list.insert(list.begin(), 0);
+      for (size_t i = 1; i < list.size(); ++i) {
+        float t1 = 0.f, t2 = 0.f;
+        if (!time_one(list[i], &t1) || !time_one(list[i], &t1)) continue;  // warm-up, timed
+        if (t1 > 1.2f * best) continue;
+        if (!time_one(list[i], &t2)) continue;
+        const float tt = t1 < t2 ? t1 : t2;
+        if (tt < best) {
+          best = tt;
+          solution = list[i];
+        }
+      }
+      (void)hipEventDestroy(e0);
+      (void)hipEventDestroy(e1);
+      g_rt.gemm_choice[key] = solution;
+    }
+  }
+  deers::LaunchScope scope("matmul", g_rt.stream);
+  rocblas_status st = run(solution);
+  if (st != rocblas_status_success && solution) st = run(0);
   if (st != rocblas_status_success)
     return fail(DEERS_ROCM_ERR_HIP, "rocblas_gemm_strided_batched_ex failed: %s",
                 rocblas_status_to_string(st));
   return DEERS_ROCM_OK;
 }
+#pragma clang diagnostic pop
 
 // ---- rotary embedding fused with the head split / merge ----
 

@@ -1,0 +1,104 @@
+// Times the end-to-end GPT training step on the ROCm device: forward, cross-entropy,
+// reverse sweep, gradient-norm clipping and AdamW, on synthetic token ids and
+// random-init weights (the reference's loop: examples/tinystories_train.rs).  Prints one
+// JSON line: wall time per step between two stream synchronisations, tokens per second,
+// and, from a second profiled pass, the time per kernel family.
+//
+//   gpt_step vocab seq n_layer n_head n_embd mlp_hidden batch steps warmup [tune]
+// `tune` lets the first step pick the fastest library GEMM kernel per problem.
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../include/deers_rocm.h"
+#include "gpt.h"
+#include "optim.h"
+
+using namespace deers_host;
+
+int main(int argc, char** argv) {
+  if (argc < 10) {
+    std::fprintf(stderr, "usage: gpt_step vocab seq n_layer n_head n_embd mlp_hidden batch steps warmup\n");
+    return 2;
+  }
+  try {
+    check(deers_rocm_init(0));
+    const bool tune = argc > 10 && std::string(argv[10]) == "tune";
+    check(deers_rocm_matmul_tune(tune ? 1 : 0));
+    GPTConfig cfg;
+    cfg.vocab_size = std::atoll(argv[1]);
+    cfg.sequence_len = std::atoll(argv[2]);
+    cfg.n_layer = std::atoll(argv[3]);
+    cfg.n_head = std::atoll(argv[4]);
+    cfg.n_embd = std::atoll(argv[5]);
+    cfg.mlp_hidden_dim = std::atoll(argv[6]);
+    cfg.rms_norm_eps = 1e-5;
+    cfg.rope_base = 10000.0f;
+    const int64_t B = std::atoll(argv[7]), T = cfg.sequence_len;
+    const int steps = std::atoi(argv[8]), warmup = std::atoi(argv[9]);
+
+    GPT model = GPT::init_random(cfg, 1234, DType::F32);
+    std::vector<Tensor> params = model.parameters();
+    int64_t n_params = 0;
+    for (const Tensor& p : params) n_params += (int64_t)p.layout().size();
+
+    std::mt19937_64 gen(99);
+    std::uniform_int_distribution<int64_t> tok(0, cfg.vocab_size - 1);
+    std::vector<int64_t> h_ids((size_t)(B * T)), h_tg((size_t)(B * T));
+    for (auto& x : h_ids) x = tok(gen);
+    for (auto& x : h_tg) x = tok(gen);
+    Tensor ids = Tensor::from_host(h_ids.data(), {B, T}, DType::I64);
+    Tensor targets = Tensor::from_host(h_tg.data(), {B * T}, DType::I64);
+
+    AdamW opt = AdamWConfig(3e-4).betas(0.9, 0.95).weight_decay(0.1).build(params);
+    float last_loss = 0.f, last_norm = 0.f;
+    auto step = [&]() {
+      Tensor loss = cross_entropy(model.forward(ids).reshape({B * T, cfg.vocab_size}), targets);
+      GradientStore grads = loss.backward();
+      double scale = 1.0;
+      last_norm = clip_grad_scale(params, grads, 1.0, &scale);  // reads 4 bytes back: one sync per step
+      opt.step_with_grads(grads, scale);
+      loss.to_host(&last_loss);
+    };
+    for (int i = 0; i < warmup; ++i) step();
+    const float first_loss = last_loss;
+    check(deers_rocm_sync());
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i) step();
+    check(deers_rocm_sync());
+    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
+
+    // profiled pass: every launch bracketed by events
+    check(deers_rocm_profile_enable(1));
+    const int prof_steps = steps < 3 ? steps : 3;
+    for (int i = 0; i < prof_steps; ++i) step();
+    int rows = 0;
+    check(deers_rocm_profile_collect(&rows));
+    std::string kernels = "{";
+    for (int r = 0; r < rows; ++r) {
+      const char* name = nullptr;
+      int64_t calls = 0;
+      float total_ms = 0;
+      check(deers_rocm_profile_row(r, &name, &calls, &total_ms));
+      char buf[256];
+      std::snprintf(buf, sizeof(buf), "%s\"%s\": {\"calls_per_step\": %.1f, \"ms_per_step\": %.4f}", r ? ", " : "",
+                    name, (double)calls / prof_steps, total_ms / prof_steps);
+      kernels += buf;
+    }
+    kernels += "}";
+    check(deers_rocm_profile_enable(0));
+
+    std::printf(
+        "{\"gemm_tuning\": %s, \"ms_per_step\": %.3f, \"tokens_per_s\": %.1f, \"parameters\": %lld, \"batch\": %lld, \"seq_len\": %lld, "
+        "\"loss_first\": %.4f, \"loss_last\": %.4f, \"grad_norm\": %.4f, \"kernels\": %s}\n",
+        tune ? "true" : "false", ms, 1e3 * (double)(B * T) / ms, (long long)n_params, (long long)B, (long long)T, first_loss, last_loss,
+        last_norm, kernels.c_str());
+    return 0;
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "gpt_step: %s\n", e.what());
+    return 1;
+  }
+}

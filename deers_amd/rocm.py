@@ -140,6 +140,14 @@ def profile_enable(on: bool = True):
     _check(load().deers_rocm_profile_enable(ctypes.c_int(1 if on else 0)))
 
 
+def matmul_tune(on: bool):
+    _check(load().deers_rocm_matmul_tune(ctypes.c_int(1 if on else 0)))
+
+
+def empty_cache():
+    _check(load().deers_rocm_empty_cache())
+
+
 def profile_collect() -> dict:
     """{kernel name: (calls, total_ms)} for launches since profile_enable(True)."""
     n = ctypes.c_int()

@@ -81,7 +81,13 @@ void* deers_rocm_stream(void);
  * src/device.rs:77-90).  `bytes` may be 0 (returns a NULL pointer). */
 int deers_rocm_alloc(size_t bytes, void** out_ptr);
 int deers_rocm_alloc_zeros(size_t bytes, void** out_ptr);
+/* Blocks are cached by size: free returns at once, without waiting for the device, and
+ * a later alloc of the same size reuses the block.  That is safe because all of the
+ * library's work runs in order on one stream (a buffer the caller also uses on another
+ * stream must be ordered by the caller).  A block leaves the cache when hipMalloc runs
+ * out of memory or deers_rocm_empty_cache is called. */
 int deers_rocm_free(void* ptr);
+int deers_rocm_empty_cache(void);
 
 /* Host->device copy, replaces CpuStorage::to(device) (src/storage/cpu.rs:26-32).
  * Returns after the host buffer may be reused. */
@@ -293,6 +299,13 @@ int deers_rocm_matmul(int dtype,
                       const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
                       const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
                       void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
+/* Off by default.  When on, the first matmul of each distinct problem (sizes, strides,
+ * transposes, batch) times every kernel the BLAS offers for it on the caller's operands
+ * and later calls of that problem use the fastest; the library's own pick is a heuristic
+ * and loses up to 2x on tall-skinny products such as the LM head's weight gradient.
+ * Costs seconds on the first training step; results are unchanged up to the summation
+ * order inside the chosen kernel. */
+int deers_rocm_matmul_tune(int on);
 
 /* ---- rotary embedding fused with the head split / merge -----------------------
  * The neighbours of the attention core in CausalSelfAttention::forward

@@ -84,3 +84,27 @@ def test_matmul_edge_cases_and_errors():
         rocm.matmul_raw(np.float32, buf.ptr, (8, 2, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 2, 3, 4)
     with pytest.raises(rocm.RocmError):
         rocm.matmul_raw(np.float32, None, (4, 1, 0), buf.ptr, (3, 1, 0), out.ptr, 1, 2, 3, 4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float16, 2e-2), (np.float32, 1e-4)])
+def test_matmul_with_kernel_tuning_gives_the_same_product(dtype, tol):
+    # with tuning on, the first call of a problem times every kernel the BLAS lists for it;
+    # whatever it settles on, the product is the same within the type's tolerance, on plain,
+    # transposed and broadcast operands, on the first (tuning) call and on later ones
+    rng = np.random.default_rng(35)
+    rocm.matmul_tune(True)
+    try:
+        for batch, m, n, k in [(1, 512, 96, 768), (2, 130, 33, 64), (1, 64, 1000, 192)]:
+            a = rng.standard_normal((batch, m, k)).astype(dtype)
+            b = (rng.standard_normal((batch, k, n)) / np.sqrt(k)).astype(dtype)
+            want = oracle.matmul(a.astype(np.float32), b.astype(np.float32))
+            for _ in range(2):
+                assert np.max(np.abs(_run(a, b, dtype).astype(np.float64) - want)) <= tol
+            # A^T stored: logical a[b,i,j] = buf[b,j,i]
+            at = np.ascontiguousarray(a.transpose(0, 2, 1))
+            for _ in range(2):
+                got = _run(a, b, dtype, a_view=(at, (1, m, m * k)))
+                assert np.max(np.abs(got.astype(np.float64) - want)) <= tol
+    finally:
+        rocm.matmul_tune(False)
