@@ -17,7 +17,8 @@ constexpr int kBwd32Blk = 128;
 #define ZEROF4 floatx4{0, 0, 0, 0}
 
 template <int D, int STEP>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(BwdParams p, int BH, int n_blocks,
+                                                                int heads_per_xcd) {
   constexpr int LD = D + 4;
   constexpr int KH = D / 2;
   constexpr int DB = D / 32;
@@ -35,8 +36,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(BwdParams p) {
   const int wave = tid >> 6;
   const int g = lane >> 5;
   const int T = p.T;
-  const int kvblk = blockIdx.x;
-  const int bh = blockIdx.y;
+  // every block of a head on one XCD, each XCD's list longest first: the first key
+  // block is seen by every query block
+  int bh, rank;
+  if (!map_block(blockIdx.x, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  const int kvblk = rank;
   const int b = bh / p.H, h = bh % p.H;
 
   const float* Q = (const float*)p.q + b * p.sq.b + h * p.sq.h;
@@ -195,7 +199,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(BwdParams p) {
 }
 
 template <int D, int STEP>
-__global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(BwdParams p, int BH, int n_blocks,
+                                                              int heads_per_xcd) {
   constexpr int LD = D + 4;
   constexpr int KH = D / 2;
   constexpr int DB = D / 32;
@@ -211,8 +216,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(BwdParams p) {
   const int wave = tid >> 6;
   const int g = lane >> 5;
   const int T = p.T;
-  const int qtile = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y;
+  int bh, rank;
+  if (!map_block(blockIdx.x, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  const int qtile = n_blocks - 1 - rank;  // the last query block sees every key block
   const int b = bh / p.H, h = bh % p.H;
 
   const float* Q = (const float*)p.q + b * p.sq.b + h * p.sq.h;
@@ -355,14 +361,19 @@ static void launch_bwd_f32_d(const BwdParams& p, int B, hipStream_t stream) {
     hipLaunchKernelGGL((attn_bwd_delta_kernel<float, D>), dim3((threads + 255) / 256), dim3(256),
                        0, stream, p, B);
   }
-  dim3 grid((p.T + kBwd32Blk - 1) / kBwd32Blk, B * p.H);
+  const int BH = B * p.H;
+  const int n_blocks = (p.T + kBwd32Blk - 1) / kBwd32Blk;
+  const int heads_per_xcd = (BH + 7) / 8;
+  const dim3 grid(8 * n_blocks * heads_per_xcd);
   {
     LaunchScope scope("attn_bwd_dkdv_f32", stream);
-    hipLaunchKernelGGL((attn_bwd_dkdv_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((attn_bwd_dkdv_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p, BH,
+                       n_blocks, heads_per_xcd);
   }
   {
     LaunchScope scope("attn_bwd_dq_f32", stream);
-    hipLaunchKernelGGL((attn_bwd_dq_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((attn_bwd_dq_f32_kernel<D, STEP>), grid, dim3(256), 0, stream, p, BH,
+                       n_blocks, heads_per_xcd);
   }
 }
 

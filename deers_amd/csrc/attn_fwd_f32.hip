@@ -14,7 +14,8 @@ namespace deers {
 constexpr int kFwd32BM = 128;
 
 template <int D, int BN>
-__global__ __launch_bounds__(256) void attn_fwd_f32_kernel(FwdParams p) {
+__global__ __launch_bounds__(256) void attn_fwd_f32_kernel(FwdParams p, int BH, int n_qtiles,
+                                                           int heads_per_xcd) {
   constexpr int LD = D + 4;   // LDS row stride in floats
   constexpr int KH = D / 2;   // contraction steps (2 elements of D per MFMA)
   constexpr int DB = D / 32;
@@ -30,8 +31,10 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(FwdParams p) {
   const int wave = tid >> 6;
   const int g = lane >> 5;
   const int T = p.T;
-  const int qtile = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y;
+  // every tile of a head on one XCD, each XCD's list longest first
+  int bh, rank;
+  if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
+  const int qtile = n_qtiles - 1 - rank;
   const int b = bh / p.H, h = bh % p.H;
 
   const float* Q = (const float*)p.q + b * p.sq.b + h * p.sq.h;
@@ -173,17 +176,23 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(FwdParams p) {
 }
 
 void launch_attn_fwd_f32(const FwdParams& p, int B, int D, hipStream_t stream) {
-  dim3 grid((p.T + kFwd32BM - 1) / kFwd32BM, B * p.H);
+  const int BH = B * p.H;
+  const int n_qtiles = (p.T + kFwd32BM - 1) / kFwd32BM;
+  const int heads_per_xcd = (BH + 7) / 8;
+  const dim3 grid(8 * n_qtiles * heads_per_xcd);
   LaunchScope scope("attn_fwd_f32", stream);
   switch (D) {
     case 32:
-      hipLaunchKernelGGL((attn_fwd_f32_kernel<32, 64>), grid, dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((attn_fwd_f32_kernel<32, 64>), grid, dim3(256), 0, stream, p, BH, n_qtiles,
+                         heads_per_xcd);
       break;
     case 64:
-      hipLaunchKernelGGL((attn_fwd_f32_kernel<64, 64>), grid, dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((attn_fwd_f32_kernel<64, 64>), grid, dim3(256), 0, stream, p, BH, n_qtiles,
+                         heads_per_xcd);
       break;
     case 128:
-      hipLaunchKernelGGL((attn_fwd_f32_kernel<128, 32>), grid, dim3(256), 0, stream, p);
+      hipLaunchKernelGGL((attn_fwd_f32_kernel<128, 32>), grid, dim3(256), 0, stream, p, BH, n_qtiles,
+                         heads_per_xcd);
       break;
   }
 }
