@@ -1,6 +1,7 @@
 #include "gpt.h"
 
 #include <cmath>
+#include <cstring>
 #include <random>
 
 namespace deers_host {
@@ -38,6 +39,12 @@ Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
 
 Tensor Block::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const {
   const Tensor h = x.add(attn_.forward(rms_norm(x, eps_), cos, sin));
+  return h.add(mlp_.forward(rms_norm(h, eps_)));
+}
+
+Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const {
+  NoGradGuard no_grad;
+  const Tensor h = x_t.add(attn_.decode_step(rms_norm(x_t, eps_), cache, cos, sin));
   return h.add(mlp_.forward(rms_norm(h, eps_)));
 }
 
@@ -120,5 +127,72 @@ Tensor GPT::forward(const Tensor& idx) const {
 }
 
 std::vector<Tensor> GPT::parameters() const { return params_; }
+
+std::vector<KvCache> GPT::new_caches(int64_t batch, int64_t capacity) const {
+  if (capacity > config_.sequence_len) throw std::logic_error("cache capacity exceeds rotary cache");
+  std::vector<KvCache> caches;
+  for (int64_t l = 0; l < config_.n_layer; ++l)
+    caches.push_back(KvCache::create(batch, config_.n_head, capacity, config_.head_dim(), params_[0].dtype()));
+  return caches;
+}
+
+Tensor GPT::decode_step(const Tensor& idx_t, std::vector<KvCache>& caches) const {
+  NoGradGuard no_grad;
+  if (idx_t.layout().ndim() != 2 || idx_t.shape()[1] != 1)
+    throw std::logic_error("decode_step expects token ids with shape [B, 1]");
+  if ((int64_t)caches.size() != config_.n_layer) throw std::logic_error("decode_step: one cache per block");
+  const int64_t B = idx_t.shape()[0];
+  Tensor x = wte_.forward(idx_t);  // [B, 1, C]
+  for (size_t l = 0; l < blocks_.size(); ++l) x = blocks_[l].decode_step(x, caches[l], cos_, sin_);
+  x = rms_norm(x, config_.rms_norm_eps);
+  return x.reshape({B, config_.n_embd}).matmul(lm_head_).reshape({B, 1, config_.vocab_size});
+}
+
+std::vector<int64_t> GPT::generate_greedy(const std::vector<int64_t>& prompt, int64_t batch,
+                                          int64_t n_new) const {
+  if (batch < 1 || prompt.empty() || prompt.size() % (size_t)batch)
+    throw std::logic_error("generate: the prompt is [batch, T0] with T0 >= 1");
+  const int64_t t0 = (int64_t)prompt.size() / batch, total = t0 + n_new, V = config_.vocab_size;
+  std::vector<KvCache> caches = new_caches(batch, total);
+  std::vector<int64_t> out((size_t)(batch * total));
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t t = 0; t < t0; ++t) out[b * total + t] = prompt[b * t0 + t];
+  const bool f16 = params_[0].dtype() == DType::F16;
+  std::vector<char> host((size_t)(batch * V) * size_in_bytes(params_[0].dtype()));
+  std::vector<int64_t> cur((size_t)batch);
+  for (int64_t t = 0; t < total - 1; ++t) {
+    for (int64_t b = 0; b < batch; ++b) cur[b] = out[b * total + t];
+    const Tensor logits = decode_step(Tensor::from_host(cur.data(), {batch, 1}, DType::I64), caches);
+    if (t + 1 < t0) continue;  // still inside the prompt
+    logits.to_host(host.data());
+    for (int64_t b = 0; b < batch; ++b) {
+      int64_t best = 0;
+      float best_v = -INFINITY;
+      for (int64_t v = 0; v < V; ++v) {
+        float x;
+        if (f16) {
+          const uint16_t h = ((const uint16_t*)host.data())[b * V + v];
+          // f16 -> f32 keeps order for finite values once the sign is handled
+          const uint32_t sign = (uint32_t)(h & 0x8000) << 16, mag = h & 0x7fff;
+          uint32_t bits;
+          if (mag >= 0x7c00) bits = sign | 0x7f800000u | ((uint32_t)(mag & 0x3ff) << 13);
+          else if (mag >= 0x0400) bits = sign | ((uint32_t)(mag + 0x1c000) << 13);
+          else {  // zero or subnormal: value = mag * 2^-24
+            x = (float)mag * 5.9604644775390625e-8f;
+            if (sign) x = -x;
+            if (x > best_v) { best_v = x; best = v; }
+            continue;
+          }
+          std::memcpy(&x, &bits, 4);
+        } else {
+          x = ((const float*)host.data())[b * V + v];
+        }
+        if (x > best_v) { best_v = x; best = v; }
+      }
+      out[b * total + t + 1] = best;
+    }
+  }
+  return out;
+}
 
 }  // namespace deers_host

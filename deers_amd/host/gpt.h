@@ -39,6 +39,8 @@ class Block {
  public:
   Block(CausalSelfAttention attn, MLP mlp, double eps);
   Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
+  // One generated position: x_t [B,1,C] at position cache.len (inference, no autograd).
+  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
   std::vector<Tensor> parameters() const;  // attention, then MLP
 
  private:
@@ -67,6 +69,19 @@ class GPT {
 
   Tensor forward(const Tensor& idx) const;  // I64 [B,T] -> logits [B,T,V]
   std::vector<Tensor> parameters() const;
+
+  // Generation with a KV cache per block (f16 models; head width 64 or 128).  The
+  // reference has no cache: its sampling loop re-runs the whole window for every new
+  // token (examples/tinystories_train.rs:250-276).  Here each token costs one pass over
+  // the weights and one streaming pass over the cached keys and values.
+  std::vector<KvCache> new_caches(int64_t batch, int64_t capacity) const;
+  // idx_t I64 [B,1], the token at position caches[0].len -> logits [B,1,V]; equal to row
+  // caches[0].len of forward() on the whole prefix.  Inference only.
+  Tensor decode_step(const Tensor& idx_t, std::vector<KvCache>& caches) const;
+  // Greedy continuation of a prompt (host-side I64 [B, T0], row-major): feeds the prompt
+  // token by token, then appends n_new argmax tokens.  Returns [B, T0 + n_new] on the host.
+  std::vector<int64_t> generate_greedy(const std::vector<int64_t>& prompt, int64_t batch,
+                                       int64_t n_new) const;
   const GPTConfig& config() const { return config_; }
 
  private:

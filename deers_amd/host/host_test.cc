@@ -529,6 +529,77 @@ static int run_gpt(const std::string& dir) {
   return 0;
 }
 
+// Generation with per-block KV caches on an f16 model: the logits of every decode step
+// next to the full causal forward over the same tokens, and a greedy continuation.
+static int run_generate(const std::string& dir) {
+  check(deers_rocm_init(0));
+  GPTConfig cfg;
+  int64_t B, T, n_new;
+  {
+    std::ifstream f(dir + "/case.txt");
+    if (!(f >> cfg.vocab_size >> cfg.sequence_len >> cfg.n_layer >> cfg.n_head >> cfg.n_embd >>
+          cfg.mlp_hidden_dim >> cfg.rms_norm_eps >> cfg.rope_base >> B >> T >> n_new)) {
+      std::printf("FAIL bad case.txt\n");
+      return 2;
+    }
+  }
+  const int64_t C = cfg.n_embd, Hd = cfg.mlp_hidden_dim, V = cfg.vocab_size;
+  std::vector<std::vector<int64_t>> shapes{{V, C}};
+  for (int64_t l = 0; l < cfg.n_layer; ++l)
+    for (auto s : std::vector<std::vector<int64_t>>{{C, C}, {C, C}, {C, C}, {C, C}, {C, Hd}, {Hd, C}}) shapes.push_back(s);
+  shapes.push_back({C, V});
+  std::vector<Tensor> weights;
+  for (size_t i = 0; i < shapes.size(); ++i) {
+    auto bytes = read_file(dir + "/w" + std::to_string(i) + ".bin");
+    if (bytes.size() != (size_t)(shapes[i][0] * shapes[i][1]) * 2) { std::printf("FAIL size of w%zu\n", i); return 2; }
+    weights.push_back(Tensor::from_host(bytes.data(), shapes[i], DType::F16));
+  }
+  auto ids_b = read_file(dir + "/ids.bin");
+  if (ids_b.size() != (size_t)(B * T) * 8) { std::printf("FAIL ids size\n"); return 2; }
+  const int64_t* h_ids = (const int64_t*)ids_b.data();
+  GPT model(cfg, weights);
+  // full forward for comparison
+  {
+    NoGradGuard guard;
+    Tensor logits = model.forward(Tensor::from_host(ids_b.data(), {B, T}, DType::I64));
+    dump(logits, dir + "/logits_full.bin");
+  }
+  // the same tokens one position at a time through the caches
+  std::vector<KvCache> caches = model.new_caches(B, T);
+  std::vector<char> all((size_t)(B * T * V) * 2);
+  std::vector<char> one((size_t)(B * V) * 2);
+  std::vector<int64_t> cur((size_t)B);
+  for (int64_t t = 0; t < T; ++t) {
+    for (int64_t b = 0; b < B; ++b) cur[b] = h_ids[b * T + t];
+    Tensor l = model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), caches);
+    EXPECT((l.shape() == std::vector<int64_t>{B, 1, V}) && !l.requires_grad());
+    l.to_host(one.data());
+    for (int64_t b = 0; b < B; ++b)
+      std::memcpy(all.data() + ((b * T + t) * V) * 2, one.data() + (b * V) * 2, (size_t)V * 2);
+  }
+  EXPECT(caches[0].len == T);
+  write_file(dir + "/logits_steps.bin", all.data(), all.size());
+  bool threw = false;
+  try { model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), caches); } catch (const std::logic_error&) { threw = true; }
+  EXPECT(threw);  // the caches are full
+  // greedy continuation of the first T0 = T/2 tokens
+  const int64_t t0 = T / 2;
+  std::vector<int64_t> prompt((size_t)(B * t0));
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t t = 0; t < t0; ++t) prompt[b * t0 + t] = h_ids[b * T + t];
+  std::vector<int64_t> gen = model.generate_greedy(prompt, B, n_new);
+  EXPECT((int64_t)gen.size() == B * (t0 + n_new));
+  write_file(dir + "/generated.bin", gen.data(), gen.size() * 8);
+  // teacher-forced full forward over what was generated: its argmax must be the next token
+  {
+    NoGradGuard guard;
+    Tensor l = model.forward(Tensor::from_host(gen.data(), {B, t0 + n_new}, DType::I64));
+    dump(l, dir + "/logits_generated.bin");
+  }
+  std::printf("ok generate\n");
+  return 0;
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "graph";
   try {
@@ -546,10 +617,12 @@ int main(int argc, char** argv) {
       if (int rc = run_optim(argv[2])) return rc;
     } else if (mode == "gpt" && argc > 2) {
       if (int rc = run_gpt(argv[2])) return rc;
+    } else if (mode == "generate" && argc > 2) {
+      if (int rc = run_generate(argv[2])) return rc;
     } else if (mode == "module" && argc > 2) {
       if (int rc = run_module(argv[2])) return rc;
     } else {
-      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | optim <dir> | gpt <dir> | module <dir>\n");
+      std::printf("usage: host_test graph | gpu <dir> | lsm <dir> | optim <dir> | gpt <dir> | generate <dir> | module <dir>\n");
       return 2;
     }
   } catch (const std::exception& e) {

@@ -282,3 +282,47 @@ def test_host_gpt_training_step_matches_oracle(tmp_path, cfg, B, T):
         # a gradient entry near zero may pick either sign: compare where the step is decided
         d = np.abs(out(f"w{i}_out.bin", a.shape) - a)
         assert np.quantile(d, 0.999) <= 1e-4 and d.max() <= 2.5 * steps * lr, i
+
+
+@pytest.mark.gpu
+def test_host_gpt_generation_with_kv_caches(tmp_path):
+    """An f16 GPT generating through per-block KV caches: every decode step's logits equal
+    the matching row of the full causal forward (device) and the f32 oracle on the same
+    f16 weights; the greedy continuation picks the teacher-forced argmax at every position."""
+    from oracle import gpt as ogpt
+    from test_oracle_gpt import make_weights
+    cfg = dict(vocab_size=300, sequence_len=48, n_layer=2, n_head=2, n_embd=128, mlp_hidden_dim=256,
+               rms_norm_eps=1e-5, rope_base=10000.0)
+    B, T, n_new = 3, 24, 10
+    rng = np.random.default_rng(23)
+    ids = rng.integers(0, cfg["vocab_size"], (B, T)).astype(np.int64)
+    w = [a.astype(np.float16) for a in make_weights(cfg, 29, dtype=np.float32)]
+    for i, a in enumerate(w):
+        a.tofile(tmp_path / f"w{i}.bin")
+    ids.tofile(tmp_path / "ids.bin")
+    (tmp_path / "case.txt").write_text(
+        f"{cfg['vocab_size']} {cfg['sequence_len']} {cfg['n_layer']} {cfg['n_head']} {cfg['n_embd']} "
+        f"{cfg['mlp_hidden_dim']} {cfg['rms_norm_eps']} {cfg['rope_base']} {B} {T} {n_new}\n")
+    r = _run("generate", str(tmp_path))
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "ok generate" in r.stdout and "all passed" in r.stdout
+    V = cfg["vocab_size"]
+    full = np.fromfile(tmp_path / "logits_full.bin", dtype=np.float16).reshape(B, T, V).astype(np.float32)
+    steps = np.fromfile(tmp_path / "logits_steps.bin", dtype=np.float16).reshape(B, T, V).astype(np.float32)
+    want = ogpt.gpt_forward(cfg, [a.astype(np.float32) for a in w], ids)
+    scale = np.abs(want).max()
+    assert np.abs(full - want).max() <= 2e-2 * scale
+    assert np.abs(steps - want).max() <= 2e-2 * scale
+    assert np.abs(steps - full).max() <= 2e-2 * scale
+    # greedy continuation
+    t0 = T // 2
+    gen = np.fromfile(tmp_path / "generated.bin", dtype=np.int64).reshape(B, t0 + n_new)
+    assert np.array_equal(gen[:, :t0], ids[:, :t0])
+    assert gen.min() >= 0 and gen.max() < V
+    forced = np.fromfile(tmp_path / "logits_generated.bin", dtype=np.float16).reshape(B, t0 + n_new, V)
+    forced = forced.astype(np.float32)
+    for t in range(t0 - 1, t0 + n_new - 1):
+        row = forced[:, t]
+        picked = row[np.arange(B), gen[:, t + 1]]
+        # the generated token is the teacher-forced maximum up to f16 rounding of the logits
+        assert (row.max(axis=1) - picked <= 2e-2 * scale).all(), t
