@@ -289,6 +289,15 @@ def bench_gpt(steps: int, warmup: int):
                        "seq 1024, batch 8 (BASELINE configs[4]); synthetic token ids, random-init weights")
     out["flops_per_step"] = {"matmul": gemm_flops, "attention": attn}
     out["model_tflops"] = (gemm_flops + attn) / (out["ms_per_step"] * 1e-3) / 1e12
+    # greedy generation with KV caches on the same architecture in f16 (32 sequences, 512 cached
+    # tokens, 256 new ones): one decode step = one pass over the weights and the caches
+    rg = subprocess.run([exe, "generate"] + [str(cfg[k]) for k in ("vocab_size", "seq_len", "n_layer",
+                                                                     "n_head", "n_embd", "mlp_hidden")]
+                        + ["32", "512", "256"], capture_output=True, text=True, timeout=600)
+    if rg.returncode == 0:
+        out["generation_f16"] = json.loads(rg.stdout.strip().splitlines()[-1])
+    else:
+        out["generation_f16"] = {"error": rg.stderr.strip()}
     mm = out["kernels"].get("matmul")
     if mm:
         mm["tflops"] = gemm_flops / (mm["ms_per_step"] * 1e-3) / 1e12
@@ -415,7 +424,8 @@ def main():
         try:
             g = bench_gpt(5, 2)
             out["gpt_train_step"] = {k: g[k] for k in ("workload", "ms_per_step", "tokens_per_s",
-                                                       "parameters", "model_tflops", "kernels")}
+                                                       "parameters", "model_tflops", "kernels",
+                                                       "generation_f16")}
         except Exception as e:  # the headline line must not depend on it
             out["gpt_train_step"] = {"error": str(e)}
     if not args.no_cpu_baseline:

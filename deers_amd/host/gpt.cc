@@ -97,9 +97,10 @@ GPT GPT::init_random(const GPTConfig& c, uint64_t seed, DType dtype) {
       std::uniform_real_distribution<float> d(-k, k);
       for (float& x : host) x = d(gen);
     }
-    Tensor t = Tensor::from_host(host.data(), {rows, cols}, DType::F32);
-    if (dtype == DType::F16) throw std::logic_error("GPT::init_random: f16 initialisation is not built");
-    return t;
+    if (dtype == DType::F32) return Tensor::from_host(host.data(), {rows, cols}, DType::F32);
+    std::vector<uint16_t> half(host.size());
+    for (size_t i = 0; i < host.size(); ++i) half[i] = f32_to_f16_bits(host[i]);
+    return Tensor::from_host(half.data(), {rows, cols}, DType::F16);
   };
   std::vector<Tensor> w;
   w.push_back(make(c.vocab_size, c.n_embd, true));

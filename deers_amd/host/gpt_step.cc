@@ -19,7 +19,60 @@
 
 using namespace deers_host;
 
+// gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens:
+// greedy generation with KV caches on an f16 model; times the decode steps that follow
+// the prompt.
+static int run_generate(int argc, char** argv) {
+  if (argc < 11) {
+    std::fprintf(stderr, "usage: gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens\n");
+    return 2;
+  }
+  check(deers_rocm_init(0));
+  GPTConfig cfg;
+  cfg.vocab_size = std::atoll(argv[2]);
+  cfg.sequence_len = std::atoll(argv[3]);
+  cfg.n_layer = std::atoll(argv[4]);
+  cfg.n_head = std::atoll(argv[5]);
+  cfg.n_embd = std::atoll(argv[6]);
+  cfg.mlp_hidden_dim = std::atoll(argv[7]);
+  cfg.rms_norm_eps = 1e-5;
+  cfg.rope_base = 10000.0f;
+  const int64_t B = std::atoll(argv[8]), t0 = std::atoll(argv[9]), n_new = std::atoll(argv[10]);
+  GPT model = GPT::init_random(cfg, 1234, DType::F16);
+  std::mt19937_64 gen(7);
+  std::uniform_int_distribution<int64_t> tok(0, cfg.vocab_size - 1);
+  std::vector<KvCache> caches = model.new_caches(B, t0 + n_new);
+  std::vector<int64_t> cur((size_t)B);
+  auto feed = [&]() {
+    for (auto& x : cur) x = tok(gen);
+    return model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), caches);
+  };
+  for (int64_t t = 0; t < t0; ++t) feed();  // the prompt fills the caches (untimed)
+  check(deers_rocm_sync());
+  const auto s0 = std::chrono::steady_clock::now();
+  for (int64_t t = 0; t < n_new; ++t) feed();
+  check(deers_rocm_sync());
+  const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s0).count() / n_new;
+  int64_t n_params = 0;
+  for (const Tensor& p : model.parameters()) n_params += (int64_t)p.layout().size();
+  const double kv_bytes = 2.0 * cfg.n_layer * B * cfg.n_head * (t0 + n_new / 2.0) * cfg.head_dim() * 2;
+  const double w_bytes = 2.0 * (n_params - cfg.vocab_size * cfg.n_embd);  // every weight but the embedding table
+  std::printf("{\"mode\": \"generate\", \"ms_per_token_step\": %.4f, \"tokens_per_s\": %.1f, \"batch\": %lld, "
+              "\"context\": %lld, \"new_tokens\": %lld, \"bytes_per_step\": %.0f, \"GB_per_s\": %.1f}\n",
+              ms, 1e3 * B / ms, (long long)B, (long long)t0, (long long)n_new, kv_bytes + w_bytes,
+              (kv_bytes + w_bytes) / (ms * 1e-3) / 1e9);
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc > 1 && std::string(argv[1]) == "generate") {
+    try {
+      return run_generate(argc, argv);
+    } catch (const std::exception& e) {
+      std::fprintf(stderr, "gpt_step: %s\n", e.what());
+      return 1;
+    }
+  }
   if (argc < 10) {
     std::fprintf(stderr, "usage: gpt_step vocab seq n_layer n_head n_embd mlp_hidden batch steps warmup\n");
     return 2;

@@ -20,6 +20,8 @@ Tensor empty(const std::vector<int64_t>& shape, DType dtype, bool is_backed) {
   return Tensor(std::move(st), std::move(l), false, nullptr);
 }
 
+}  // namespace
+
 // IEEE binary16 bits of a float, round to nearest even (what f16::from_f32 does).
 uint16_t f32_to_f16_bits(float f) {
   uint32_t x;
@@ -38,6 +40,8 @@ uint16_t f32_to_f16_bits(float f) {
   const uint32_t q = (x - 0x38000000u) >> 13, rem = x & 0x1fffu;
   return (uint16_t)(sign | (q + ((rem > 0x1000u) || (rem == 0x1000u && (q & 1)))));
 }
+
+namespace {
 
 // A [B,H,T,D] view the kernels take as is: unit D stride (alignment is the
 // library's check).  Anything else is compacted.

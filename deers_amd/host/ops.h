@@ -12,6 +12,10 @@
 
 namespace deers_host {
 
+// IEEE binary16 bits of a float, round to nearest even (what f16::from_f32 does); the
+// host compiler has no half type.
+uint16_t f32_to_f16_bits(float f);
+
 class Neg : public TensorOp {
  public:
   explicit Neg(Tensor arg) : arg_(std::move(arg)) {}
