@@ -62,6 +62,16 @@ void launch_adamw(int dtype_f16, void* w, const void* g, void* m, void* v, int64
 void launch_sumsq(int dtype_f16, const void* g, int64_t n, float* partial, float* out,
                   int accumulate, hipStream_t stream);
 void launch_scale(int dtype_f16, void* x, int64_t n, double scale, hipStream_t stream);
+int multi_max_tensors();
+int64_t multi_blocks(int dtype_f16, int64_t n);
+void launch_adamw_multi(int dtype_f16, int count, void* const* w, const void* const* g, void* const* m,
+                        void* const* v, const int64_t* sizes, double lr, double beta1, double beta2,
+                        double eps, double weight_decay, int step, double grad_scale,
+                        hipStream_t stream);
+int launch_sumsq_multi(int dtype_f16, int count, const void* const* x, const int64_t* sizes,
+                       float* partial, hipStream_t stream);
+void launch_sumsq_final(const float* partial, int n_partial, float* out, int accumulate,
+                        hipStream_t stream);
 void launch_copy_view(int dtype_f16, const void* src, const int64_t* src_strides, void* dst,
                       const int64_t* dst_strides, const int64_t* shape, int ndim,
                       hipStream_t stream);
@@ -892,6 +902,100 @@ int deers_rocm_sum_squares(int dtype, const void* x, int64_t n, float* total, in
   void* ws = nullptr;
   if (int rc = workspace(deers::sumsq_partial_count() * sizeof(float), &ws)) return rc;
   deers::launch_sumsq(dtype == DEERS_ROCM_F16, x, n, (float*)ws, total, accumulate, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// Tensors the multi-tensor kernels take: non-empty and 16-byte aligned.
+static bool multi_ok(const void* p, int64_t n) { return n > 0 && ((uintptr_t)p & 15) == 0; }
+
+int deers_rocm_adamw_step_multi(int dtype, int n_tensors, void* const* w, const void* const* grad,
+                                void* const* m, void* const* v, const int64_t* sizes, double lr,
+                                double beta1, double beta2, double eps, double weight_decay,
+                                int64_t step, double grad_scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n_tensors < 0) return fail(DEERS_ROCM_ERR_ARG, "adamw_step_multi: negative tensor count");
+  if (step < 1 || step > INT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "adamw_step_multi: step counts from 1 (got %lld)", (long long)step);
+  if (n_tensors == 0) return DEERS_ROCM_OK;
+  if (!w || !grad || !m || !v || !sizes) return fail(DEERS_ROCM_ERR_ARG, "adamw_step_multi: null table");
+  const int f16 = dtype == DEERS_ROCM_F16;
+  for (int i = 0; i < n_tensors; ++i) {
+    if (sizes[i] < 0) return fail(DEERS_ROCM_ERR_ARG, "adamw_step_multi: tensor %d has a negative size", i);
+    if (sizes[i] > 0 && (!w[i] || !grad[i] || !m[i] || !v[i]))
+      return fail(DEERS_ROCM_ERR_ARG, "adamw_step_multi: tensor %d has a null pointer", i);
+  }
+  // groups of aligned tensors go out together; an unaligned one takes the single-tensor kernels
+  const int cap = deers::multi_max_tensors();
+  std::vector<void*> gw, gm, gv;
+  std::vector<const void*> gg;
+  std::vector<int64_t> gn;
+  int64_t group_blocks = 0;
+  auto flush = [&]() {
+    if (gw.empty()) return;
+    deers::launch_adamw_multi(f16, (int)gw.size(), gw.data(), gg.data(), gm.data(), gv.data(), gn.data(), lr,
+                              beta1, beta2, eps, weight_decay, (int)step, grad_scale, g_rt.stream);
+    gw.clear(); gg.clear(); gm.clear(); gv.clear(); gn.clear();
+    group_blocks = 0;
+  };
+  for (int i = 0; i < n_tensors; ++i) {
+    if (sizes[i] == 0) continue;
+    if (multi_ok(w[i], sizes[i]) && multi_ok(grad[i], sizes[i]) && multi_ok(m[i], sizes[i]) &&
+        multi_ok(v[i], sizes[i])) {
+      const int64_t nb = deers::multi_blocks(f16, sizes[i]);
+      if ((int)gw.size() == cap || group_blocks + nb > INT32_MAX / 2) flush();
+      gw.push_back(w[i]); gg.push_back(grad[i]); gm.push_back(m[i]); gv.push_back(v[i]); gn.push_back(sizes[i]);
+      group_blocks += nb;
+    } else {
+      deers::launch_adamw(f16, w[i], grad[i], m[i], v[i], sizes[i], lr, beta1, beta2, eps, weight_decay,
+                          (int)step, grad_scale, g_rt.stream);
+    }
+  }
+  flush();
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_sum_squares_multi(int dtype, int n_tensors, const void* const* x, const int64_t* sizes,
+                                 float* total, int accumulate) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n_tensors < 0) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: negative tensor count");
+  if (!total) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: null total");
+  if (n_tensors > 0 && (!x || !sizes)) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: null table");
+  const int f16 = dtype == DEERS_ROCM_F16;
+  int64_t blocks = 0;
+  for (int i = 0; i < n_tensors; ++i) {
+    if (sizes[i] < 0) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: tensor %d has a negative size", i);
+    if (sizes[i] > 0 && !x[i]) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: tensor %d is null", i);
+    if (sizes[i] > 0 && ((uintptr_t)x[i] & 15))
+      return fail(DEERS_ROCM_ERR_LAYOUT, "sum_squares_multi: tensor %d is not 16-byte aligned; use "
+                  "deers_rocm_sum_squares for it", i);
+    blocks += deers::multi_blocks(f16, sizes[i]);
+  }
+  if (blocks > INT32_MAX / 2) return fail(DEERS_ROCM_ERR_ARG, "sum_squares_multi: too many elements for one call");
+  void* ws = nullptr;  // one partial per block of every tensor, then one fixed-order sum
+  if (int rc = workspace((size_t)(blocks > 0 ? blocks : 1) * sizeof(float), &ws)) return rc;
+  float* partial = (float*)ws;
+  const int cap = deers::multi_max_tensors();
+  int written = 0;
+  std::vector<const void*> gx;
+  std::vector<int64_t> gn;
+  auto flush = [&]() {
+    if (gx.empty()) return;
+    written += deers::launch_sumsq_multi(f16, (int)gx.size(), gx.data(), gn.data(), partial + written, g_rt.stream);
+    gx.clear(); gn.clear();
+  };
+  for (int i = 0; i < n_tensors; ++i) {
+    if (sizes[i] == 0) continue;
+    if ((int)gx.size() == cap) flush();
+    gx.push_back(x[i]); gn.push_back(sizes[i]);
+  }
+  flush();
+  deers::launch_sumsq_final(partial, written, total, accumulate, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -1,6 +1,7 @@
 #include "optim.h"
 
 #include <cmath>
+#include <cstdint>
 
 #include "../../include/deers_rocm.h"
 
@@ -36,20 +37,41 @@ void AdamW::backward_step(const Tensor& loss) {
 
 void AdamW::step_with_grads(const GradientStore& grads, double grad_scale) {
   step_ += 1;  // src/optim.rs:215
+  // every parameter that has a gradient, gathered per type for the multi-tensor launch
+  // (the compacted gradients are kept alive in `held` until the launches are enqueued)
+  struct Group {
+    std::vector<void*> w, m, v;
+    std::vector<const void*> g;
+    std::vector<int64_t> n;
+  };
+  Group groups[2];
+  std::vector<Tensor> held;
   for (const Tensor& param : parameters_) {
     const Tensor* found = grads.get(param.id());
     if (!found) continue;
     if (!param.is_compact()) throw std::logic_error("AdamW: parameters must be compact");
     if (found->shape() != param.shape() || found->dtype() != param.dtype())
       throw std::logic_error("AdamW: gradient does not match its parameter");
-    const Tensor grad = found->compact();
+    if (param.dtype() != DType::F16 && param.dtype() != DType::F32)
+      throw std::logic_error("AdamW: parameters are f16 or f32");
+    held.push_back(found->compact());
     auto m = m_.find(param.id());
     if (m == m_.end()) m = m_.emplace(param.id(), param.zeros_like()).first;
     auto v = v_.find(param.id());
     if (v == v_.end()) v = v_.emplace(param.id(), param.zeros_like()).first;
-    check(deers_rocm_adamw_step((int)param.dtype(), param.data(), grad.data(), m->second.data(),
-                                v->second.data(), (int64_t)param.layout().size(), lr_, beta1_,
-                                beta2_, eps_, weight_decay_, (int64_t)step_, grad_scale));
+    Group& grp = groups[param.dtype() == DType::F16 ? 0 : 1];
+    grp.w.push_back(param.data());
+    grp.g.push_back(held.back().data());
+    grp.m.push_back(m->second.data());
+    grp.v.push_back(v->second.data());
+    grp.n.push_back((int64_t)param.layout().size());
+  }
+  for (int t = 0; t < 2; ++t) {
+    const Group& grp = groups[t];
+    if (grp.w.empty()) continue;
+    check(deers_rocm_adamw_step_multi(t == 0 ? DEERS_ROCM_F16 : DEERS_ROCM_F32, (int)grp.w.size(),
+                                      grp.w.data(), grp.g.data(), grp.m.data(), grp.v.data(), grp.n.data(),
+                                      lr_, beta1_, beta2_, eps_, weight_decay_, (int64_t)step_, grad_scale));
   }
 }
 
@@ -59,13 +81,30 @@ float clip_grad_scale(const std::vector<Tensor>& parameters, const GradientStore
   if (scale) *scale = 1.0;
   if (parameters.empty()) return 0.0f;
   Tensor total = Tensor::zeros({1}, DType::F32);
+  // all gradients of a type in one reduction; one that is not 16-byte aligned (a view
+  // into a larger buffer) goes through the single-tensor call
+  std::vector<Tensor> held;
+  std::vector<const void*> ptrs[2];
+  std::vector<int64_t> sizes[2];
   for (const Tensor& p : parameters) {
     const Tensor* g = grads.get(p.id());
     if (!g) continue;
-    const Tensor gc = g->compact();
-    check(deers_rocm_sum_squares((int)gc.dtype(), gc.data(), (int64_t)gc.layout().size(),
-                                 (float*)total.data(), 1));
+    held.push_back(g->compact());
+    const Tensor& gc = held.back();
+    const int64_t n = (int64_t)gc.layout().size();
+    if (n == 0) continue;
+    if ((uintptr_t)gc.data() & 15) {
+      check(deers_rocm_sum_squares((int)gc.dtype(), gc.data(), n, (float*)total.data(), 1));
+      continue;
+    }
+    const int t = gc.dtype() == DType::F16 ? 0 : 1;
+    ptrs[t].push_back(gc.data());
+    sizes[t].push_back(n);
   }
+  for (int t = 0; t < 2; ++t)
+    if (!ptrs[t].empty())
+      check(deers_rocm_sum_squares_multi(t == 0 ? DEERS_ROCM_F16 : DEERS_ROCM_F32, (int)ptrs[t].size(),
+                                         ptrs[t].data(), sizes[t].data(), (float*)total.data(), 1));
   float sum = 0.0f;
   total.to_host(&sum);  // the one synchronisation, as to_vec is in the reference
   const float norm = std::sqrt(sum);

@@ -280,6 +280,27 @@ def sum_squares_raw(dtype, x, n, total, accumulate=False):
                                          total, ctypes.c_int(1 if accumulate else 0)))
 
 
+def _ptr_table(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*[p.value if isinstance(p, ctypes.c_void_p) else p for p in ptrs])
+
+
+def adamw_step_multi_raw(dtype, w, grad, m, v, sizes, lr, beta1, beta2, eps, weight_decay, step,
+                         grad_scale=1.0):
+    n = len(sizes)
+    _check(load().deers_rocm_adamw_step_multi(
+        ctypes.c_int(dtype_code(dtype)), ctypes.c_int(n), _ptr_table(w), _ptr_table(grad), _ptr_table(m),
+        _ptr_table(v), (ctypes.c_int64 * n)(*sizes), ctypes.c_double(lr), ctypes.c_double(beta1),
+        ctypes.c_double(beta2), ctypes.c_double(eps), ctypes.c_double(weight_decay), ctypes.c_int64(step),
+        ctypes.c_double(grad_scale)))
+
+
+def sum_squares_multi_raw(dtype, x, sizes, total, accumulate=False):
+    n = len(sizes)
+    _check(load().deers_rocm_sum_squares_multi(ctypes.c_int(dtype_code(dtype)), ctypes.c_int(n),
+                                               _ptr_table(x), (ctypes.c_int64 * n)(*sizes), total,
+                                               ctypes.c_int(1 if accumulate else 0)))
+
+
 def scale_raw(dtype, x, n, scale):
     _check(load().deers_rocm_scale(ctypes.c_int(dtype_code(dtype)), x, ctypes.c_int64(n),
                                    ctypes.c_double(scale)))

@@ -267,6 +267,21 @@ int deers_rocm_cross_entropy_bwd(int dtype, const void* logits, const int64_t* t
 int deers_rocm_adamw_step(int dtype, void* w, const void* grad, void* m, void* v, int64_t n,
                           double lr, double beta1, double beta2, double eps, double weight_decay,
                           int64_t step, double grad_scale);
+/* The same update for n_tensors parameter tensors in as few launches as their number
+ * allows (48 tensors per launch): w, grad, m, v are host arrays of device pointers, sizes
+ * the element counts; every tensor gets exactly what deers_rocm_adamw_step would give it.
+ * This is the whole parameter loop of AdamW::step_with_grads (src/optim.rs:221-247) for
+ * the parameters that have a gradient. */
+int deers_rocm_adamw_step_multi(int dtype, int n_tensors, void* const* w, const void* const* grad,
+                                void* const* m, void* const* v, const int64_t* sizes, double lr,
+                                double beta1, double beta2, double eps, double weight_decay,
+                                int64_t step, double grad_scale);
+/* *total = or += the sum of squares of all the tensors, the whole reduction loop of
+ * clip_grad_norm (src/optim.rs:270-277) in one or two launches plus a fixed-order final
+ * sum; tensors must be 16-byte aligned (DEERS_ROCM_ERR_LAYOUT otherwise).  Reproducible;
+ * the order of additions differs from per-tensor deers_rocm_sum_squares calls. */
+int deers_rocm_sum_squares_multi(int dtype, int n_tensors, const void* const* x, const int64_t* sizes,
+                                 float* total, int accumulate);
 /* *total (a float in device memory) = or += sum of x[i]^2 in f32, the reduction of
  * clip_grad_norm (src/optim.rs:270-277) for one gradient; the partition and the order
  * of additions are fixed, so repeated calls give the same bits. */

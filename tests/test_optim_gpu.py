@@ -171,3 +171,51 @@ def test_optimizer_argument_errors():
         rocm.sum_squares_raw(np.float32, buf.ptr, 16, ctypes.c_void_p())
     with pytest.raises(rocm.RocmError):
         rocm.scale_raw(np.float32, buf.ptr, -1, 2.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_multi_tensor_step_and_norm_equal_the_single_tensor_calls(dtype):
+    # 110 tensors (more than one launch's worth) of ragged sizes, one of them a view that is
+    # not 16-byte aligned: every tensor gets exactly the bits of its own single-tensor call
+    rng = np.random.default_rng(57)
+    sizes = [1, 3, 4, 5, 768, 4096 + 1, 3 * 4096, 100_000] + [int(s) for s in rng.integers(1, 30_000, 102)]
+    eps = 1e-8 if dtype == np.float32 else 1e-3
+    item = np.dtype(dtype).itemsize
+    states = [_state(n + 8, dtype, 100 + i) for i, n in enumerate(sizes)]
+    skew = [0] * len(sizes)
+    skew[6] = 1  # an unaligned view
+    a = [[rocm.DeviceBuffer.from_numpy(x) for x in st] for st in states]
+    b = [[rocm.DeviceBuffer.from_numpy(x) for x in st] for st in states]
+    at = lambda buf, k: ctypes.c_void_p(buf.ptr.value + k * item)
+    rocm.adamw_step_multi_raw(dtype, *[[at(t[j], skew[i]) for i, t in enumerate(a)] for j in range(4)], sizes,
+                              1e-2, 0.9, 0.95, eps, 0.1, 5, grad_scale=0.5)
+    for i, (t, n) in enumerate(zip(b, sizes)):
+        rocm.adamw_step_raw(dtype, *(at(x, skew[i]) for x in t), n, 1e-2, 0.9, 0.95, eps, 0.1, 5, grad_scale=0.5)
+    for i, (ta, tb) in enumerate(zip(a, b)):
+        for j in range(4):
+            assert _same_bits(ta[j].numpy(), tb[j].numpy()), (i, j)
+    # and against the oracle for a few of them
+    for i in (0, 4, 6, 7, 50):
+        w, g, m, v = (x[skew[i]:skew[i] + sizes[i]] for x in states[i])
+        gs = (g * oracle._scalar(0.5, dtype)).astype(dtype)
+        ww, wm, wv = oracle.adamw_step(w, gs, m, v, 5, 1e-2, (0.9, 0.95), eps, 0.1, dtype=dtype)
+        assert _same_bits(a[i][0].numpy()[skew[i]:skew[i] + sizes[i]], ww)
+        assert _same_bits(a[i][2].numpy()[skew[i]:skew[i] + sizes[i]], wm)
+    # the norm: all aligned gradients in one reduction
+    ptrs = [t[1].ptr for i, t in enumerate(a) if skew[i] == 0]
+    ns = [n + 8 for i, n in enumerate(sizes) if skew[i] == 0]
+    total = rocm.DeviceBuffer((1,), np.float32)
+    rocm.sum_squares_multi_raw(dtype, ptrs, ns, total.ptr)
+    want = sum(float((st[1].astype(np.float64) ** 2).sum()) for i, st in enumerate(states) if skew[i] == 0)
+    got = float(total.numpy()[0])
+    assert abs(got - want) <= 1e-6 * want
+    again = rocm.DeviceBuffer((1,), np.float32)
+    rocm.sum_squares_multi_raw(dtype, ptrs, ns, again.ptr)
+    assert again.numpy()[0] == total.numpy()[0]
+    rocm.sum_squares_multi_raw(dtype, ptrs, ns, again.ptr, accumulate=True)
+    assert abs(float(again.numpy()[0]) - 2 * got) <= 1e-6 * got
+    with pytest.raises(rocm.RocmError):
+        rocm.sum_squares_multi_raw(dtype, [at(a[0][1], 1)], [4], total.ptr)
+    rocm.sum_squares_multi_raw(dtype, [], [], total.ptr)
+    assert total.numpy()[0] == 0.0
