@@ -343,6 +343,8 @@ __global__ __launch_bounds__(256) void mean_rows_kernel(const float* row_loss, i
 // Backward: dlogits[i, c] = (exp(x[i, c] - lse_i) - [c == target_i]) * upstream / N, one
 // streaming pass over the flat [N * V] array in aligned 16-byte chunks (a chunk may
 // straddle two rows).  `upstream` is the gradient of the scalar loss, in device memory.
+constexpr int kCeSlab = 1024;  // 16-byte chunks per block
+
 template <typename T>
 __global__ __launch_bounds__(256) void cross_entropy_bwd_kernel(
     const T* logits, const int64_t* targets, const float* row_lse, const float* upstream, T* dlogits,
@@ -359,9 +361,13 @@ __global__ __launch_bounds__(256) void cross_entropy_bwd_kernel(
     return (p - (targets[r] == c ? 1.0f : 0.0f)) * g;
   };
   const int64_t n_chunks = total > lead ? (total - lead) / kEpc : 0;
-  const int64_t stride = (int64_t)gridDim.x * 256;
   const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  for (int64_t c = tid; c < n_chunks; c += stride) {
+  // each block owns one contiguous slab of kCeSlab chunks (16 KB per array): with a read
+  // and a write stream, neighbouring blocks on neighbouring addresses move more bytes per
+  // second than a grid-stride sweep
+  const int64_t slab0 = (int64_t)blockIdx.x * kCeSlab;
+  const int64_t slab1 = slab0 + kCeSlab < n_chunks ? slab0 + kCeSlab : n_chunks;
+  for (int64_t c = slab0 + threadIdx.x; c < slab1; c += 256) {
     const int64_t flat0 = lead + c * kEpc;
     const Vec16<T> vx = load16_stream(logits + flat0);
     // one division per chunk; the elements after a row boundary step to the next row
@@ -529,7 +535,7 @@ void launch_cross_entropy_bwd(int dtype_f16, const void* logits, const int64_t* 
   const bool same_phase = (((uintptr_t)logits ^ (uintptr_t)dlogits) & 15) == 0;
   if (dtype_f16) {
     if (same_phase)
-      hipLaunchKernelGGL(cross_entropy_bwd_kernel<half_t>, dim3(stream_grid(total / 8 + 16)), dim3(256),
+      hipLaunchKernelGGL(cross_entropy_bwd_kernel<half_t>, dim3((unsigned)(total / 8 / kCeSlab + 1)), dim3(256),
                          0, stream, (const half_t*)logits, targets, row_lse, upstream,
                          (half_t*)dlogits, n_rows, width, inv_n);
     else
@@ -538,7 +544,7 @@ void launch_cross_entropy_bwd(int dtype_f16, const void* logits, const int64_t* 
                          (half_t*)dlogits, n_rows, width, inv_n);
   } else {
     if (same_phase)
-      hipLaunchKernelGGL(cross_entropy_bwd_kernel<float>, dim3(stream_grid(total / 4 + 16)), dim3(256),
+      hipLaunchKernelGGL(cross_entropy_bwd_kernel<float>, dim3((unsigned)(total / 4 / kCeSlab + 1)), dim3(256),
                          0, stream, (const float*)logits, targets, row_lse, upstream, (float*)dlogits,
                          n_rows, width, inv_n);
     else
