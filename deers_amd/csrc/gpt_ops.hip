@@ -413,6 +413,70 @@ __global__ __launch_bounds__(256) void cross_entropy_bwd_unaligned_kernel(
   }
 }
 
+// ---- argmax over the last axis: the greedy sampling step, kept on the device so that a
+// generation loop never waits for the host ----
+// One workgroup per row; ties go to the lowest index; NaNs are never selected.
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const T* x, int64_t* out, int width) {
+  __shared__ float red_v[4];
+  __shared__ int red_i[4];
+  constexpr int kEpc = 16 / sizeof(T);
+  constexpr int kInFlight = 4;
+  const T* row = x + (int64_t)blockIdx.x * width;
+  // 16-byte chunks counted from the 16-byte boundary at or before the row start (rows
+  // start at any element), the two edge chunks masked; several chunks in flight per
+  // thread: a row of 50257 logits is otherwise a chain of dependent round trips
+  const int head = (int)((uintptr_t)row & 15) / (int)sizeof(T);
+  const T* base = row - head;
+  const int n_chunks = (head + width + kEpc - 1) / kEpc;
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c0 = threadIdx.x; c0 < n_chunks; c0 += 256 * kInFlight) {
+    Vec16<T> v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      v[u] = Vec16<T>{};
+      if (c0 + 256 * u < n_chunks) v[u] = load16_stream(base + (c0 + 256 * u) * kEpc);
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int lo = (c0 + 256 * u) * kEpc - head;  // row position of element 0 of the chunk
+#pragma unroll
+      for (int e = 0; e < kEpc; ++e) {
+        const int c = lo + e;
+        const float f = (float)v[u].e[e];
+        // positions ascend within a thread, so a strict comparison keeps the lowest index
+        if (c >= 0 && c < width && c0 + 256 * u < n_chunks && f > best) {
+          best = f;
+          best_i = c;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float v2 = __shfl_xor(best, off, 64);
+    const int i2 = __shfl_xor(best_i, off, 64);
+    if (v2 > best || (v2 == best && i2 < best_i)) {
+      best = v2;
+      best_i = i2;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    red_v[threadIdx.x >> 6] = best;
+    red_i[threadIdx.x >> 6] = best_i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (red_v[w] > best || (red_v[w] == best && red_i[w] < best_i)) {
+        best = red_v[w];
+        best_i = red_i[w];
+      }
+    out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;  // a row of NaNs / -inf picks 0
+  }
+}
+
 unsigned stream_grid(int64_t work_items) {
   const int64_t blocks = (work_items + 255) / 256;
   const int64_t cap = 256 * 16;
@@ -510,6 +574,17 @@ void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int
     if (bwd) relu_sq_t<float, true>((const float*)x, (const float*)dy, (float*)out, n, stream);
     else relu_sq_t<float, false>((const float*)x, nullptr, (float*)out, n, stream);
   }
+}
+
+void launch_argmax_rows(int dtype_f16, const void* x, int64_t* out, int64_t outer, int width,
+                        hipStream_t stream) {
+  LaunchScope scope("argmax_rows", stream);
+  if (dtype_f16)
+    hipLaunchKernelGGL(argmax_rows_kernel<half_t>, dim3((unsigned)outer), dim3(256), 0, stream,
+                       (const half_t*)x, out, width);
+  else
+    hipLaunchKernelGGL(argmax_rows_kernel<float>, dim3((unsigned)outer), dim3(256), 0, stream,
+                       (const float*)x, out, width);
 }
 
 void launch_cross_entropy_fwd(int dtype_f16, const void* logits, const int64_t* targets, float* row_lse,

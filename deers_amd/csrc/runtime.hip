@@ -49,6 +49,8 @@ void launch_rms_norm(int dtype_f16, const void* x, const void* dy, void* out, in
                      float eps, int bwd, hipStream_t stream);
 void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int64_t n, int bwd,
                     hipStream_t stream);
+void launch_argmax_rows(int dtype_f16, const void* x, int64_t* out, int64_t outer, int width,
+                        hipStream_t stream);
 void launch_cross_entropy_fwd(int dtype_f16, const void* logits, const int64_t* targets, float* row_lse,
                               float* row_loss, float* loss, int64_t n_rows, int width, int* flag,
                               hipStream_t stream);
@@ -837,6 +839,17 @@ int deers_rocm_relu_sq_bwd(int dtype, const void* x, const void* dy, void* dx, i
   if (n == 0) return DEERS_ROCM_OK;
   if (!x || !dy || !dx) return fail(DEERS_ROCM_ERR_ARG, "relu_sq_bwd: null pointer");
   deers::launch_relu_sq(dtype == DEERS_ROCM_F16, x, dy, dx, n, 1, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_argmax_rows(int dtype, const void* x, int64_t* out, int64_t outer, int64_t inner) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("argmax_rows", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !out) return fail(DEERS_ROCM_ERR_ARG, "argmax_rows: null pointer");
+  deers::launch_argmax_rows(dtype == DEERS_ROCM_F16, x, out, outer, (int)inner, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -1,5 +1,7 @@
 #include "gpt.h"
 
+#include "../../include/deers_rocm.h"
+
 #include <cmath>
 #include <cstring>
 #include <random>
@@ -153,45 +155,41 @@ std::vector<int64_t> GPT::generate_greedy(const std::vector<int64_t>& prompt, in
                                           int64_t n_new) const {
   if (batch < 1 || prompt.empty() || prompt.size() % (size_t)batch)
     throw std::logic_error("generate: the prompt is [batch, T0] with T0 >= 1");
+  NoGradGuard no_grad;
   const int64_t t0 = (int64_t)prompt.size() / batch, total = t0 + n_new, V = config_.vocab_size;
   std::vector<KvCache> caches = new_caches(batch, total);
+  // the prompt goes up once, position-major, so that every step's ids are one contiguous
+  // [batch] slice; after it each step's ids are the previous step's argmax, picked on the
+  // device: nothing in the loop waits for the host
+  std::vector<int64_t> by_pos((size_t)(t0 * batch));
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t t = 0; t < t0; ++t) by_pos[t * batch + b] = prompt[b * t0 + t];
+  const Tensor prompt_dev = Tensor::from_host(by_pos.data(), {t0 * batch}, DType::I64);
+  std::vector<Tensor> picked;  // one [batch] id tensor per generated position
+  for (int64_t t = 0; t < total - 1; ++t) {
+    Tensor ids_t;
+    if (t < t0) {
+      // a [batch, 1] tensor of its own (layouts with an offset do not count as compact)
+      auto st = std::make_shared<RocmStorage>((size_t)batch, DType::I64, true);
+      ids_t = Tensor(st, Layout({batch, 1}), false, nullptr);
+      check(deers_rocm_dtod(ids_t.data(), (const char*)prompt_dev.data() + t * batch * 8, (size_t)batch * 8));
+    } else {
+      ids_t = Tensor(picked.back().storage(), Layout({batch, 1}), false, nullptr);
+    }
+    const Tensor logits = decode_step(ids_t, caches);  // [batch, 1, V], compact
+    if (t + 1 < t0) continue;                           // still inside the prompt
+    auto st = std::make_shared<RocmStorage>((size_t)batch, DType::I64, true);
+    Tensor next(st, Layout({batch}), false, nullptr);
+    check(deers_rocm_argmax_rows((int)logits.dtype(), logits.data(), (int64_t*)next.data(), batch, V));
+    picked.push_back(next);
+  }
   std::vector<int64_t> out((size_t)(batch * total));
   for (int64_t b = 0; b < batch; ++b)
     for (int64_t t = 0; t < t0; ++t) out[b * total + t] = prompt[b * t0 + t];
-  const bool f16 = params_[0].dtype() == DType::F16;
-  std::vector<char> host((size_t)(batch * V) * size_in_bytes(params_[0].dtype()));
-  std::vector<int64_t> cur((size_t)batch);
-  for (int64_t t = 0; t < total - 1; ++t) {
-    for (int64_t b = 0; b < batch; ++b) cur[b] = out[b * total + t];
-    const Tensor logits = decode_step(Tensor::from_host(cur.data(), {batch, 1}, DType::I64), caches);
-    if (t + 1 < t0) continue;  // still inside the prompt
-    logits.to_host(host.data());
-    for (int64_t b = 0; b < batch; ++b) {
-      int64_t best = 0;
-      float best_v = -INFINITY;
-      for (int64_t v = 0; v < V; ++v) {
-        float x;
-        if (f16) {
-          const uint16_t h = ((const uint16_t*)host.data())[b * V + v];
-          // f16 -> f32 keeps order for finite values once the sign is handled
-          const uint32_t sign = (uint32_t)(h & 0x8000) << 16, mag = h & 0x7fff;
-          uint32_t bits;
-          if (mag >= 0x7c00) bits = sign | 0x7f800000u | ((uint32_t)(mag & 0x3ff) << 13);
-          else if (mag >= 0x0400) bits = sign | ((uint32_t)(mag + 0x1c000) << 13);
-          else {  // zero or subnormal: value = mag * 2^-24
-            x = (float)mag * 5.9604644775390625e-8f;
-            if (sign) x = -x;
-            if (x > best_v) { best_v = x; best = v; }
-            continue;
-          }
-          std::memcpy(&x, &bits, 4);
-        } else {
-          x = ((const float*)host.data())[b * V + v];
-        }
-        if (x > best_v) { best_v = x; best = v; }
-      }
-      out[b * total + t + 1] = best;
-    }
+  std::vector<int64_t> col((size_t)batch);
+  for (size_t i = 0; i < picked.size(); ++i) {
+    picked[i].to_host(col.data());
+    for (int64_t b = 0; b < batch; ++b) out[b * total + t0 + (int64_t)i] = col[b];
   }
   return out;
 }

@@ -47,20 +47,60 @@ static int run_generate(int argc, char** argv) {
     for (auto& x : cur) x = tok(gen);
     return model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), caches);
   };
-  for (int64_t t = 0; t < t0; ++t) feed();  // the prompt fills the caches (untimed)
+  Tensor logits;
+  for (int64_t t = 0; t < t0; ++t) logits = feed();  // the prompt fills the caches (untimed)
   check(deers_rocm_sync());
+  // the generated part: every step's ids are the previous step's argmax, picked on the
+  // device, so the host only enqueues
   const auto s0 = std::chrono::steady_clock::now();
-  for (int64_t t = 0; t < n_new; ++t) feed();
+  for (int64_t t = 0; t < n_new; ++t) {
+    auto st = std::make_shared<RocmStorage>((size_t)B, DType::I64, true);
+    Tensor next(st, Layout({B, 1}), false, nullptr);
+    check(deers_rocm_argmax_rows((int)logits.dtype(), logits.data(), (int64_t*)next.data(), B, cfg.vocab_size));
+    logits = model.decode_step(next, caches);
+  }
   check(deers_rocm_sync());
   const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s0).count() / n_new;
+  // a few more steps with every launch bracketed by events: device time per kernel family
+  std::string kernels = "{";
+  {
+    const int prof_steps = 8;
+    std::vector<KvCache> c2 = model.new_caches(B, t0 + prof_steps);
+    for (int64_t t = 0; t < t0; ++t) {
+      for (auto& x : cur) x = tok(gen);
+      logits = model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), c2);
+    }
+    check(deers_rocm_sync());
+    check(deers_rocm_profile_enable(1));
+    for (int t = 0; t < prof_steps; ++t) {
+      auto st = std::make_shared<RocmStorage>((size_t)B, DType::I64, true);
+      Tensor next(st, Layout({B, 1}), false, nullptr);
+      check(deers_rocm_argmax_rows((int)logits.dtype(), logits.data(), (int64_t*)next.data(), B, cfg.vocab_size));
+      logits = model.decode_step(next, c2);
+    }
+    int rows = 0;
+    check(deers_rocm_profile_collect(&rows));
+    for (int r = 0; r < rows; ++r) {
+      const char* name = nullptr;
+      int64_t calls = 0;
+      float total_ms = 0;
+      check(deers_rocm_profile_row(r, &name, &calls, &total_ms));
+      char buf[256];
+      std::snprintf(buf, sizeof(buf), "%s\"%s\": {\"calls_per_step\": %.1f, \"us_per_step\": %.1f}", r ? ", " : "",
+                    name, (double)calls / prof_steps, 1e3 * total_ms / prof_steps);
+      kernels += buf;
+    }
+    check(deers_rocm_profile_enable(0));
+  }
+  kernels += "}";
   int64_t n_params = 0;
   for (const Tensor& p : model.parameters()) n_params += (int64_t)p.layout().size();
   const double kv_bytes = 2.0 * cfg.n_layer * B * cfg.n_head * (t0 + n_new / 2.0) * cfg.head_dim() * 2;
   const double w_bytes = 2.0 * (n_params - cfg.vocab_size * cfg.n_embd);  // every weight but the embedding table
   std::printf("{\"mode\": \"generate\", \"ms_per_token_step\": %.4f, \"tokens_per_s\": %.1f, \"batch\": %lld, "
-              "\"context\": %lld, \"new_tokens\": %lld, \"bytes_per_step\": %.0f, \"GB_per_s\": %.1f}\n",
+              "\"context\": %lld, \"new_tokens\": %lld, \"bytes_per_step\": %.0f, \"GB_per_s\": %.1f, \"kernels\": %s}\n",
               ms, 1e3 * B / ms, (long long)B, (long long)t0, (long long)n_new, kv_bytes + w_bytes,
-              (kv_bytes + w_bytes) / (ms * 1e-3) / 1e9);
+              (kv_bytes + w_bytes) / (ms * 1e-3) / 1e9, kernels.c_str());
   return 0;
 }
 

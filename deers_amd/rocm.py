@@ -256,6 +256,11 @@ def relu_sq_bwd_raw(dtype, x, dy, dx, n):
     _check(load().deers_rocm_relu_sq_bwd(ctypes.c_int(dtype_code(dtype)), x, dy, dx, ctypes.c_int64(n)))
 
 
+def argmax_rows_raw(dtype, x, out, outer, inner):
+    _check(load().deers_rocm_argmax_rows(ctypes.c_int(dtype_code(dtype)), x, out, ctypes.c_int64(outer),
+                                         ctypes.c_int64(inner)))
+
+
 def cross_entropy_fwd_raw(dtype, logits, targets, row_lse, loss, n_rows, n_classes):
     _check(load().deers_rocm_cross_entropy_fwd(ctypes.c_int(dtype_code(dtype)), logits, targets, row_lse,
                                                loss, ctypes.c_int64(n_rows), ctypes.c_int64(n_classes)))

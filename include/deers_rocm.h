@@ -241,6 +241,12 @@ int deers_rocm_rms_norm_bwd(int dtype, const void* x, const void* dy, void* dx, 
  * its backward dx = dy * 2 * relu(x). */
 int deers_rocm_relu_sq_fwd(int dtype, const void* x, void* y, int64_t n);
 int deers_rocm_relu_sq_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t n);
+/* out[i] (int64, device) = index of the largest element of row i of compact
+ * [outer, inner] data, the lowest index on ties: the greedy (temperature 0) case of
+ * the reference's sampling, which it does on the host after to_vec
+ * (examples/tinystories_train.rs:262-272).  Keeping the pick on the device lets the next
+ * token's embedding lookup read it without a host round trip. */
+int deers_rocm_argmax_rows(int dtype, const void* x, int64_t* out, int64_t outer, int64_t inner);
 /* loss::cross_entropy (src/loss.rs:11-24): *loss (a float in device memory) =
  * -mean_i log_softmax(logits)[i, targets[i]] over compact [n_rows, n_classes] logits,
  * without writing the log-probabilities; row_lse [n_rows] (f32, device) receives each

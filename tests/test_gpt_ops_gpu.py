@@ -203,3 +203,18 @@ def test_gpt_ops_argument_errors():
         rocm.cross_entropy_fwd_raw(np.float32, buf.ptr, idx.ptr, buf.ptr, buf.ptr, 0, 4)
     rocm.index_select_raw(np.float32, null, null, null, 4, 0, 4)  # empty: no-op
     rocm.sync()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("outer,inner", [(1, 1), (3, 7), (32, 300), (5, 50257)])
+def test_argmax_rows(dtype, outer, inner):
+    x = synth.normal((outer, inner), synth.tensor_seed(76, "argmax", "x"), 2.0).astype(dtype)
+    if inner > 4:
+        x[0, 3] = x[0].max()          # a tie: the lowest index wins
+        x[0, inner - 1] = x[0].max()
+        x[outer - 1, :] = -np.inf      # nothing to pick: index 0
+    bx = _dev(x)
+    out = _dev(np.full(outer, -1, np.int64))
+    rocm.argmax_rows_raw(dtype, bx.ptr, out.ptr, outer, inner)
+    assert np.array_equal(out.numpy(), np.argmax(x, axis=1))
