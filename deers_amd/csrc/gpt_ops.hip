@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void index_select_kernel(const T* table, const
 // idx[i] if no earlier position names it, finds every later position that does (a
 // bitmap in LDS, built from the index vector, which stays in L2), and adds their source
 // rows in order.  Other workgroups leave at once.
-constexpr int kIndexAddMaxIdx = 1 << 19;  // bitmap of 64 KB
+constexpr int kIndexAddMaxIdx = 1 << 18;  // bitmap of 32 KB of dynamic LDS
 
 template <typename T>
 __global__ __launch_bounds__(256) void index_add_kernel(const T* src, const int64_t* idx, T* dst,

@@ -227,7 +227,7 @@ int deers_rocm_index_select(int dtype, const void* table, const int64_t* indices
  * (src/storage.rs:272-280; CPU src/storage/cpu.rs:612-660, 954-975), the backward of
  * index_select (src/ops.rs:1429-1447).  dst [n_rows, width] is accumulated into (zero
  * it first for the reference's semantics); additions happen in the reference's order,
- * so the result is the same bits and reproducible.  At most 2^19 indices per call. */
+ * so the result is the same bits and reproducible.  At most 2^18 indices per call. */
 int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, void* dst,
                          int64_t n_rows, int64_t n_indices, int64_t width);
 /* y = x * (mean(x^2 over the last axis) + eps)^-0.5: RMSNorm::forward (src/nn.rs:244-251)

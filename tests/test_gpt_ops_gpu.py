@@ -81,7 +81,7 @@ def test_index_literals_of_the_reference_and_out_of_range():
         grad.numpy()
     assert (grad.numpy()[1] == 1).all()
     with pytest.raises(rocm.RocmError):
-        rocm.index_add_raw(np.float32, grad.ptr, bad.ptr, grad.ptr, 4, (1 << 19) + 1, 3)
+        rocm.index_add_raw(np.float32, grad.ptr, bad.ptr, grad.ptr, 4, (1 << 18) + 1, 3)
 
 
 @pytest.mark.gpu
@@ -218,3 +218,17 @@ def test_argmax_rows(dtype, outer, inner):
     out = _dev(np.full(outer, -1, np.int64))
     rocm.argmax_rows_raw(dtype, bx.ptr, out.ptr, outer, inner)
     assert np.array_equal(out.numpy(), np.argmax(x, axis=1))
+
+
+@pytest.mark.gpu
+def test_index_add_at_the_largest_index_count():
+    # 2^18 positions: the bitmap fills the dynamic LDS the kernel may ask for
+    n, vocab, width = 1 << 18, 997, 4
+    idx = _tokens(n, vocab, 77, repeats=False)
+    g = synth.normal((n, width), synth.tensor_seed(77, "emb", "g"), 1.0).astype(np.float32)
+    dg, di = _dev(g), _dev(idx)
+    dst = rocm.DeviceBuffer((vocab, width), np.float32, zeros=True)
+    rocm.index_add_raw(np.float32, dg.ptr, di.ptr, dst.ptr, vocab, n, width)
+    want = np.zeros((vocab, width), np.float32)
+    np.add.at(want, idx, g)  # unbuffered, in position order: the same sequence of f32 additions
+    assert np.array_equal(dst.numpy(), want)
