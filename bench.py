@@ -305,6 +305,33 @@ def bench_gpt(steps: int, warmup: int):
     return out
 
 
+def cpu_baseline_gpt():
+    """The composed CPU oracle (numpy GEMMs on all host threads + the C attention oracle) on
+    a bounded sample of the GPT step: one of the 8 sequences (batch 1, T = 1024) through the
+    full 12-layer model, forward + loss + backward + AdamW, timed once after no warm-up.
+    kind "port": the Rust reference cannot be built here."""
+    import oracle  # the checker; only ever the thing measured in this baseline leg
+    from oracle import gpt as ogpt
+    cfg = dict(vocab_size=50257, sequence_len=1024, n_layer=12, n_head=12, n_embd=768,
+               mlp_hidden_dim=3072, rms_norm_eps=1e-5, rope_base=10000.0)
+    rng = np.random.default_rng(0)
+    C, Hd, V = cfg["n_embd"], cfg["mlp_hidden_dim"], cfg["vocab_size"]
+    uni = lambda r, c: rng.uniform(-1 / np.sqrt(r), 1 / np.sqrt(r), (r, c)).astype(np.float32)
+    w = [rng.standard_normal((V, C)).astype(np.float32)]
+    for _ in range(cfg["n_layer"]):
+        w += [uni(C, C), uni(C, C), uni(C, C), uni(C, C), uni(C, Hd), uni(Hd, C)]
+    w.append(uni(C, V))
+    ids = rng.integers(0, V, (1, 1024))
+    targets = rng.integers(0, V, 1024)
+    mom = [(np.zeros_like(a), np.zeros_like(a)) for a in w]
+    t0 = time.perf_counter()
+    ogpt.train_step(cfg, w, mom, 1, ids, targets, 3e-4, (0.9, 0.95), 1e-8, 0.1, max_norm=1.0)
+    sec = time.perf_counter() - t0
+    return {"value": 1024 / sec, "unit": "tokens/s", "cores": oracle.max_threads(), "kind": "port",
+            "seconds_per_step": sec,
+            "sample": "1 of the 8 sequences (batch 1, T=1024), whole 12-layer model, one training step"}
+
+
 def cpu_baseline():
     """The CPU oracle (kind "port": a restatement of the reference's materialised CPU
     attention; the Rust reference itself cannot be built here) on the full B=8 H=12
@@ -430,6 +457,11 @@ def main():
             out["gpt_train_step"] = {"error": str(e)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        if "gpt_train_step" in out and "error" not in out["gpt_train_step"]:
+            try:
+                out["gpt_train_step"]["cpu_baseline"] = cpu_baseline_gpt()
+            except Exception as e:
+                out["gpt_train_step"]["cpu_baseline"] = {"error": str(e)}
     print(json.dumps(out))
 
 
