@@ -51,7 +51,9 @@ constexpr float kLazyRescale = 8.0f;
 
 template <int D>
 struct FwdCfg {
-  static constexpr int P = 2;                   // prefetch distance in iterations
+  // prefetch distance in iterations; D = 128 keeps one tile less in flight so that two
+  // workgroups' rings (2 x 64 KB) share a CU
+  static constexpr int P = D == 128 ? 1 : 2;
   static constexpr int NS = P + 1;              // ring slots per tensor
   static constexpr int RB = D * 2;              // row bytes
   static constexpr int TILE_B = kFwdBN * RB;    // tile bytes
@@ -59,7 +61,7 @@ struct FwdCfg {
 };
 
 template <int D>
-__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(FwdParams p, int BH, int n_qtiles,
+__global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int BH, int n_qtiles,
                                                               int heads_per_xcd) {
   using Cfg = FwdCfg<D>;
   constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
@@ -238,9 +240,38 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
     request(j + 1 + P, j - 1 + P);
-    half8 kfr[HAS_S ? 2 * KS : 1], vfr[HAS_PV ? 4 * DB : 1];
-    if constexpr (HAS_PV) load_v(j - 1, vfr);
-    if constexpr (HAS_S) load_k(j + 1, kfr);
+    // D <= 64: every fragment of the iteration is fetched here, ahead of the vector work.
+    // D = 128: that would be 128 registers of operands; instead a window of kJit
+    // fragments runs ahead of the MFMAs that consume them (see the chunk loop).
+    constexpr bool JIT = D == 128;
+    constexpr int kJit = 4;
+    constexpr int NMS_ = HAS_S ? 2 * KS : 0;
+    constexpr int NM_ = NMS_ + (HAS_PV ? 4 * DB : 0);
+    half8 kfr[(HAS_S && !JIT) ? 2 * KS : 1], vfr[(HAS_PV && !JIT) ? 4 * DB : 1];
+    half8 fr[JIT ? kJit : 1];
+    // fragment of MFMA number mi of this iteration (S(j+1) first, then PV(j-1)); the
+    // address is formed at the fetch (an add or two) rather than kept for the iteration
+    const uint32_t kb_jit = lds0 + ((j + 1) % NS) * TILE_B;
+    const uint32_t vb_jit = lds0 + (NS + (j + NS - 1) % NS) * TILE_B;
+    auto fetch = [&](int mi) -> half8 {
+      if (mi < NMS_) {
+        const int ks = mi >> 1;
+        const uint32_t addr = opaque(kb_jit + koff[ks]);
+        return *(DEERS_LDS const half8*)(uintptr_t)(addr + (mi & 1) * 32 * RB);
+      }
+      const int ms = (mi - NMS_) / DB, db = (mi - NMS_) % DB;
+      const uint32_t ro = 16 * ms * RB;
+      const half4 lo = lds_read_tr16_at(opaque(vb_jit + voff_lo[db]) + ro);
+      const half4 hi = lds_read_tr16_at(opaque(vb_jit + voff_hi[db]) + ro);
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    if constexpr (JIT) {
+#pragma unroll
+      for (int mi = 0; mi < kJit && mi < NM_; ++mi) fr[mi] = fetch(mi);
+    } else {
+      if constexpr (HAS_PV) load_v(j - 1, vfr);
+      if constexpr (HAS_S) load_k(j + 1, kfr);
+    }
     __builtin_amdgcn_sched_barrier(0);  // keep the fetches ahead of the vector work below
 
     if (kv0 + kFwdBN - 1 > qw0) {  // tile reaches past this wave's first row: element mask
@@ -308,13 +339,18 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_fwd_f16_kernel(F
       for (int mi = i * NM / 16; mi < (i + 1) * NM / 16; ++mi) {
         if (mi < NMS) {
           const int ks = mi >> 1;
+          const half8 a = JIT ? fr[mi % kJit] : kfr[JIT ? 0 : mi];
           if (mi & 1)
-            n1 = mfma_f16(kfr[2 * ks + 1], qf[ks], n1);
+            n1 = mfma_f16(a, qf[ks], n1);
           else
-            n0 = mfma_f16(kfr[2 * ks], qf[ks], n0);
+            n0 = mfma_f16(a, qf[ks], n0);
         } else {
           const int ms = (mi - NMS) / DB, db = (mi - NMS) % DB;
-          oacc[db] = mfma_f16(vfr[ms * DB + db], pf[ms], oacc[db]);
+          const half8 a = JIT ? fr[mi % kJit] : vfr[JIT ? 0 : ms * DB + db];
+          oacc[db] = mfma_f16(a, pf[ms], oacc[db]);
+        }
+        if constexpr (JIT) {
+          if (mi + kJit < NM) fr[mi % kJit] = fetch(mi + kJit);
         }
       }
       floatx16& cc = (i < 8) ? c0 : c1;
