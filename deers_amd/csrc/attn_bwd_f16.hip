@@ -285,18 +285,10 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     half_t* dkrow = dK + (int64_t)kvrow * p.sdk.t;
     half_t* dvrow = dV + (int64_t)kvrow * p.sdv.t;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        half4 ok, ov;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          ok[e] = (half_t)(dkacc[db][4 * rq + e] * p.scale);
-          ov[e] = (half_t)(dvacc[db][4 * rq + e]);
-        }
-        *(half4*)(dkrow + 32 * db + 8 * rq + 4 * g) = ok;
-        *(half4*)(dvrow + 32 * db + 8 * rq + 4 * g) = ov;
-      }
+    for (int db = 0; db < DB; ++db) {
+      store_block_f16(dkrow + 32 * db, dkacc[db], p.scale, g);
+      store_block_f16(dvrow + 32 * db, dvacc[db], 1.f, g);
+    }
   }
   DEERS_TRACE_POINT(30);
 }
@@ -499,14 +491,7 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
   if (qrow < T) {
     half_t* dqrow = dQ + (int64_t)qrow * p.sdq.t;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        half4 out;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = (half_t)(dqacc[db][4 * rq + e] * p.scale);
-        *(half4*)(dqrow + 32 * db + 8 * rq + 4 * g) = out;
-      }
+    for (int db = 0; db < DB; ++db) store_block_f16(dqrow + 32 * db, dqacc[db], p.scale, g);
   }
   DEERS_TRACE_POINT(30);
 }

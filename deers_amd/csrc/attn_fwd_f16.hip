@@ -426,14 +426,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
     const float inv = 1.f / lsum;
     half_t* orow = O + (int64_t)qrow * p.so.t;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        half4 out;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = (half_t)(oacc[db][4 * rq + e] * inv);
-        *(half4*)(orow + 32 * db + 8 * rq + 4 * g) = out;
-      }
+    for (int db = 0; db < DB; ++db) store_block_f16(orow + 32 * db, oacc[db], inv, g);
     if (g == 0) p.lse[(int64_t)bh * T + qrow] = (m * c + fast_log2(lsum)) * kLn2;
   }
   DEERS_TRACE_POINT(30);

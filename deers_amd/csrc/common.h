@@ -52,6 +52,29 @@ __device__ __forceinline__ float pair_sum(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// Writes one 32-column block of an output row from a 32x32 accumulator (the lane owns
+// the row; element 4*rq + e is column 8*rq + 4*g + e, g = lane / 32).  A lane holds 4
+// consecutive columns of each 8-column group and its partner (lane ^ 32) the other 4:
+// the pair trades halves of two groups, so each lane writes 16 contiguous bytes (two
+// 16-byte stores per block instead of four 8-byte ones).  `dst` points at the block's
+// first column in this lane's row and must be 16-byte aligned.
+__device__ __forceinline__ void store_block_f16(half_t* dst, const floatx16& acc, float mul, int g) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int rp = 0; rp < 2; ++rp) {
+    half4 x, y;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x[e] = (half_t)(acc[8 * rp + e] * mul);
+      y[e] = (half_t)(acc[8 * rp + 4 + e] * mul);
+    }
+    const u32x2 xu = __builtin_bit_cast(u32x2, x), yu = __builtin_bit_cast(u32x2, y);
+    const auto r0 = __builtin_amdgcn_permlane32_swap(xu[0], yu[0], false, false);
+    const auto r1 = __builtin_amdgcn_permlane32_swap(xu[1], yu[1], false, false);
+    *(u32x4*)(dst + 16 * rp + 8 * g) = u32x4{r0[0], r1[0], r0[1], r1[1]};
+  }
+}
 // Kept for the f32 kernels: exchange with the lane 32 away.
 __device__ __forceinline__ float swap32(float x) { return __shfl_xor(x, 32, 64); }
 
