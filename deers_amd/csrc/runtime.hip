@@ -19,6 +19,7 @@
 #include <vector>
 
 #include "common.h"
+#include "storage_ops.h"
 
 namespace deers {
 void launch_attn_fwd_f16(const FwdParams& p, int B, int D, hipStream_t stream);
@@ -883,6 +884,175 @@ int deers_rocm_cross_entropy_bwd(int dtype, const void* logits, const int64_t* t
     return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_bwd: null pointer");
   deers::launch_cross_entropy_bwd(dtype == DEERS_ROCM_F16, logits, targets, row_lse, upstream, dlogits,
                                   n_rows, (int)n_classes, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+// ---- the generic BackendStorage kernels ----
+static_assert(deers::kUnaryNeg == DEERS_ROCM_UNARY_NEG && deers::kUnaryPowf == DEERS_ROCM_UNARY_POWF &&
+                  deers::kUnaryScalarAdd == DEERS_ROCM_UNARY_SCALAR_ADD &&
+                  deers::kBinaryAdd == DEERS_ROCM_BINARY_ADD && deers::kBinaryEq == DEERS_ROCM_BINARY_EQ,
+              "op codes of the header and of storage_ops.h must agree");
+
+// Collapses (shape, strides) into a StridedView: dimensions of extent 1 dropped, a
+// dimension merged into its inner neighbour where the two are contiguous with each
+// other.  Returns false if the view is compact (no StridedView needed).
+static bool make_view(int ndim, const int64_t* shape, const int64_t* strides, deers::StridedView* v) {
+  v->ndim = 0;
+  if (!strides) return false;
+  int64_t s[deers::kMaxViewDims], t[deers::kMaxViewDims];
+  int n = 0;
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] == 1) continue;
+    if (n > 0 && t[n - 1] == strides[d] * shape[d]) {  // outer stride spans the inner dimension
+      s[n - 1] *= shape[d];
+      t[n - 1] = strides[d];
+    } else {
+      s[n] = shape[d];
+      t[n] = strides[d];
+      ++n;
+    }
+  }
+  if (n == 0 || (n == 1 && t[0] == 1)) return false;
+  v->ndim = n;
+  for (int d = 0; d < n; ++d) {
+    v->shape[d] = (uint32_t)s[d];
+    v->stride[d] = t[d];
+  }
+  return true;
+}
+
+// element count of `shape`, or -1 if a dimension is negative or the view is too large
+static int64_t view_elements(const char* what, int ndim, const int64_t* shape) {
+  if (ndim < 1 || ndim > deers::kMaxViewDims) {
+    fail(DEERS_ROCM_ERR_ARG, "%s: ndim %d not in 1..%d", what, ndim, deers::kMaxViewDims);
+    return -1;
+  }
+  if (!shape) {
+    fail(DEERS_ROCM_ERR_ARG, "%s: null shape", what);
+    return -1;
+  }
+  int64_t n = 1;
+  for (int d = 0; d < ndim; ++d) {
+    if (shape[d] < 0) {
+      fail(DEERS_ROCM_ERR_LAYOUT, "%s: negative extent in dim %d", what, d);
+      return -1;
+    }
+    if (shape[d] > 0 && n > INT64_MAX / shape[d]) {
+      fail(DEERS_ROCM_ERR_ARG, "%s: element count overflows", what);
+      return -1;
+    }
+    n *= shape[d];
+  }
+  return n;
+}
+
+int deers_rocm_unary(int dtype, int op, const void* x, int ndim, const int64_t* shape,
+                     const int64_t* strides, double param, void* out) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (op < 0 || op >= deers::kUnaryCount) return fail(DEERS_ROCM_ERR_ARG, "unary: unknown op %d", op);
+  const int64_t n = view_elements("unary", ndim, shape);
+  if (n < 0) return DEERS_ROCM_ERR_ARG;
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!x || !out) return fail(DEERS_ROCM_ERR_ARG, "unary: null pointer");
+  deers::StridedView view;
+  const bool strided = make_view(ndim, shape, strides, &view);
+  if ((strided || ((uintptr_t)x & 15) || ((uintptr_t)out & 15)) && n > (int64_t)UINT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "unary: a strided or unaligned operand is limited to 2^32 - 1 elements");
+  deers::launch_unary(dtype == DEERS_ROCM_F16, op, x, strided ? &view : nullptr, out, n, param, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_binary(int dtype, int op, const void* a, const int64_t* a_strides, const void* b,
+                      const int64_t* b_strides, int ndim, const int64_t* shape, void* out) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (op < 0 || op >= deers::kBinaryCount) return fail(DEERS_ROCM_ERR_ARG, "binary: unknown op %d", op);
+  const int64_t n = view_elements("binary", ndim, shape);
+  if (n < 0) return DEERS_ROCM_ERR_ARG;
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!a || !b || !out) return fail(DEERS_ROCM_ERR_ARG, "binary: null pointer");
+  deers::StridedView va, vb;
+  const bool sa = make_view(ndim, shape, a_strides, &va), sb = make_view(ndim, shape, b_strides, &vb);
+  const bool vector_path = !sa && !sb && !((uintptr_t)a & 15) && !((uintptr_t)b & 15) && !((uintptr_t)out & 15);
+  if (!vector_path && n > (int64_t)UINT32_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "binary: strided or unaligned operands are limited to 2^32 - 1 elements");
+  deers::launch_binary(dtype == DEERS_ROCM_F16, op, a, sa ? &va : nullptr, b, sb ? &vb : nullptr, out, n,
+                       g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_reduce(int dtype, int op, const void* x, void* out, int64_t outer, int64_t reduce_size) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("reduce", dtype, outer, reduce_size)) return rc;
+  if (op != DEERS_ROCM_REDUCE_SUM && op != DEERS_ROCM_REDUCE_MAX)
+    return fail(DEERS_ROCM_ERR_ARG, "reduce: unknown op %d", op);
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !out) return fail(DEERS_ROCM_ERR_ARG, "reduce: null pointer");
+  deers::launch_reduce(dtype == DEERS_ROCM_F16, op == DEERS_ROCM_REDUCE_MAX, x, out, outer, reduce_size,
+                       g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_log_sum_exp(int dtype, const void* x, void* out, int64_t outer, int64_t reduce_size) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("log_sum_exp", dtype, outer, reduce_size)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !out) return fail(DEERS_ROCM_ERR_ARG, "log_sum_exp: null pointer");
+  deers::launch_log_sum_exp(dtype == DEERS_ROCM_F16, x, out, outer, reduce_size, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+static int dim_check(const char* what, int64_t left, int64_t dim, int64_t index_len, int64_t right) {
+  if (left < 0 || dim < 0 || index_len < 0 || right < 0)
+    return fail(DEERS_ROCM_ERR_ARG, "%s: negative extent", what);
+  const int64_t lim = (int64_t)1 << 40;
+  if (left > lim || dim > lim || index_len > lim || right > lim ||
+      (double)left * (double)right * (double)(dim > index_len ? dim : index_len) > 9.0e18)
+    return fail(DEERS_ROCM_ERR_ARG, "%s: element count overflows", what);
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_gather(int dtype, const void* src, const int64_t* indices, void* out, int64_t left,
+                      int64_t src_dim, int64_t index_len, int64_t right) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (dtype != DEERS_ROCM_F16 && dtype != DEERS_ROCM_F32 && dtype != DEERS_ROCM_I64)
+    return fail(DEERS_ROCM_ERR_ARG, "gather: unknown dtype %d", dtype);
+  if (int rc = dim_check("gather", left, src_dim, index_len, right)) return rc;
+  if (left * index_len * right == 0) return DEERS_ROCM_OK;
+  if (!src || !indices || !out) return fail(DEERS_ROCM_ERR_ARG, "gather: null pointer");
+  int* flag = nullptr;
+  if (int rc = index_flag(&flag)) return rc;
+  const int bytes = dtype == DEERS_ROCM_F16 ? 2 : dtype == DEERS_ROCM_F32 ? 4 : 8;
+  deers::launch_gather(bytes, src, indices, out, left, src_dim, index_len, right, flag, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_scatter_add(int dtype, const void* src, const int64_t* indices, void* dst, int64_t left,
+                           int64_t dst_dim, int64_t index_len, int64_t right) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (int rc = dim_check("scatter_add", left, dst_dim, index_len, right)) return rc;
+  if (left * index_len * right == 0) return DEERS_ROCM_OK;
+  if (!src || !indices || !dst) return fail(DEERS_ROCM_ERR_ARG, "scatter_add: null pointer");
+  if (left * right > (int64_t)INT32_MAX * 256)
+    return fail(DEERS_ROCM_ERR_ARG, "scatter_add: too many columns for one call");
+  int* flag = nullptr;
+  if (int rc = index_flag(&flag)) return rc;
+  deers::launch_scatter_add(dtype == DEERS_ROCM_F16, src, indices, dst, left, dst_dim, index_len, right,
+                            flag, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -272,6 +272,56 @@ def cross_entropy_bwd_raw(dtype, logits, targets, row_lse, upstream, dlogits, n_
                                                ctypes.c_int64(n_classes)))
 
 
+# op codes of deers_rocm_unary / deers_rocm_binary / deers_rocm_reduce (include/deers_rocm.h)
+UNARY_OPS = {"neg": 0, "exp": 1, "log": 2, "sin": 3, "cos": 4, "tanh": 5, "relu": 6,
+             "relu_backward": 7, "scalar_add": 8, "scalar_mul": 9, "scalar_div": 10, "powf": 11}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "eq": 5}
+REDUCE_OPS = {"sum": 0, "max": 1}
+I64 = 2
+
+
+def _i64_array(values):
+    if values is None:
+        return None
+    return (ctypes.c_int64 * len(values))(*[int(x) for x in values])
+
+
+def unary_raw(dtype, op, x, shape, strides, param, out):
+    """out (compact over `shape`) = op(x read through element `strides`; None = compact)."""
+    _check(load().deers_rocm_unary(ctypes.c_int(dtype_code(dtype)), ctypes.c_int(UNARY_OPS[op]), x,
+                                   ctypes.c_int(len(shape)), _i64_array(shape), _i64_array(strides),
+                                   ctypes.c_double(param), out))
+
+
+def binary_raw(dtype, op, a, a_strides, b, b_strides, shape, out):
+    _check(load().deers_rocm_binary(ctypes.c_int(dtype_code(dtype)), ctypes.c_int(BINARY_OPS[op]), a,
+                                    _i64_array(a_strides), b, _i64_array(b_strides),
+                                    ctypes.c_int(len(shape)), _i64_array(shape), out))
+
+
+def reduce_raw(dtype, op, x, out, outer, reduce_size):
+    _check(load().deers_rocm_reduce(ctypes.c_int(dtype_code(dtype)), ctypes.c_int(REDUCE_OPS[op]), x, out,
+                                    ctypes.c_int64(outer), ctypes.c_int64(reduce_size)))
+
+
+def log_sum_exp_raw(dtype, x, out, outer, reduce_size):
+    _check(load().deers_rocm_log_sum_exp(ctypes.c_int(dtype_code(dtype)), x, out, ctypes.c_int64(outer),
+                                         ctypes.c_int64(reduce_size)))
+
+
+def gather_raw(dtype, src, indices, out, left, src_dim, index_len, right):
+    code = I64 if np.dtype(dtype) == np.int64 else dtype_code(dtype)
+    _check(load().deers_rocm_gather(ctypes.c_int(code), src, indices, out, ctypes.c_int64(left),
+                                    ctypes.c_int64(src_dim), ctypes.c_int64(index_len),
+                                    ctypes.c_int64(right)))
+
+
+def scatter_add_raw(dtype, src, indices, dst, left, dst_dim, index_len, right):
+    _check(load().deers_rocm_scatter_add(ctypes.c_int(dtype_code(dtype)), src, indices, dst,
+                                         ctypes.c_int64(left), ctypes.c_int64(dst_dim),
+                                         ctypes.c_int64(index_len), ctypes.c_int64(right)))
+
+
 def adamw_step_raw(dtype, w, grad, m, v, n, lr, beta1, beta2, eps, weight_decay, step,
                    grad_scale=1.0):
     _check(load().deers_rocm_adamw_step(

@@ -42,6 +42,7 @@ extern "C" {
 
 #define DEERS_ROCM_F16 0
 #define DEERS_ROCM_F32 1
+#define DEERS_ROCM_I64 2 /* DType::I64 data: accepted by deers_rocm_gather only */
 
 #define DEERS_ROCM_OK 0
 #define DEERS_ROCM_ERR_HIP 1         /* a HIP runtime call failed */
@@ -230,6 +231,85 @@ int deers_rocm_index_select(int dtype, const void* table, const int64_t* indices
  * so the result is the same bits and reproducible.  At most 2^18 indices per call. */
 int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, void* dst,
                          int64_t n_rows, int64_t n_indices, int64_t width);
+/* index_select / index_add along a dimension other than the first
+ * (src/storage/cpu.rs:936-975 with left_len > 1): the `left` slabs of a compact
+ * [left, dim, right] tensor are contiguous, so the caller issues one call per slab with
+ * width = right.  CpuStorage::cat (src/storage/cpu.rs:47-90) concatenates compact
+ * buffers: one deers_rocm_dtod per part. */
+
+/* ---- the generic kernels of BackendStorage (src/storage.rs:227-306) ------------------
+ * What the reference's op graph calls where no fused op applies.  Outputs are compact
+ * (src/storage.rs:224-226).  Arithmetic is f32 with one rounding to the storage type,
+ * as the reference's f16 kernels do (convert, operate, convert back). */
+
+/* `op` of deers_rocm_unary: the UnaryOp kernels of src/storage.rs:32-123 and
+ * ewise_powf (src/storage.rs:228).  `param` is the scalar of the SCALAR_* ops (cast
+ * f64 -> f32 -> storage type, src/storage.rs:105-123) or the exponent of POWF (cast
+ * f64 -> f32 only, src/storage/cpu.rs:203-235); ignored otherwise. */
+#define DEERS_ROCM_UNARY_NEG 0
+#define DEERS_ROCM_UNARY_EXP 1
+#define DEERS_ROCM_UNARY_LOG 2
+#define DEERS_ROCM_UNARY_SIN 3
+#define DEERS_ROCM_UNARY_COS 4
+#define DEERS_ROCM_UNARY_TANH 5
+#define DEERS_ROCM_UNARY_RELU 6          /* max(x, 0); NaN -> 0 as f32::max */
+#define DEERS_ROCM_UNARY_RELU_BACKWARD 7 /* x > 0 ? 1 : 0 */
+#define DEERS_ROCM_UNARY_SCALAR_ADD 8
+#define DEERS_ROCM_UNARY_SCALAR_MUL 9
+#define DEERS_ROCM_UNARY_SCALAR_DIV 10
+#define DEERS_ROCM_UNARY_POWF 11
+/* out (compact, row-major over `shape`) = op(x read through element `strides`).
+ * BackendStorage::unary_op / ewise_powf; CPU src/storage/cpu.rs:203-265, 1021-1061.
+ * ndim in 1..8; strides NULL = compact, otherwise any sign, 0 = broadcast.  A strided
+ * or not 16-byte aligned operand is limited to 2^32 - 1 elements. */
+int deers_rocm_unary(int dtype, int op, const void* x, int ndim, const int64_t* shape,
+                     const int64_t* strides, double param, void* out);
+
+/* `op` of deers_rocm_binary: the BinaryOp kernels of src/storage.rs:126-190. */
+#define DEERS_ROCM_BINARY_ADD 0
+#define DEERS_ROCM_BINARY_SUB 1
+#define DEERS_ROCM_BINARY_MUL 2
+#define DEERS_ROCM_BINARY_DIV 3
+#define DEERS_ROCM_BINARY_POW 4 /* powf(a, b) */
+#define DEERS_ROCM_BINARY_EQ 5  /* a == b ? 1 : 0 */
+/* out (compact) = op(a, b), both operands of `shape` read through their own strides
+ * (NULL = compact; the Broadcast op hands over stride-0 views, src/ops.rs:730-804).
+ * BackendStorage::binary_op; CPU src/storage/cpu.rs:267-321, 982-1019. */
+int deers_rocm_binary(int dtype, int op, const void* a, const int64_t* a_strides, const void* b,
+                      const int64_t* b_strides, int ndim, const int64_t* shape, void* out);
+
+#define DEERS_ROCM_REDUCE_SUM 0
+#define DEERS_ROCM_REDUCE_MAX 1 /* NaNs ignored unless the whole run is NaN, as f32::max */
+/* out[i] = sum / max of x[i*reduce_size .. (i+1)*reduce_size), x compact.
+ * BackendStorage::reduce (src/storage.rs:238; CPU src/storage/cpu.rs:323-357).  Runs of
+ * up to 32 elements are reduced left to right in the storage type (the reference's
+ * order and rounding); longer runs are summed in f32 in a fixed tree order, so a sum
+ * differs from the reference's by reassociation (f32) and is more accurate than its
+ * f16 accumulator (f16). */
+int deers_rocm_reduce(int dtype, int op, const void* x, void* out, int64_t outer,
+                      int64_t reduce_size);
+/* out[i] = ln sum_j exp(x[i, j]) over compact rows: the maximum, then
+ * ln(sum exp(x - max)) + max, special values as in the reference.
+ * BackendStorage::log_sum_exp (src/storage.rs:282-283; CPU src/storage/cpu.rs:755-791). */
+int deers_rocm_log_sum_exp(int dtype, const void* x, void* out, int64_t outer,
+                           int64_t reduce_size);
+
+/* out[l, i, r] = src[l, indices[l, i, r], r]; src compact [left, src_dim, right],
+ * indices and out compact [left, index_len, right].  BackendStorage::gather
+ * (src/storage.rs:243-249; CPU src/storage/cpu.rs:398-462, 891-912); F16, F32 or I64
+ * data.  Out-of-range indices are skipped and reported as DEERS_ROCM_ERR_INDEX by the
+ * next deers_rocm_sync / deers_rocm_dtoh. */
+int deers_rocm_gather(int dtype, const void* src, const int64_t* indices, void* out, int64_t left,
+                      int64_t src_dim, int64_t index_len, int64_t right);
+/* dst[l, indices[l, i, r], r] += src[l, i, r] for i ascending; src and indices compact
+ * [left, index_len, right], dst compact [left, dst_dim, right], accumulated into (zero
+ * it first for the reference's semantics).  BackendStorage::scatter_add
+ * (src/storage.rs:252-260; CPU src/storage/cpu.rs:464-553, 914-934).  One thread owns an
+ * output column (l, :, r) and applies its additions in the reference's order with its
+ * rounding (the storage type after every addition): same bits, no atomics. */
+int deers_rocm_scatter_add(int dtype, const void* src, const int64_t* indices, void* dst,
+                           int64_t left, int64_t dst_dim, int64_t index_len, int64_t right);
+
 /* y = x * (mean(x^2 over the last axis) + eps)^-0.5: RMSNorm::forward (src/nn.rs:244-251)
  * in one pass over compact [outer, inner]; and its backward
  * dx = inv * dy - x * inv^3 * sum(dy * x) / inner from x and dy. */

@@ -1,0 +1,340 @@
+"""The generic storage kernels (deers_rocm_unary / _binary / _reduce / _log_sum_exp / _gather /
+_scatter_add) against oracle/storage_ops.py, the numpy restatement of src/storage/cpu.rs.
+
+Bar: bit-exact for everything that is exact arithmetic, a copy or an index operation (neg, relu,
+relu_backward, the scalar ops, add/sub/mul/div/eq, max, short sums, gather, scatter_add); for the
+transcendental kernels and long sums the f32 results agree to a few ulp (the device's math
+library and numpy's are different implementations; the reference's libm is a third), which is
+far inside the 1e-4 the f32 path is held to, and f16 results are at most one f16 ulp apart."""
+import numpy as np
+import pytest
+
+from deers_amd import rocm
+from oracle import storage_ops as so
+
+EXACT_UNARY = ("neg", "relu", "relu_backward", "scalar_add", "scalar_mul", "scalar_div")
+EXACT_BINARY = ("add", "sub", "mul", "div", "eq")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    if not rocm.available():
+        pytest.skip("no gfx950 device")
+    rocm.init(0)
+
+
+def _dev(a):
+    return rocm.DeviceBuffer.from_numpy(a)
+
+
+def _rand(shape, seed, dtype, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(dtype)
+
+
+def _ulps16(a, b):
+    ia, ib = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+    ia, ib = np.where(ia < 0, -32768 - ia, ia), np.where(ib < 0, -32768 - ib, ib)
+    return np.abs(ia - ib)
+
+
+def _same(got, want, exact):
+    assert got.shape == want.shape and got.dtype == want.dtype
+    nan_g, nan_w = np.isnan(got), np.isnan(want)
+    assert np.array_equal(nan_g, nan_w)
+    g, w = np.where(nan_g, 0, got), np.where(nan_w, 0, want)
+    if exact:
+        assert np.array_equal(g, w)
+        assert np.array_equal(np.signbit(g), np.signbit(w))
+    elif got.dtype == np.float16:
+        fin = np.isfinite(w)
+        assert np.array_equal(g[~fin], w[~fin])
+        assert _ulps16(g[fin], w[fin]).max(initial=0) <= 1
+    else:
+        fin = np.isfinite(w)
+        assert np.array_equal(g[~fin], w[~fin])
+        np.testing.assert_allclose(g[fin], w[fin], rtol=4e-6, atol=1e-7)
+
+
+def _views(base_shape, seed, dtype, scale):
+    """(name, host array viewed, backing array, element offset, element strides or None)."""
+    out = []
+    a = _rand(base_shape, seed, dtype, scale)
+    out.append(("compact", a, a, 0, None))
+    t = a.transpose(*reversed(range(a.ndim)))
+    out.append(("transposed", t, a, 0, [s // a.itemsize for s in t.strides]))
+    row = _rand(base_shape[-1:], seed + 1, dtype, scale)
+    b = np.broadcast_to(row, base_shape)
+    out.append(("broadcast", b, row, 0, [s // row.itemsize for s in b.strides]))
+    flat = _rand(int(np.prod(base_shape)) + 3, seed + 2, dtype, scale)
+    u = flat[3:].reshape(base_shape)  # starts off a 16-byte boundary
+    out.append(("offset", u, flat, 3, None))
+    if len(base_shape) >= 2:
+        sl = a[:, ::2]
+        out.append(("sliced", sl, a, 0, [s // a.itemsize for s in sl.strides]))
+    return out
+
+
+def _ptr(buf, elem_offset, itemsize):
+    import ctypes
+    return ctypes.c_void_p(buf.ptr.value + elem_offset * itemsize)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("op", so.UNARY)
+def test_unary_over_layouts(op, dtype):
+    param = {"scalar_add": 0.1, "scalar_mul": 1.0 / 3.0, "scalar_div": 7.3, "powf": 2.5}.get(op, 0.0)
+    for name, view, backing, off, strides in _views((6, 5, 24), 100, dtype, 2.0):
+        host = np.ascontiguousarray(view)
+        if op in ("log", "powf"):
+            backing = (np.abs(backing) + dtype(0.05)).astype(dtype)
+            host = (np.abs(host) + dtype(0.05)).astype(dtype)
+        d_in = _dev(backing)
+        d_out = rocm.DeviceBuffer(host.shape, dtype)
+        rocm.unary_raw(dtype, op, _ptr(d_in, off, backing.itemsize), host.shape, strides, param, d_out.ptr)
+        _same(d_out.numpy(), so.unary(op, host, param), op in EXACT_UNARY)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_unary_special_values_and_large(dtype):
+    x = np.array([np.nan, -np.inf, np.inf, -0.0, 0.0, 1.0, -1.0, 65504.0, 6e-8], dtype)
+    for op in so.UNARY:
+        d_in, d_out = _dev(x), rocm.DeviceBuffer(x.shape, dtype)
+        rocm.unary_raw(dtype, op, d_in.ptr, x.shape, None, 0.5, d_out.ptr)
+        _same(d_out.numpy(), so.unary(op, x, 0.5), op in EXACT_UNARY)
+    big = _rand((1 << 22) + 5, 7, dtype, 3.0)  # vector path with a scalar tail
+    d_in, d_out = _dev(big), rocm.DeviceBuffer(big.shape, dtype)
+    rocm.unary_raw(dtype, "scalar_mul", d_in.ptr, big.shape, None, 0.37, d_out.ptr)
+    _same(d_out.numpy(), so.unary("scalar_mul", big, 0.37), True)
+    rocm.unary_raw(dtype, "exp", d_in.ptr, big.shape, None, 0.0, d_out.ptr)
+    _same(d_out.numpy(), so.unary("exp", big), False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("op", so.BINARY)
+def test_binary_over_layouts(op, dtype):
+    shape = (4, 7, 16)
+    views_a = _views(shape, 200, dtype, 2.0)
+    views_b = _views(shape, 300, dtype, 2.0)
+    for (na, va, ba, oa, sa) in views_a:
+        for (nb, vb, bb, ob, sb) in views_b:
+            if va.shape != vb.shape:
+                continue
+            ha, hb, back_a = np.ascontiguousarray(va), np.ascontiguousarray(vb), ba
+            if op == "pow":
+                back_a, ha = (np.abs(ba) + dtype(0.05)).astype(dtype), (np.abs(ha) + dtype(0.05)).astype(dtype)
+            if op == "eq":
+                continue  # covered below with operands that do collide
+            da, db = _dev(back_a), _dev(bb)
+            d_out = rocm.DeviceBuffer(ha.shape, dtype)
+            rocm.binary_raw(dtype, op, _ptr(da, oa, ba.itemsize), sa, _ptr(db, ob, bb.itemsize), sb,
+                            ha.shape, d_out.ptr)
+            _same(d_out.numpy(), so.binary(op, ha, hb), op in EXACT_BINARY)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_binary_eq_and_special_values(dtype):
+    a = np.array([1.0, 2.0, np.nan, np.inf, -0.0, 3.0, -np.inf, 5.0], dtype)
+    b = np.array([1.0, 2.5, np.nan, np.inf, 0.0, -3.0, 1.0, 0.0], dtype)
+    for op in so.BINARY:
+        da, db, d_out = _dev(a), _dev(b), rocm.DeviceBuffer(a.shape, dtype)
+        rocm.binary_raw(dtype, op, da.ptr, None, db.ptr, None, a.shape, d_out.ptr)
+        _same(d_out.numpy(), so.binary(op, a, b), op in EXACT_BINARY)
+    # the mask add of the attention path: [B,1,T,T] mask broadcast over heads (src/models/gpt.rs:141)
+    B, H, T = 2, 3, 33
+    scores = _rand((B, H, T, T), 9, dtype)
+    mask = np.where(np.triu(np.ones((T, T), bool), 1), -np.inf, 0).astype(dtype)
+    mask = np.ascontiguousarray(np.broadcast_to(mask, (B, 1, T, T)))
+    ds, dm, d_out = _dev(scores), _dev(mask), rocm.DeviceBuffer(scores.shape, dtype)
+    rocm.binary_raw(dtype, "add", ds.ptr, None, dm.ptr, [T * T, 0, T, 1], scores.shape, d_out.ptr)
+    _same(d_out.numpy(), so.binary("add", scores, np.broadcast_to(mask, scores.shape)), True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("outer,rs", [(2, 3), (1, 1), (1000, 7), (513, 32), (77, 33), (300, 257), (64, 4096),
+                                      (5, 50257), (3, 70001), (4096, 64)])
+def test_reduce(dtype, outer, rs):
+    x = _rand((outer, rs), outer * 31 + rs, dtype, 2.0)
+    if outer > 2:
+        x[1, rs // 2] = np.nan  # ignored by max, poisons that row's sum
+    d_in, d_out = _dev(x), rocm.DeviceBuffer((outer,), dtype)
+    rocm.reduce_raw(dtype, "max", d_in.ptr, d_out.ptr, outer, rs)
+    _same(d_out.numpy(), so.reduce("max", x), True)
+    rocm.reduce_raw(dtype, "sum", d_in.ptr, d_out.ptr, outer, rs)
+    got = d_out.numpy()
+    if rs <= 32:
+        _same(got, so.reduce("sum", x), True)  # the reference's order and rounding
+        return
+    exact = x.astype(np.float64).sum(axis=1)
+    mag = np.abs(x.astype(np.float64)).sum(axis=1)
+    ok = ~np.isnan(exact)
+    assert np.array_equal(np.isnan(got), ~ok)
+    if dtype == np.float32:  # reassociated f32 sum: error bounded by eps * sum |x|, as the reference's own
+        assert (np.abs(got[ok] - exact[ok]) <= 1e-6 * mag[ok] + 1e-30).all()
+        ref_err = np.abs(so.reduce("sum", x)[ok] - exact[ok])
+        assert (np.abs(got[ok] - exact[ok]) <= np.maximum(ref_err * 4, 1e-6 * mag[ok])).all()
+    else:  # f32 accumulation rounded once: within one f16 ulp of the exact sum
+        want = exact[ok].astype(np.float16)
+        fin = np.isfinite(want)
+        assert _ulps16(got[ok][fin], want[fin]).max(initial=0) <= 1
+
+
+@pytest.mark.gpu
+def test_reduce_max_all_nan_row():
+    x = np.full((3, 100), np.nan, np.float32)
+    x[1, 5] = 2.0
+    d_in, d_out = _dev(x), rocm.DeviceBuffer((3,), np.float32)
+    rocm.reduce_raw(np.float32, "max", d_in.ptr, d_out.ptr, 3, 100)
+    r = d_out.numpy()
+    assert np.isnan(r[0]) and r[1] == 2.0 and np.isnan(r[2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("outer,rs", [(2, 3), (1, 1), (1000, 7), (77, 33), (300, 257), (64, 4096), (5, 50257),
+                                      (3, 70001), (8192, 1024)])
+def test_log_sum_exp(dtype, outer, rs):
+    x = _rand((outer, rs), outer * 17 + rs, dtype, 3.0)
+    d_in, d_out = _dev(x), rocm.DeviceBuffer((outer,), dtype)
+    rocm.log_sum_exp_raw(dtype, d_in.ptr, d_out.ptr, outer, rs)
+    got, want = d_out.numpy(), so.log_sum_exp(x)
+    if dtype == np.float16:
+        assert _ulps16(got, want).max() <= 1
+    else:
+        # the reference adds the row's exponentials left to right in f32; the device adds them as a
+        # tree, so on long rows the two differ by the reference's own accumulated rounding.  Both
+        # are held to the exact value, the device more tightly.
+        import scipy.special
+        exact = scipy.special.logsumexp(x.astype(np.float64), axis=1)
+        np.testing.assert_allclose(got, exact, rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(want, exact, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_log_sum_exp_reference_literal_and_special_rows():
+    x = np.array([[1.0, 2.0, 3.0], [1.5, 0.5, -1.0]], np.float32)  # tests/tensor.rs:1885-1909
+    d_in, d_out = _dev(x), rocm.DeviceBuffer((2,), np.float32)
+    rocm.log_sum_exp_raw(np.float32, d_in.ptr, d_out.ptr, 2, 3)
+    np.testing.assert_allclose(d_out.numpy(), so.log_sum_exp(x), rtol=1e-6)
+    inf = np.inf
+    s = np.array([[-inf, 1.0, -inf], [-inf, -inf, -inf], [inf, 0.0, 1.0], [np.nan, 0.0, 1.0],
+                  [1000.0, 1000.0, 1000.0]], np.float32)
+    d_in, d_out = _dev(s), rocm.DeviceBuffer((5,), np.float32)
+    rocm.log_sum_exp_raw(np.float32, d_in.ptr, d_out.ptr, 5, 3)
+    got, want = d_out.numpy(), so.log_sum_exp(s)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(want).tolist() == [False, True, True, True, False]
+    np.testing.assert_allclose(got[[0, 4]], want[[0, 4]], rtol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int64])
+@pytest.mark.parametrize("shape,dim,index_len", [((2, 3), 1, 1), ((5, 7, 4), 0, 9), ((5, 7, 4), 1, 3),
+                                                 ((5, 7, 4), 2, 6), ((8192, 1000), 1, 1), ((3, 50257), 1, 5),
+                                                 ((64, 33, 128), 1, 40)])
+def test_gather(dtype, shape, dim, index_len):
+    rng = np.random.default_rng(sum(shape) + dim)
+    src = (rng.standard_normal(shape) * 100).astype(dtype)
+    ishape = list(shape)
+    ishape[dim] = index_len
+    idx = rng.integers(0, shape[dim], ishape).astype(np.int64)
+    left = int(np.prod(shape[:dim], dtype=np.int64))
+    right = int(np.prod(shape[dim + 1:], dtype=np.int64))
+    d_src, d_idx, d_out = _dev(src), _dev(idx), rocm.DeviceBuffer(ishape, dtype)
+    rocm.gather_raw(dtype, d_src.ptr, d_idx.ptr, d_out.ptr, left, shape[dim], index_len, right)
+    assert np.array_equal(d_out.numpy(), so.gather(src, dim, idx))
+
+
+@pytest.mark.gpu
+def test_gather_reference_literal():
+    data = np.array([[10, 20, 30], [40, 50, 60]], np.float32)  # tests/tensor.rs:2226-2257
+    idx = np.array([[1], [2]], np.int64)
+    d_src, d_idx, d_out = _dev(data), _dev(idx), rocm.DeviceBuffer((2, 1), np.float32)
+    rocm.gather_raw(np.float32, d_src.ptr, d_idx.ptr, d_out.ptr, 2, 3, 1, 1)
+    assert d_out.numpy().ravel().tolist() == [20.0, 60.0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("ishape,dim,dst_dim", [((2, 1), 1, 3), ((4, 6, 3), 0, 5), ((4, 6, 3), 1, 5),
+                                                ((4, 6, 3), 2, 2), ((8192, 1), 1, 1000), ((300, 1), 0, 3),
+                                                ((32, 50, 256), 1, 7), ((2000, 130), 0, 9)])
+def test_scatter_add_keeps_the_reference_order(dtype, ishape, dim, dst_dim):
+    rng = np.random.default_rng(sum(ishape) + dim)
+    src = (rng.standard_normal(ishape) * 20).astype(dtype)
+    idx = rng.integers(0, dst_dim, ishape).astype(np.int64)
+    dshape = list(ishape)
+    dshape[dim] = dst_dim
+    left = int(np.prod(ishape[:dim], dtype=np.int64))
+    right = int(np.prod(ishape[dim + 1:], dtype=np.int64))
+    d_src, d_idx = _dev(src), _dev(idx)
+    d_dst = rocm.DeviceBuffer(dshape, dtype, zeros=True)
+    rocm.scatter_add_raw(dtype, d_src.ptr, d_idx.ptr, d_dst.ptr, left, dst_dim, ishape[dim], right)
+    assert np.array_equal(d_dst.numpy(), so.scatter_add(src, dim, idx, dshape))  # same bits, collisions included
+
+
+@pytest.mark.gpu
+def test_gather_then_scatter_add_is_the_loss_path():
+    # src/loss.rs:11-24: gather(log_probs, 1, targets) forward, scatter_add of the upstream backward
+    n, v = 512, 1000
+    logp = _rand((n, v), 3, np.float32)
+    tgt = np.random.default_rng(4).integers(0, v, (n, 1)).astype(np.int64)
+    d_lp, d_t, d_pick = _dev(logp), _dev(tgt), rocm.DeviceBuffer((n, 1), np.float32)
+    rocm.gather_raw(np.float32, d_lp.ptr, d_t.ptr, d_pick.ptr, n, v, 1, 1)
+    assert np.array_equal(d_pick.numpy()[:, 0], logp[np.arange(n), tgt[:, 0]])
+    up = _rand((n, 1), 5, np.float32)
+    d_up, d_g = _dev(up), rocm.DeviceBuffer((n, v), np.float32, zeros=True)
+    rocm.scatter_add_raw(np.float32, d_up.ptr, d_t.ptr, d_g.ptr, n, v, 1, 1)
+    want = np.zeros((n, v), np.float32)
+    want[np.arange(n), tgt[:, 0]] = up[:, 0]
+    assert np.array_equal(d_g.numpy(), want)
+
+
+@pytest.mark.gpu
+def test_out_of_range_index_is_reported_at_the_next_sync():
+    src = _rand((4, 5), 1, np.float32)
+    idx = np.array([[0], [5], [1], [2]], np.int64)  # 5 is out of range
+    d_src, d_idx, d_out = _dev(src), _dev(idx), rocm.DeviceBuffer((4, 1), np.float32, zeros=True)
+    rocm.gather_raw(np.float32, d_src.ptr, d_idx.ptr, d_out.ptr, 4, 5, 1, 1)
+    with pytest.raises(rocm.RocmError, match="index"):
+        rocm.sync()
+    rocm.sync()  # the flag is cleared by the report
+    d_dst = rocm.DeviceBuffer((4, 5), np.float32, zeros=True)
+    bad = np.array([[0], [-1], [1], [2]], np.int64)
+    d_bad, d_up = _dev(bad), _dev(_rand((4, 1), 2, np.float32))
+    rocm.scatter_add_raw(np.float32, d_up.ptr, d_bad.ptr, d_dst.ptr, 4, 5, 1, 1)
+    with pytest.raises(rocm.RocmError, match="index"):
+        rocm.sync()
+    assert d_dst.numpy()[1].tolist() == [0.0] * 5  # the bad source was skipped
+
+
+@pytest.mark.gpu
+def test_argument_errors():
+    x = _dev(_rand((4, 4), 1, np.float32))
+    out = rocm.DeviceBuffer((4, 4), np.float32)
+    lib = rocm.load()
+    import ctypes
+    sh = (ctypes.c_int64 * 2)(4, 4)
+    assert lib.deers_rocm_unary(1, 99, x.ptr, 2, sh, None, ctypes.c_double(0), out.ptr) != 0
+    assert lib.deers_rocm_unary(1, 0, x.ptr, 0, sh, None, ctypes.c_double(0), out.ptr) != 0
+    assert lib.deers_rocm_unary(1, 0, x.ptr, 9, sh, None, ctypes.c_double(0), out.ptr) != 0
+    assert lib.deers_rocm_unary(1, 0, None, 2, sh, None, ctypes.c_double(0), out.ptr) != 0
+    assert lib.deers_rocm_unary(7, 0, x.ptr, 2, sh, None, ctypes.c_double(0), out.ptr) != 0
+    assert lib.deers_rocm_binary(1, 6, x.ptr, None, x.ptr, None, 2, sh, out.ptr) != 0
+    assert lib.deers_rocm_binary(1, 0, x.ptr, None, None, None, 2, sh, out.ptr) != 0
+    assert lib.deers_rocm_reduce(1, 2, x.ptr, out.ptr, ctypes.c_int64(4), ctypes.c_int64(4)) != 0
+    assert lib.deers_rocm_reduce(1, 0, x.ptr, out.ptr, ctypes.c_int64(4), ctypes.c_int64(0)) != 0
+    assert lib.deers_rocm_log_sum_exp(1, None, out.ptr, ctypes.c_int64(4), ctypes.c_int64(4)) != 0
+    assert lib.deers_rocm_gather(5, x.ptr, x.ptr, out.ptr, ctypes.c_int64(1), ctypes.c_int64(1),
+                                 ctypes.c_int64(1), ctypes.c_int64(1)) != 0
+    assert lib.deers_rocm_scatter_add(2, x.ptr, x.ptr, out.ptr, ctypes.c_int64(1), ctypes.c_int64(1),
+                                      ctypes.c_int64(1), ctypes.c_int64(1)) != 0
+    # empty inputs are fine
+    assert lib.deers_rocm_reduce(1, 0, None, None, ctypes.c_int64(0), ctypes.c_int64(4)) == 0
+    sh0 = (ctypes.c_int64 * 2)(0, 4)
+    assert lib.deers_rocm_unary(1, 0, None, 2, sh0, None, ctypes.c_double(0), None) == 0
+    rocm.sync()
