@@ -221,6 +221,64 @@ def bench_log_softmax(steps: int, warmup: int):
     return out
 
 
+def bench_storage(steps: int, warmup: int):
+    """The generic storage kernels at the shapes the reference's unfused attention chain gives
+    them at C2's geometry in f32 (src/models/gpt.rs:139-144: scores [8,12,1024,1024] = 403 MB):
+    scalar_mul, add of the head-broadcast mask, log_sum_exp over the rows, sub of the
+    row-broadcast lse, exp; plus row sum / max, a transposed (strided) unary pass, and the
+    loss's gather / scatter_add at [8192, 50257].  All HBM-bound; bytes are the algorithmic
+    minimum (every operand once)."""
+    B, H, T = C2["B"], C2["H"], C2["T"]
+    n = B * H * T * T
+    one = 4.0 * n
+    x = rocm.DeviceBuffer((B, H, T, T), np.float32)
+    rocm.fill_raw(np.float32, x.ptr, n, 0.25)
+    y = rocm.DeviceBuffer((B, H, T, T), np.float32)
+    z = rocm.DeviceBuffer((B, H, T, T), np.float32)
+    mask = rocm.DeviceBuffer((B, 1, T, T), np.float32, zeros=True)
+    rows = rocm.DeviceBuffer((B * H * T,), np.float32)
+    nv, vv = 8192, 50257
+    logp = rocm.DeviceBuffer((nv, vv), np.float32)  # 1.65 GB
+    rocm.fill_raw(np.float32, logp.ptr, nv * vv, -10.0)
+    tgt = rocm.DeviceBuffer.from_numpy(
+        (np.arange(nv, dtype=np.int64) * 7919 % vv).reshape(nv, 1))
+    pick = rocm.DeviceBuffer((nv, 1), np.float32)
+    shape = (B, H, T, T)
+    plan = [
+        ("unary_scalar_mul", 2 * one, lambda: rocm.unary_raw(np.float32, "scalar_mul", x.ptr, shape, None, 0.125, y.ptr)),
+        ("binary_add", 2 * one + 4.0 * B * T * T,
+         lambda: rocm.binary_raw(np.float32, "add", y.ptr, None, mask.ptr, [T * T, 0, T, 1], shape, z.ptr)),
+        ("log_sum_exp", one, lambda: rocm.log_sum_exp_raw(np.float32, z.ptr, rows.ptr, B * H * T, T)),
+        ("binary_sub", 2 * one + 4.0 * B * H * T,
+         lambda: rocm.binary_raw(np.float32, "sub", z.ptr, None, rows.ptr, [H * T, T, 1, 0], shape, y.ptr)),
+        ("unary_exp", 2 * one, lambda: rocm.unary_raw(np.float32, "exp", y.ptr, shape, None, 0.0, z.ptr)),
+        ("binary_mul", 3 * one, lambda: rocm.binary_raw(np.float32, "mul", x.ptr, None, z.ptr, None, shape, y.ptr)),
+        ("reduce_sum", one, lambda: rocm.reduce_raw(np.float32, "sum", z.ptr, rows.ptr, B * H * T, T)),
+        ("reduce_max", one, lambda: rocm.reduce_raw(np.float32, "max", z.ptr, rows.ptr, B * H * T, T)),
+        ("unary_neg", 2 * one,  # last two axes swapped: the strided path
+         lambda: rocm.unary_raw(np.float32, "neg", x.ptr, shape, [H * T * T, T * T, 1, T], 0.0, y.ptr)),
+        ("gather", 16.0 * nv, lambda: rocm.gather_raw(np.float32, logp.ptr, tgt.ptr, pick.ptr, nv, vv, 1, 1)),
+        ("scatter_add", 20.0 * nv, lambda: rocm.scatter_add_raw(np.float32, pick.ptr, tgt.ptr, logp.ptr, nv, vv, 1, 1)),
+    ]
+    strided_name = "unary_neg"
+    out = {"shape": list(shape), "dtype": "f32"}
+    for name, nbytes, fn in plan:
+        for _ in range(max(1, warmup // 4)):
+            fn()
+        rocm.sync()
+        rocm.profile_enable(True)
+        for _ in range(max(3, steps // 10)):
+            fn()
+        prof = rocm.profile_collect()
+        rocm.profile_enable(False)
+        calls, ms = prof[name]
+        us = 1e3 * ms / calls
+        key = name + ("_transposed_view" if name == strided_name else "")
+        out[key] = {"avg_us": us, "bytes_per_launch": nbytes, "GB/s": nbytes / (us * 1e-6) / 1e9,
+                    "frac_hbm_peak": nbytes / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
 def bench_adamw(steps: int, warmup: int):
     """Fused AdamW step over 124,439,808 f32 parameters (GPT-2 small, as one tensor), and
     the sum of squares of as many gradients.  HBM-bound: the step reads w, g, m, v and
@@ -365,7 +423,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gpt", action="store_true",
                     help="skip the end-to-end GPT training step reported beside the headline")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw", "gpt"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw", "gpt", "storage"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -387,6 +445,8 @@ def main():
         elif args.only == "adamw":
             print(json.dumps({"only": "adamw",
                               **bench_adamw(min(args.steps, 20), min(args.warmup, 5))}))
+        elif args.only == "storage":
+            print(json.dumps({"only": "storage", **bench_storage(args.steps, args.warmup)}))
         elif args.only == "gpt":
             print(json.dumps({"only": "gpt", **bench_gpt(min(args.steps, 10), min(args.warmup, 3))}))
         elif args.only == "copy":

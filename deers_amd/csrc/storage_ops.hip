@@ -131,6 +131,61 @@ __global__ __launch_bounds__(256) void binary_strided_kernel(const T* a, Strided
                               (float)b[view_offset(vb, (uint32_t)i)]);
 }
 
+// Strided operands whose innermost dimension is contiguous (stride 1) or broadcast
+// (stride 0), with an extent that is a multiple of a 16-byte chunk and chunk-aligned
+// outer strides: one index decomposition per chunk, 16-byte loads (or one scalar load
+// fanned out).  This is the shape of the attention chain's broadcasts: a [B,1,T,T] mask
+// over the heads, a [B,H,T,1] row statistic over the keys.
+template <typename T>
+__device__ __forceinline__ Vec16<T> load_chunk(const T* base, const StridedView& v, uint32_t elem) {
+  const T* p = base + view_offset(v, elem);
+  if (v.stride[v.ndim - 1] != 0) return *reinterpret_cast<const Vec16<T>*>(p);
+  Vec16<T> r;
+  const T x = *p;
+#pragma unroll
+  for (int e = 0; e < (int)(16 / sizeof(T)); ++e) r.e[e] = x;
+  return r;
+}
+template <typename T, int OP>
+__global__ __launch_bounds__(256) void unary_rows_kernel(const T* x, StridedView v, T* out,
+                                                         uint32_t n_chunks, float p) {
+  constexpr int kEpc = 16 / sizeof(T);
+  const uint32_t stride = gridDim.x * 256u;
+  for (uint64_t c = blockIdx.x * 256u + threadIdx.x; c < n_chunks; c += stride) {
+    const Vec16<T> vx = load_chunk(x, v, (uint32_t)c * kEpc);
+    Vec16<T> o;
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) o.e[e] = (T)unary_fn<OP>((float)vx.e[e], p);
+    store16(o, out + c * kEpc);
+  }
+}
+template <typename T, int OP>
+__global__ __launch_bounds__(256) void binary_rows_kernel(const T* a, StridedView va, const T* b,
+                                                          StridedView vb, T* out, uint32_t n_chunks) {
+  constexpr int kEpc = 16 / sizeof(T);
+  const uint32_t stride = gridDim.x * 256u;
+  for (uint64_t c = blockIdx.x * 256u + threadIdx.x; c < n_chunks; c += stride) {
+    const Vec16<T> xa = load_chunk(a, va, (uint32_t)c * kEpc), xb = load_chunk(b, vb, (uint32_t)c * kEpc);
+    Vec16<T> o;
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) o.e[e] = (T)binary_fn<OP>((float)xa.e[e], (float)xb.e[e]);
+    store16(o, out + c * kEpc);
+  }
+}
+// true if a chunk of 16 / elem_bytes consecutive elements (in row-major order over the
+// view's shape, starting at a multiple of the chunk) never straddles the view's
+// innermost dimension and can be fetched as described above
+inline bool chunkable(const void* base, const StridedView& v, int elem_bytes) {
+  const int epc = 16 / elem_bytes;
+  const int64_t s_in = v.stride[v.ndim - 1];
+  if (v.shape[v.ndim - 1] % epc != 0) return false;
+  if (s_in == 0) return true;  // scalar loads: no alignment needed
+  if (s_in != 1 || !aligned16(base)) return false;
+  for (int d = 0; d + 1 < v.ndim; ++d)
+    if (v.stride[d] % epc != 0) return false;
+  return true;
+}
+
 // ---- row reductions ----
 struct SumOp {
   static constexpr float kIdentity = 0.f;
@@ -302,6 +357,12 @@ void unary_t(const T* x, const StridedView* view, T* out, int64_t n, float p, hi
                        flat, out, (uint32_t)n, p);
     return;
   }
+  if (aligned16(out) && chunkable(x, *view, sizeof(T))) {
+    const uint32_t n_chunks = (uint32_t)(n / (16 / sizeof(T)));
+    hipLaunchKernelGGL((unary_rows_kernel<T, OP>), dim3(stream_blocks(n_chunks)), dim3(256), 0, stream, x,
+                       *view, out, n_chunks, p);
+    return;
+  }
   hipLaunchKernelGGL((unary_strided_kernel<T, OP>), dim3(stream_blocks(n)), dim3(256), 0, stream, x,
                      *view, out, (uint32_t)n, p);
 }
@@ -317,8 +378,16 @@ void binary_t(const T* a, const StridedView* va, const T* b, const StridedView* 
   flat.ndim = 1;
   flat.shape[0] = (uint32_t)n;
   flat.stride[0] = 1;
-  hipLaunchKernelGGL((binary_strided_kernel<T, OP>), dim3(stream_blocks(n)), dim3(256), 0, stream, a,
-                     va ? *va : flat, b, vb ? *vb : flat, out, (uint32_t)n);
+  const StridedView& wa = va ? *va : flat;
+  const StridedView& wb = vb ? *vb : flat;
+  if (aligned16(out) && chunkable(a, wa, sizeof(T)) && chunkable(b, wb, sizeof(T))) {
+    const uint32_t n_chunks = (uint32_t)(n / (16 / sizeof(T)));
+    hipLaunchKernelGGL((binary_rows_kernel<T, OP>), dim3(stream_blocks(n_chunks)), dim3(256), 0, stream, a,
+                       wa, b, wb, out, n_chunks);
+    return;
+  }
+  hipLaunchKernelGGL((binary_strided_kernel<T, OP>), dim3(stream_blocks(n)), dim3(256), 0, stream, a, wa,
+                     b, wb, out, (uint32_t)n);
 }
 
 template <typename T, int... OPS>

@@ -155,6 +155,21 @@ def test_binary_eq_and_special_values(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("T", [64, 33])
+def test_binary_row_statistic_broadcast_along_the_last_axis(dtype, T):
+    # x - lse with lse [B,H,T,1] broadcast over the keys (src/tensor.rs:456-458): innermost stride 0
+    B, H = 2, 3
+    x = _rand((B, H, T, T), 12, dtype)
+    lse = _rand((B, H, T, 1), 13, dtype)
+    dx, dl, d_out = _dev(x), _dev(lse), rocm.DeviceBuffer(x.shape, dtype)
+    rocm.binary_raw(dtype, "sub", dx.ptr, None, dl.ptr, [H * T, T, 1, 0], x.shape, d_out.ptr)
+    _same(d_out.numpy(), so.binary("sub", x, np.broadcast_to(lse, x.shape)), True)
+    rocm.binary_raw(dtype, "mul", dl.ptr, [H * T, T, 1, 0], dx.ptr, [H * T * T, T * T, 1, T], x.shape, d_out.ptr)
+    _same(d_out.numpy(), so.binary("mul", np.broadcast_to(lse, x.shape), x.transpose(0, 1, 3, 2)), True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("outer,rs", [(2, 3), (1, 1), (1000, 7), (513, 32), (77, 33), (300, 257), (64, 4096),
                                       (5, 50257), (3, 70001), (4096, 64)])
 def test_reduce(dtype, outer, rs):
