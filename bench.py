@@ -221,6 +221,39 @@ def bench_log_softmax(steps: int, warmup: int):
     return out
 
 
+def bench_composed_chain(steps: int, warmup: int):
+    """C2's forward as the reference's own op chain on the device (seven storage kernels and
+    two [8,12,1024,1024] f16 intermediates, rocm.attn_fwd_composed_raw) beside the fused kernel
+    on the same inputs: what fusing buys on this GPU, not a headline number."""
+    B, H, T, D = C2["B"], C2["H"], C2["T"], C2["D"]
+    dt = np.float16
+    q, k, v = (rocm.DeviceBuffer.from_numpy(
+        synth.normal((B, H, T, D), synth.tensor_seed(0, "c2", n), 1.0).astype(dt)) for n in "qkv")
+    mask = rocm.DeviceBuffer.from_numpy(rocm.causal_mask_host(B, T, dt))
+    o = rocm.DeviceBuffer((B, H, T, D), dt)
+    lse16 = rocm.DeviceBuffer((B, H, T), dt)
+    lse32 = rocm.DeviceBuffer((B, H, T), np.float32)
+    s, p = rocm.DeviceBuffer((B, H, T, T), dt), rocm.DeviceBuffer((B, H, T, T), dt)
+    scale = rocm.default_scale(D)
+    reps = max(5, steps // 10)
+    times = {}
+    for name, fn in (("composed", lambda: rocm.attn_fwd_composed_raw(dt, q.ptr, k.ptr, v.ptr, mask.ptr, o.ptr,
+                                                                     lse16.ptr, s.ptr, p.ptr, B, H, T, D, scale)),
+                     ("fused", lambda: rocm.attn_fwd_raw(dt, q.ptr, k.ptr, v.ptr, o.ptr, lse32.ptr, B, H, T, D, scale))):
+        for _ in range(3):
+            fn()
+        rocm.sync()
+        t = rocm.Timer()
+        t.start()
+        for _ in range(reps):
+            fn()
+        t.stop()
+        times[name] = 1e3 * t.elapsed_ms() / reps
+    return {"composed_chain_us": times["composed"], "fused_kernel_us": times["fused"],
+            "ratio": times["composed"] / times["fused"],
+            "intermediate_bytes": 2.0 * B * H * T * T * 2}
+
+
 def bench_storage(steps: int, warmup: int):
     """The generic storage kernels at the shapes the reference's unfused attention chain gives
     them at C2's geometry in f32 (src/models/gpt.rs:139-144: scores [8,12,1024,1024] = 403 MB):
@@ -262,6 +295,7 @@ def bench_storage(steps: int, warmup: int):
     ]
     strided_name = "unary_neg"
     out = {"shape": list(shape), "dtype": "f32"}
+    out["attention_forward_composed_f16_c2"] = bench_composed_chain(steps, warmup)
     for name, nbytes, fn in plan:
         for _ in range(max(1, warmup // 4)):
             fn()

@@ -409,6 +409,44 @@ def attn_fwd(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float | None = 
     return o.numpy(), lse.numpy()
 
 
+def attn_fwd_composed_raw(dtype, q, k, v, mask, o, lse, s, p, B, H, T, D, scale):
+    """The reference's own op chain for the attention core (src/models/gpt.rs:139-144,
+    softmax of src/tensor.rs:456-458) on the device, one storage kernel per tensor op:
+    matmul, scalar_mul, add of the [B,1,T,T] mask broadcast over the heads, log_sum_exp,
+    sub of the [B,H,T,1] statistic broadcast over the keys, exp, matmul.  What a
+    Device::Rocm backend executes where the fused op does not apply (any head width).
+    `s`, `p`: two [B,H,T,T] scratch buffers of `dtype`; `lse`: [B,H,T] of `dtype`."""
+    BH, shape = B * H, (B, H, T, T)
+    matmul_raw(dtype, q, (D, 1, T * D), k, (1, D, T * D), s, BH, T, T, D)            # q @ k^T
+    unary_raw(dtype, "scalar_mul", s, shape, None, scale, p)                          # * scale
+    binary_raw(dtype, "add", p, None, mask, [T * T, 0, T, 1], shape, s)               # + mask
+    log_sum_exp_raw(dtype, s, lse, BH * T, T)
+    binary_raw(dtype, "sub", s, None, lse, [H * T, T, 1, 0], shape, p)                # - lse
+    unary_raw(dtype, "exp", p, shape, None, 0.0, s)
+    matmul_raw(dtype, s, (T, 1, T * T), v, (D, 1, T * D), o, BH, T, D, T)             # @ v
+
+
+def causal_mask_host(B: int, T: int, dtype) -> np.ndarray:
+    """Additive mask [B,1,T,T]: -inf above the diagonal, as src/nn/functional.rs:12-55 builds it
+    on the host before every forward."""
+    m = np.where(np.triu(np.ones((T, T), bool), 1), -np.inf, 0.0).astype(dtype)
+    return np.ascontiguousarray(np.broadcast_to(m, (B, 1, T, T)))
+
+
+def attn_fwd_composed(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float | None = None):
+    """Returns (o, lse) computed by the unfused chain; compact [B,H,T,D] inputs of one dtype."""
+    B, H, T, D = q.shape
+    scale = default_scale(D) if scale is None else scale
+    bq, bk, bv = (DeviceBuffer.from_numpy(a) for a in (q, k, v))
+    mask = DeviceBuffer.from_numpy(causal_mask_host(B, T, q.dtype))
+    o = DeviceBuffer(q.shape, q.dtype)
+    lse = DeviceBuffer((B, H, T), q.dtype)
+    s, p = DeviceBuffer((B, H, T, T), q.dtype), DeviceBuffer((B, H, T, T), q.dtype)
+    attn_fwd_composed_raw(q.dtype, bq.ptr, bk.ptr, bv.ptr, mask.ptr, o.ptr, lse.ptr, s.ptr, p.ptr,
+                          B, H, T, D, scale)
+    return o.numpy(), lse.numpy()
+
+
 def attn_fwd_bwd(q, k, v, do, scale: float | None = None):
     """Returns (o, lse, dq, dk, dv): forward then backward through the C ABI."""
     B, H, T, D = q.shape
