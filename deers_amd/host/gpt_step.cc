@@ -19,15 +19,18 @@
 
 using namespace deers_host;
 
-// gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens:
+// gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens [tune]:
 // greedy generation with KV caches on an f16 model; times the decode steps that follow
-// the prompt.
+// the prompt.  `tune` picks the library GEMM kernel of each of the step's four problems by
+// timing during the prompt.
 static int run_generate(int argc, char** argv) {
   if (argc < 11) {
-    std::fprintf(stderr, "usage: gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens\n");
+    std::fprintf(stderr, "usage: gpt_step generate vocab seq n_layer n_head n_embd mlp_hidden batch prompt_len new_tokens [tune]\n");
     return 2;
   }
   check(deers_rocm_init(0));
+  const bool tune = argc > 11 && std::string(argv[11]) == "tune";
+  check(deers_rocm_matmul_tune(tune ? 1 : 0));
   GPTConfig cfg;
   cfg.vocab_size = std::atoll(argv[2]);
   cfg.sequence_len = std::atoll(argv[3]);

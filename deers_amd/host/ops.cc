@@ -520,19 +520,31 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   const int dt = (int)x_t.dtype();
   const size_t el = size_in_bytes(x_t.dtype());
   const Tensor x_flat = x_t.reshape({B, C});
-  const Tensor q = x_flat.matmul(wq_), k = x_flat.matmul(wk_), v = x_flat.matmul(wv_);  // [B, H*D]
+  if (!cache.wqkv.defined()) {
+    cache.wqkv = empty({C, 3 * C}, x_t.dtype(), true);
+    const Tensor* w[3] = {&wq_, &wk_, &wv_};
+    for (int i = 0; i < 3; ++i) {
+      const Tensor wc = w[i]->compact();
+      const int64_t wshape[2] = {C, C}, src[2] = {C, 1}, dst[2] = {3 * C, 1};
+      check(deers_rocm_copy_view(dt, wc.data(), src, (char*)cache.wqkv.data() + i * C * el, dst, wshape, 2));
+    }
+  }
+  const Tensor qkv = x_flat.matmul(cache.wqkv);  // [B, 3C]: q | k | v, each [B, H*D]
+  const char* q_data = (const char*)qkv.data();
+  const char* k_data = q_data + C * el;
+  const char* v_data = q_data + 2 * C * el;
   // row `pos` of the compact [1,T,1,D/2] tables
   const Tensor cc = cos.compact(), sc = sin.compact();
   const char* cos_t = (const char*)cc.data() + pos * (D / 2) * el;
   const char* sin_t = (const char*)sc.data() + pos * (D / 2) * el;
-  const int64_t x_strides[4] = {H * D, H * D, D, 1};                 // [B,1,H,D] over [B, H*D]
+  const int64_t x_strides[4] = {3 * C, 3 * C, D, 1};                 // [B,1,H,D] inside a [B, 3C] row
   const int64_t cache_strides[4] = {H * cap * D, cap * D, D, 1};     // [B,H,1,D] at one cache row
   Tensor qh = empty({B, H, D}, x_t.dtype(), true);
-  check(deers_rocm_rope_fwd(dt, q.data(), x_strides, cos_t, sin_t, qh.data(), nullptr, B, 1, H, D));
-  check(deers_rocm_rope_fwd(dt, k.data(), x_strides, cos_t, sin_t,
+  check(deers_rocm_rope_fwd(dt, q_data, x_strides, cos_t, sin_t, qh.data(), nullptr, B, 1, H, D));
+  check(deers_rocm_rope_fwd(dt, k_data, x_strides, cos_t, sin_t,
                             (char*)cache.k.data() + pos * D * el, cache_strides, B, 1, H, D));
-  const int64_t shape[3] = {B, H, D}, v_src[3] = {H * D, D, 1}, v_dst[3] = {H * cap * D, cap * D, 1};
-  check(deers_rocm_copy_view(dt, v.data(), v_src, (char*)cache.v.data() + pos * D * el, v_dst, shape, 3));
+  const int64_t shape[3] = {B, H, D}, v_src[3] = {3 * C, D, 1}, v_dst[3] = {H * cap * D, cap * D, 1};
+  check(deers_rocm_copy_view(dt, v_data, v_src, (char*)cache.v.data() + pos * D * el, v_dst, shape, 3));
   cache.len = pos + 1;
   Tensor o = empty({B, H * D}, x_t.dtype(), true);
   const int64_t kv_strides[3] = {H * cap * D, cap * D, D};

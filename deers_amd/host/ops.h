@@ -232,6 +232,10 @@ Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
 // token (examples/tinystories_train.rs:250-276).
 struct KvCache {
   Tensor k, v;
+  // [C, 3C] = (Wq | Wk | Wv), packed by the first decode_step that uses this cache so a
+  // step runs one projection GEMM instead of three; the weights must not change while
+  // the cache lives
+  Tensor wqkv;
   int64_t len = 0, capacity = 0;
   static KvCache create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType dtype);
 };
