@@ -4,6 +4,11 @@
 // causal_mask + add, log_sum_exp, sub, exp, matmul) with one kernel that never
 // materialises the [T,T] score tensor.
 //
+// Two kernels share this decomposition: the software-pipelined one described below
+// (two workgroups per CU) and, for D = 64 launches whose tiles number between two and
+// three per CU, a plain one at three workgroups per CU with every workgroup resident
+// from the start (attn_fwd_f16_resident_kernel, further down).
+//
 // Work decomposition
 //   grid  = one workgroup per (head, 128-row query tile), dealt to the XCDs so a
 //           head stays on one XCD; 256 threads = 4 waves; wave w owns query rows
@@ -29,7 +34,11 @@
 // (global_load_lds_dwordx4) into rings of P+1 slots, requested P iterations ahead
 // of their use so HBM/L2 latency is off the critical path; tiles are unpadded and
 // XOR-swizzled by 16-byte chunk.  One barrier per iteration.
+#include <algorithm>
+#include <map>
+#include <tuple>
 #include <type_traits>
+#include <vector>
 
 #include "common.h"
 
@@ -90,6 +99,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
   const half_t* V = (const half_t*)p.v + b * p.sv.b + h * p.sv.h;
   half_t* O = (half_t*)p.o + b * p.so.b + h * p.so.h;
 
+  [[maybe_unused]] const int trace_row = blockIdx.x;
   DEERS_TRACE_POINT(0);
   const int q0 = qtile * kFwdBM;
   const int qw0 = q0 + 32 * wave;        // first query row of this wave
@@ -240,10 +250,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
     request(j + 1 + P, j - 1 + P);
-    // D <= 64: every fragment of the iteration is fetched here, ahead of the vector work.
-    // D = 128: that would be 128 registers of operands; instead a window of kJit
-    // fragments runs ahead of the MFMAs that consume them (see the chunk loop).
-    constexpr bool JIT = D == 128;
+    // D = 32: every fragment of the iteration is fetched here, ahead of the vector work.
+    // D >= 64: a window of kJit fragments runs ahead of the MFMAs that consume them (see
+    // the chunk loop).  At D = 128 the whole set would be 128 registers of operands; at
+    // D = 64 the window spreads the LDS reads over the iteration instead of issuing all
+    // 24 behind the barrier, where four waves' bursts queue up (31.5 -> 30.7 us at
+    // 8x12x1024x64, 252 -> 208 registers).
+    constexpr bool JIT = D >= 64;
     constexpr int kJit = 4;
     constexpr int NMS_ = HAS_S ? 2 * KS : 0;
     constexpr int NM_ = NMS_ + (HAS_PV ? 4 * DB : 0);
@@ -432,6 +445,259 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
   DEERS_TRACE_POINT(30);
 }
 
+// ---- variant: three workgroups per CU, no software pipeline inside the wave ----
+// Each iteration is S = K Q^T, softmax, O += V^T P in program order on ONE S
+// accumulator; the overlap of matrix and vector work comes from three waves per SIMD
+// instead of from interleaving inside one (<= 168 registers).  K(j) and V(j) travel
+// together, P iterations ahead.
+template <int D>
+__global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams p, int BH, int n_qtiles,
+                                                                   int heads_per_xcd,
+                                                                   const int32_t* __restrict__ order) {
+  using Cfg = FwdCfg<D>;
+  constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
+  constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
+  constexpr int RPW = 1024 / RB, NWLW = TILE_B / 4096, LPI = 2 * NWLW;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5;
+  const int T = p.T;
+  int bh, qtile;
+  if (order) {  // every workgroup is resident at once: position -> tile chosen for even CU totals
+    const int code = order[blockIdx.x >> 3];
+    bh = (code >> 16) * 8 + (blockIdx.x & 7);
+    qtile = code & 0xffff;
+    if (bh >= BH) return;
+  } else {
+    int rank;
+    if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
+    qtile = n_qtiles - 1 - rank;
+  }
+  [[maybe_unused]] const int trace_row = blockIdx.x;
+  DEERS_TRACE_POINT(0);
+  const int b = bh / p.H, h = bh % p.H;
+  const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
+  const half_t* K = (const half_t*)p.k + b * p.sk.b + h * p.sk.h;
+  const half_t* V = (const half_t*)p.v + b * p.sv.b + h * p.sv.h;
+  half_t* O = (half_t*)p.o + b * p.so.b + h * p.so.h;
+  const int q0 = qtile * kFwdBM, qw0 = q0 + 32 * wave, qrow = qw0 + (lane & 31);
+  const int n_tiles = min(q0 + kFwdBM - 1, T - 1) / kFwdBN + 1;
+  const uint32_t lds0 = lds_address(smem);
+  const int tail_tile = (T - 1) / kFwdBN;
+  const int skt = (int)p.sk.t, svt = (int)p.sv.t;
+  uint32_t ld_k[NWLW], ld_v[NWLW], ld_k_tail[NWLW], ld_v_tail[NWLW];
+#pragma unroll
+  for (int i = 0; i < NWLW; ++i) {
+    const int row = (wave * NWLW + i) * RPW + lane / CH;
+    const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
+    const int row_tail = min(row, T - 1 - tail_tile * kFwdBN);
+    ld_k[i] = (uint32_t)(row * skt * 2 + col);
+    ld_v[i] = (uint32_t)(row * svt * 2 + col);
+    ld_k_tail[i] = (uint32_t)(row_tail * skt * 2 + col);
+    ld_v_tail[i] = (uint32_t)(row_tail * svt * 2 + col);
+  }
+  auto request = [&](int t) {  // K(t) and V(t) into slot t % NS; past the end: clamped, never consumed
+    const int tc = min(t, n_tiles - 1);
+    const uint32_t kdst = lds0 + (t % NS) * TILE_B + wave * (NWLW * 1024);
+    const uint32_t vdst = kdst + NS * TILE_B;
+    const half_t* kbase = K + (uint32_t)(tc * kFwdBN * skt);
+    const half_t* vbase = V + (uint32_t)(tc * kFwdBN * svt);
+#pragma unroll
+    for (int i = 0; i < NWLW; ++i) {
+      async_load16_to_lds(kbase, tc == tail_tile ? ld_k_tail[i] : ld_k[i], kdst + i * 1024);
+      async_load16_to_lds(vbase, tc == tail_tile ? ld_v_tail[i] : ld_v[i], vdst + i * 1024);
+    }
+  };
+#pragma unroll
+  for (int t = 0; t < P; ++t) request(t);
+  half8 qf[KS];
+  {
+    const half_t* qp = Q + (int64_t)min(qrow, T - 1) * p.sq.t + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const half8*)(qp + 16 * ks);
+  }
+  int koff[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    koff[ks] = (lane & 31) * RB + (((2 * ks + g) ^ lds_swizzle<CH>(lane & 31)) << 4);
+  int voff_lo[DB], voff_hi[DB];
+  {
+    const int lrow = 4 * g + ((lane & 15) >> 2);
+    const int c4 = lane & 3;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + (c4 >> 1);
+      voff_lo[db] = lrow * RB + ((chunk ^ lds_swizzle<CH>(lrow)) << 4) + (c4 & 1) * 8;
+      voff_hi[db] = (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
+    }
+  }
+  floatx16 oacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) oacc[i] = ZERO16;
+  float m = -INFINITY, lsum = 0.f;
+  const float c = p.scale_log2;
+  wait_all_vmem();  // Q fragments (and with them every request so far)
+  DEERS_TRACE_POINT(1);
+
+  for (int j = 0; j < n_tiles; ++j) {
+    const int kv0 = j * kFwdBN;
+    wait_vmcnt<(P - 1) * LPI>();
+    __syncthreads();
+    request(j + P);
+    const uint32_t kb = lds0 + (j % NS) * TILE_B;
+    const uint32_t vb = kb + NS * TILE_B;
+    // ---- S^T = K Q^T ----
+    floatx16 c0 = ZERO16, c1 = ZERO16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint32_t addr = opaque(kb + koff[ks]);
+      const half8 a0 = *(DEERS_LDS const half8*)(uintptr_t)addr;
+      const half8 a1 = *(DEERS_LDS const half8*)(uintptr_t)(addr + 32 * RB);
+      c0 = mfma_f16(a0, qf[ks], c0);
+      c1 = mfma_f16(a1, qf[ks], c1);
+    }
+    // V fragments of the first half of the PV product, fetched while the vector pipe works
+    constexpr int kVPre = 1;  // 16-key groups of V fetched ahead
+    half8 vfr[kVPre * DB];
+#pragma unroll
+    for (int ms = 0; ms < kVPre; ++ms)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const uint32_t ro = 16 * ms * RB;
+        const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
+        const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
+        vfr[ms * DB + db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    if (kv0 + kFwdBN - 1 > qw0) {
+      const int dist = qrow - 4 * g - kv0;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kr = 8 * (r >> 2) + (r & 3);
+        if (kr > dist) c0[r] = -INFINITY;
+        if (kr + 32 > dist) c1[r] = -INFINITY;
+      }
+    }
+    float mx4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mx4[i] = fmaxf(c0[i], c1[i]);
+#pragma unroll
+    for (int r = 4; r < 16; ++r) mx4[r & 3] = fmaxf(fmaxf(mx4[r & 3], c0[r]), c1[r]);
+    float mx = pair_max(fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3])));
+    if (__any((mx - m) * c > kLazyRescale)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = fast_exp2((m - m_new) * c);
+      m = m_new;
+      lsum *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+    }
+    const float mc = m * c;
+    uint32_t pw[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      floatx16& cc = (i < 8) ? c0 : c1;
+      const int r = 2 * (i & 7);
+      const float e0 = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
+      const float e1 = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
+      pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)e0, (half_t)e1});
+      lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
+    }
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int ms = 0; ms < 4; ++ms) {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const half8 pb = __builtin_bit_cast(half8, u32x4{pw[4 * ms], pw[4 * ms + 1], pw[4 * ms + 2], pw[4 * ms + 3]});
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        half8 a;
+        if (ms < kVPre) {
+          a = vfr[ms * DB + db];
+        } else {
+          const uint32_t ro = 16 * ms * RB;
+          const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
+          const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
+          a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+        oacc[db] = mfma_f16(a, pb, oacc[db]);
+      }
+    }
+    DEERS_TRACE_POINT(2 + j);
+  }
+  lsum = pair_sum(lsum);
+  if (qrow < T) {
+    const float inv = 1.f / lsum;
+    half_t* orow = O + (int64_t)qrow * p.so.t;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) store_block_f16(orow + 32 * db, oacc[db], inv, g);
+    if (g == 0) p.lse[(int64_t)bh * T + qrow] = (m * c + fast_log2(lsum)) * kLn2;
+  }
+  DEERS_TRACE_POINT(30);
+}
+
+// Position -> tile table for a launch whose workgroups are all resident at once (their
+// number does not exceed what the chip holds).  Workgroup position p of an XCD (id / 8)
+// lands on CU p % cus_per_xcd when the dispatcher fills an empty chip, so positions p,
+// p + cus, p + 2 cus share a CU and its issue ports: tiles are dealt longest first to the
+// CU with the smallest total that still has a free slot.  Returns nullptr when the tiles
+// do not all fit (then the dispatcher's own longest-first hand-out is the better order)
+// or fit the pipelined kernel's two workgroups per CU as well.
+// Built at the first launch of a geometry and kept for the life of the process.
+template <int D>
+static const int32_t* resident_order(int heads_per_xcd, int T) {
+  struct Key {
+    int dev, heads, T;
+    bool operator<(const Key& o) const { return std::tie(dev, heads, T) < std::tie(o.dev, o.heads, o.T); }
+  };
+  static std::map<Key, const int32_t*> cache;  // launches are serialised by the caller
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const Key key{dev, heads_per_xcd, T};
+  auto it = cache.find(key);
+  if (it != cache.end()) return it->second;
+  int cus = 0, per_cu = 0;
+  (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_fwd_f16_resident_kernel<D>, 256,
+                                                     FwdCfg<D>::kLds);
+  const int n_cu = std::max(cus / 8, 1);
+  const int n_qtiles = (T + kFwdBM - 1) / kFwdBM;
+  const int n_items = heads_per_xcd * n_qtiles;
+  const int32_t* result = nullptr;
+  if (per_cu > 2 && n_items > 2 * n_cu && n_items <= n_cu * per_cu) {
+    struct Item { int cost, code; };
+    std::vector<Item> items;
+    for (int qt = n_qtiles - 1; qt >= 0; --qt)
+      for (int h = 0; h < heads_per_xcd; ++h)
+        items.push_back({std::min(T - 1, qt * kFwdBM + kFwdBM - 1) / kFwdBN + 1, (h << 16) | qt});
+    std::vector<long> load(n_cu, 0);
+    std::vector<int> used(n_cu, 0);
+    std::vector<int32_t> host((size_t)n_items, 0);
+    std::vector<char> filled((size_t)n_cu * per_cu, 0);
+    for (const Item& item : items) {  // items are in descending cost already
+      int best = -1;
+      for (int c = 0; c < n_cu; ++c)
+        if (used[c] < per_cu && (size_t)(used[c] * n_cu + c) < host.size() &&
+            (best < 0 || load[c] < load[best]))
+          best = c;
+      if (best < 0) break;
+      host[(size_t)used[best] * n_cu + best] = item.code;
+      filled[(size_t)used[best] * n_cu + best] = 1;
+      load[best] += item.cost;
+      ++used[best];
+    }
+    bool complete = true;
+    for (int i = 0; i < n_items; ++i) complete = complete && filled[i];
+    if (complete) {
+      int32_t* dev_table = nullptr;
+      if (hipMalloc(&dev_table, host.size() * sizeof(int32_t)) == hipSuccess &&
+          hipMemcpy(dev_table, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess)
+        result = dev_table;
+    }
+  }
+  cache.emplace(key, result);
+  return result;
+}
+
 template <int D>
 static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
   const int BH = B * p.H;
@@ -445,6 +711,18 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
     attr_set = true;
   }
   LaunchScope scope("attn_fwd_f16", stream);
+  if constexpr (D == 64) {
+    // More tiles than the pipelined kernel holds at once (two workgroups per CU) but no
+    // more than the three-per-CU kernel does: every workgroup is resident from the start,
+    // placed for even CU totals, and nothing is left to a tail of late, short workgroups
+    // (8x12x1024x64: 32.2 -> 30.0 us; 4x12x2048x64: 49.5 -> 48.2 us).  Smaller and
+    // larger launches are as fast or faster on the pipelined kernel.
+    if (const int32_t* order = resident_order<D>(heads_per_xcd, p.T)) {
+      hipLaunchKernelGGL(attn_fwd_f16_resident_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
+                         stream, p, BH, n_qtiles, heads_per_xcd, order);
+      return;
+    }
+  }
   hipLaunchKernelGGL(attn_fwd_f16_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
                      stream, p, BH, n_qtiles, heads_per_xcd);
 }

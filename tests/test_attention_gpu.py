@@ -98,6 +98,22 @@ def test_config2_f16_full_size():
         np.testing.assert_array_equal(a, b)                           # no atomics: bit-reproducible
 
 
+@pytest.mark.parametrize("B,H,T", [(5, 16, 1000), (3, 25, 897), (4, 12, 2048)])
+def test_forward_with_every_workgroup_resident(B, H, T):
+    """f16 D=64 geometries with between two and three query tiles per CU and XCD: the forward
+    takes the three-workgroups-per-CU kernel with the placement table (ragged last tile, a head
+    count that does not fill the last round of XCDs, and the 2048-token case).  The oracle runs
+    on the first and last batch entries; the whole output is checked for finiteness, the first
+    row, and bit-reproducibility."""
+    x = synth.attention_inputs(f"resident-{B}-{H}-{T}", B, H, T, 64, np.float16, base_seed=3)
+    o, lse, dq, dk, dv = check_case(x, 5e-3, f"resident B{B} H{H} T{T}", heads=[0, B - 1])
+    assert np.isfinite(o.astype(np.float32)).all() and np.isfinite(lse).all()
+    np.testing.assert_array_equal(o[:, :, 0], x["v"][:, :, 0])
+    o2, lse2 = rocm.attn_fwd(x["q"], x["k"], x["v"])
+    np.testing.assert_array_equal(o, o2)
+    np.testing.assert_array_equal(lse, lse2)
+
+
 def test_config3_long_context_f16():
     """B=1 H=16 T=8192 D=128 f16, sigma 0.5: GPU on all heads, oracle on heads 0 and 15."""
     x = synth.attention_inputs("c3", 1, 16, 8192, 128, np.float16, base_seed=0, sigma=0.5)
