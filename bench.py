@@ -512,7 +512,7 @@ def main():
     # HBM bytes per launch at this shape from the FETCH_SIZE / WRITE_SIZE passes of
     # profiles/c2_c4_hbm_traffic_fetch_write.txt (scaled by what the same counters read
     # for a copy of known size); a profiler measurement, not taken in this run.
-    measured_traffic = {"attn_bwd_f16": 146.5e6, "attn_fwd_f16": 53.1e6}
+    measured_traffic = {"attn_bwd_f16": 145.0e6, "attn_fwd_f16": 50.9e6}
     roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": (achieved / PEAK_F16_TFLOPS) if achieved else None,
                 "traffic": measured_traffic.get(dom), "avg_launch_us": kern[dom]["avg_us"],
