@@ -5,8 +5,8 @@
 // materialises the [T,T] score tensor.
 //
 // Two kernels share this decomposition: the software-pipelined one described below
-// (two workgroups per CU) and, for D = 64 launches whose tiles number between two and
-// three per CU, a plain one at three workgroups per CU with every workgroup resident
+// (two workgroups per CU) and, for D <= 64 launches whose tiles number more than two per
+// CU but no more than fit at once, a plain one at three or four workgroups per CU with every workgroup resident
 // from the start (attn_fwd_f16_resident_kernel, further down).
 //
 // Work decomposition
@@ -711,12 +711,13 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
     attr_set = true;
   }
   LaunchScope scope("attn_fwd_f16", stream);
-  if constexpr (D == 64) {
+  if constexpr (D <= 64) {
     // More tiles than the pipelined kernel holds at once (two workgroups per CU) but no
     // more than the three-per-CU kernel does: every workgroup is resident from the start,
     // placed for even CU totals, and nothing is left to a tail of late, short workgroups
-    // (8x12x1024x64: 32.2 -> 30.0 us; 4x12x2048x64: 49.5 -> 48.2 us).  Smaller and
-    // larger launches are as fast or faster on the pipelined kernel.
+    // (8x12x1024x64: 32.2 -> 30.0 us; 4x12x2048x64: 49.5 -> 48.2 us; 8x12x1024x32, where
+    // four workgroups fit: 22.9 -> 20.6 us).  Smaller and larger launches are as fast or
+    // faster on the pipelined kernel.
     if (const int32_t* order = resident_order<D>(heads_per_xcd, p.T)) {
       hipLaunchKernelGGL(attn_fwd_f16_resident_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
                          stream, p, BH, n_qtiles, heads_per_xcd, order);
