@@ -445,6 +445,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
   DEERS_TRACE_POINT(30);
 }
 
+// Position -> tile table of a launch whose workgroups are all resident at once, passed in
+// the kernel arguments: entry p = (head index within the XCD) << 16 | query tile for the
+// workgroup at position p = blockIdx.x / 8 of its XCD.
+constexpr int kMaxResidentTiles = 128;  // per XCD: 32 CUs x at most 4 workgroups
+struct TileOrder {
+  int32_t code[kMaxResidentTiles];
+};
+
 // ---- variant: three workgroups per CU, no software pipeline inside the wave ----
 // Each iteration is S = K Q^T, softmax, O += V^T P in program order on ONE S
 // accumulator; the overlap of matrix and vector work comes from three waves per SIMD
@@ -452,8 +460,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
 // together, P iterations ahead.
 template <int D>
 __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams p, int BH, int n_qtiles,
-                                                                   int heads_per_xcd,
-                                                                   const int32_t* __restrict__ order) {
+                                                                   int heads_per_xcd, TileOrder order) {
   using Cfg = FwdCfg<D>;
   constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -463,17 +470,11 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  int bh, qtile;
-  if (order) {  // every workgroup is resident at once: position -> tile chosen for even CU totals
-    const int code = order[blockIdx.x >> 3];
-    bh = (code >> 16) * 8 + (blockIdx.x & 7);
-    qtile = code & 0xffff;
-    if (bh >= BH) return;
-  } else {
-    int rank;
-    if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
-    qtile = n_qtiles - 1 - rank;
-  }
+  // every workgroup is resident at once: position -> tile chosen for even CU totals
+  const int code = order.code[blockIdx.x >> 3];
+  const int bh = (code >> 16) * 8 + (blockIdx.x & 7);
+  const int qtile = code & 0xffff;
+  if (bh >= BH) return;
   [[maybe_unused]] const int trace_row = blockIdx.x;
   DEERS_TRACE_POINT(0);
   const int b = bh / p.H, h = bh % p.H;
@@ -635,26 +636,31 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
   DEERS_TRACE_POINT(30);
 }
 
-// Position -> tile table for a launch whose workgroups are all resident at once (their
+// Builds the TileOrder of a launch whose workgroups are all resident at once (their
 // number does not exceed what the chip holds).  Workgroup position p of an XCD (id / 8)
 // lands on CU p % cus_per_xcd when the dispatcher fills an empty chip, so positions p,
 // p + cus, p + 2 cus share a CU and its issue ports: tiles are dealt longest first to the
 // CU with the smallest total that still has a free slot.  Returns nullptr when the tiles
 // do not all fit (then the dispatcher's own longest-first hand-out is the better order)
-// or fit the pipelined kernel's two workgroups per CU as well.
-// Built at the first launch of a geometry and kept for the life of the process.
+// or fit the pipelined kernel's two workgroups per CU as well.  Built at the first launch
+// of a geometry and kept on the host for the life of the process; no device memory.
 template <int D>
-static const int32_t* resident_order(int heads_per_xcd, int T) {
+static const TileOrder* resident_order(int heads_per_xcd, int T) {
   struct Key {
     int dev, heads, T;
     bool operator<(const Key& o) const { return std::tie(dev, heads, T) < std::tie(o.dev, o.heads, o.T); }
   };
-  static std::map<Key, const int32_t*> cache;  // launches are serialised by the caller
+  struct Entry {
+    bool usable = false;
+    TileOrder order{};
+  };
+  static std::map<Key, Entry> cache;  // launches are serialised by the caller
   int dev = 0;
   (void)hipGetDevice(&dev);
   const Key key{dev, heads_per_xcd, T};
   auto it = cache.find(key);
-  if (it != cache.end()) return it->second;
+  if (it != cache.end()) return it->second.usable ? &it->second.order : nullptr;
+  Entry& entry = cache[key];
   int cus = 0, per_cu = 0;
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_fwd_f16_resident_kernel<D>, 256,
@@ -662,40 +668,29 @@ static const int32_t* resident_order(int heads_per_xcd, int T) {
   const int n_cu = std::max(cus / 8, 1);
   const int n_qtiles = (T + kFwdBM - 1) / kFwdBM;
   const int n_items = heads_per_xcd * n_qtiles;
-  const int32_t* result = nullptr;
-  if (per_cu > 2 && n_items > 2 * n_cu && n_items <= n_cu * per_cu) {
-    struct Item { int cost, code; };
-    std::vector<Item> items;
-    for (int qt = n_qtiles - 1; qt >= 0; --qt)
-      for (int h = 0; h < heads_per_xcd; ++h)
-        items.push_back({std::min(T - 1, qt * kFwdBM + kFwdBM - 1) / kFwdBN + 1, (h << 16) | qt});
-    std::vector<long> load(n_cu, 0);
-    std::vector<int> used(n_cu, 0);
-    std::vector<int32_t> host((size_t)n_items, 0);
-    std::vector<char> filled((size_t)n_cu * per_cu, 0);
-    for (const Item& item : items) {  // items are in descending cost already
+  if (per_cu <= 2 || n_items <= 2 * n_cu || n_items > n_cu * per_cu || n_items > kMaxResidentTiles)
+    return nullptr;
+  std::vector<long> load(n_cu, 0);
+  std::vector<int> used(n_cu, 0);
+  std::vector<char> filled((size_t)n_items, 0);
+  for (int qt = n_qtiles - 1; qt >= 0; --qt) {  // descending cost
+    const int cost = std::min(T - 1, qt * kFwdBM + kFwdBM - 1) / kFwdBN + 1;
+    for (int h = 0; h < heads_per_xcd; ++h) {
       int best = -1;
       for (int c = 0; c < n_cu; ++c)
-        if (used[c] < per_cu && (size_t)(used[c] * n_cu + c) < host.size() &&
-            (best < 0 || load[c] < load[best]))
-          best = c;
-      if (best < 0) break;
-      host[(size_t)used[best] * n_cu + best] = item.code;
-      filled[(size_t)used[best] * n_cu + best] = 1;
-      load[best] += item.cost;
+        if (used[c] < per_cu && used[c] * n_cu + c < n_items && (best < 0 || load[c] < load[best])) best = c;
+      if (best < 0) return nullptr;
+      const int pos = used[best] * n_cu + best;
+      entry.order.code[pos] = (h << 16) | qt;
+      filled[pos] = 1;
+      load[best] += cost;
       ++used[best];
     }
-    bool complete = true;
-    for (int i = 0; i < n_items; ++i) complete = complete && filled[i];
-    if (complete) {
-      int32_t* dev_table = nullptr;
-      if (hipMalloc(&dev_table, host.size() * sizeof(int32_t)) == hipSuccess &&
-          hipMemcpy(dev_table, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess)
-        result = dev_table;
-    }
   }
-  cache.emplace(key, result);
-  return result;
+  for (int i = 0; i < n_items; ++i)
+    if (!filled[i]) return nullptr;
+  entry.usable = true;
+  return &entry.order;
 }
 
 template <int D>
@@ -718,9 +713,9 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
     // (8x12x1024x64: 32.2 -> 30.0 us; 4x12x2048x64: 49.5 -> 48.2 us; 8x12x1024x32, where
     // four workgroups fit: 22.9 -> 20.6 us).  Smaller and larger launches are as fast or
     // faster on the pipelined kernel.
-    if (const int32_t* order = resident_order<D>(heads_per_xcd, p.T)) {
+    if (const TileOrder* order = resident_order<D>(heads_per_xcd, p.T)) {
       hipLaunchKernelGGL(attn_fwd_f16_resident_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
-                         stream, p, BH, n_qtiles, heads_per_xcd, order);
+                         stream, p, BH, n_qtiles, heads_per_xcd, *order);
       return;
     }
   }
