@@ -548,81 +548,90 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
     request(j + P);
     const uint32_t kb = lds0 + (j % NS) * TILE_B;
     const uint32_t vb = kb + NS * TILE_B;
-    // ---- S^T = K Q^T ----
-    floatx16 c0 = ZERO16, c1 = ZERO16;
+    // A wave skips what lies entirely in its rows' future: the whole tile, or its second
+    // 32-key block (both happen only in a query tile's last two iterations).
+    if (kv0 > qw0 + 31) continue;
+    auto tile_step = [&](auto n_blocks) {
+      constexpr int NB = decltype(n_blocks)::value;  // 32-key blocks of this tile the wave needs
+      // ---- S^T = K Q^T ----
+      floatx16 cb[NB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const uint32_t addr = opaque(kb + koff[ks]);
-      const half8 a0 = *(DEERS_LDS const half8*)(uintptr_t)addr;
-      const half8 a1 = *(DEERS_LDS const half8*)(uintptr_t)(addr + 32 * RB);
-      c0 = mfma_f16(a0, qf[ks], c0);
-      c1 = mfma_f16(a1, qf[ks], c1);
-    }
-    // V fragments of the first half of the PV product, fetched while the vector pipe works
-    constexpr int kVPre = 1;  // 16-key groups of V fetched ahead
-    half8 vfr[kVPre * DB];
+      for (int nb = 0; nb < NB; ++nb) cb[nb] = ZERO16;
 #pragma unroll
-    for (int ms = 0; ms < kVPre; ++ms)
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint32_t addr = opaque(kb + koff[ks]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          cb[nb] = mfma_f16(*(DEERS_LDS const half8*)(uintptr_t)(addr + nb * 32 * RB), qf[ks], cb[nb]);
+      }
+      // V fragments of the first 16 keys, fetched while the vector pipe works
+      half8 vfr[DB];
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const uint32_t ro = 16 * ms * RB;
-        const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
-        const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
-        vfr[ms * DB + db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]));
+        const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]));
+        vfr[db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
-    if (kv0 + kFwdBN - 1 > qw0) {
-      const int dist = qrow - 4 * g - kv0;
+      if (kv0 + 32 * NB - 1 > qw0) {
+        const int dist = qrow - 4 * g - kv0;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int kr = 8 * (r >> 2) + (r & 3);
-        if (kr > dist) c0[r] = -INFINITY;
-        if (kr + 32 > dist) c1[r] = -INFINITY;
-      }
-    }
-    float mx4[4];
+        for (int r = 0; r < 16; ++r) {
+          const int kr = 8 * (r >> 2) + (r & 3);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) mx4[i] = fmaxf(c0[i], c1[i]);
-#pragma unroll
-    for (int r = 4; r < 16; ++r) mx4[r & 3] = fmaxf(fmaxf(mx4[r & 3], c0[r]), c1[r]);
-    float mx = pair_max(fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3])));
-    if (__any((mx - m) * c > kLazyRescale)) {
-      const float m_new = fmaxf(m, mx);
-      const float alpha = fast_exp2((m - m_new) * c);
-      m = m_new;
-      lsum *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-    }
-    const float mc = m * c;
-    uint32_t pw[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      floatx16& cc = (i < 8) ? c0 : c1;
-      const int r = 2 * (i & 7);
-      const float e0 = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
-      const float e1 = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
-      pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)e0, (half_t)e1});
-      lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
-    }
-    // ---- O^T += V^T P^T ----
-#pragma unroll
-    for (int ms = 0; ms < 4; ++ms) {
-      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-      const half8 pb = __builtin_bit_cast(half8, u32x4{pw[4 * ms], pw[4 * ms + 1], pw[4 * ms + 2], pw[4 * ms + 3]});
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        half8 a;
-        if (ms < kVPre) {
-          a = vfr[ms * DB + db];
-        } else {
-          const uint32_t ro = 16 * ms * RB;
-          const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
-          const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
-          a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          for (int nb = 0; nb < NB; ++nb)
+            if (kr + 32 * nb > dist) cb[nb][r] = -INFINITY;
         }
-        oacc[db] = mfma_f16(a, pb, oacc[db]);
       }
-    }
+      float mx4[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx4[i] = NB == 2 ? fmaxf(cb[0][i], cb[NB - 1][i]) : cb[0][i];
+#pragma unroll
+      for (int r = 4; r < 16; ++r)
+        mx4[r & 3] = NB == 2 ? fmaxf(fmaxf(mx4[r & 3], cb[0][r]), cb[NB - 1][r]) : fmaxf(mx4[r & 3], cb[0][r]);
+      const float mx = pair_max(fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3])));
+      if (__any((mx - m) * c > kLazyRescale)) {
+        const float m_new = fmaxf(m, mx);
+        const float alpha = fast_exp2((m - m_new) * c);
+        m = m_new;
+        lsum *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+      }
+      const float mc = m * c;
+      uint32_t pw[8 * NB];
+#pragma unroll
+      for (int i = 0; i < 8 * NB; ++i) {
+        const floatx16& cc = cb[i >> 3];
+        const int r = 2 * (i & 7);
+        const float e0 = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
+        const float e1 = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
+        pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)e0, (half_t)e1});
+        lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
+      }
+      // ---- O^T += V^T P^T ----
+#pragma unroll
+      for (int ms = 0; ms < 2 * NB; ++ms) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const half8 pb = __builtin_bit_cast(half8, u32x4{pw[4 * ms], pw[4 * ms + 1], pw[4 * ms + 2], pw[4 * ms + 3]});
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          half8 a;
+          if (ms == 0) {
+            a = vfr[db];
+          } else {
+            const uint32_t ro = 16 * ms * RB;
+            const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
+            const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
+            a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          }
+          oacc[db] = mfma_f16(a, pb, oacc[db]);
+        }
+      }
+    };
+    if (kv0 + 32 > qw0 + 31)
+      tile_step(std::integral_constant<int, 1>{});
+    else
+      tile_step(std::integral_constant<int, 2>{});
     DEERS_TRACE_POINT(2 + j);
   }
   lsum = pair_sum(lsum);
