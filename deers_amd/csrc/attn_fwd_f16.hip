@@ -5,9 +5,9 @@
 // materialises the [T,T] score tensor.
 //
 // Two kernels share this decomposition: the software-pipelined one described below
-// (two workgroups per CU) and, for D <= 64 launches whose tiles number more than two per
-// CU but no more than fit at once, a plain one at three or four workgroups per CU with every workgroup resident
-// from the start (attn_fwd_f16_resident_kernel, further down).
+// (two workgroups per CU) and, for D <= 64 launches with more than two tiles per CU, a
+// plain one at three or four workgroups per CU (attn_fwd_f16_resident_kernel, further
+// down), whose workgroups are all resident from the start when they fit.
 //
 // Work decomposition
 //   grid  = one workgroup per (head, 128-row query tile), dealt to the XCDs so a
@@ -470,11 +470,18 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  // every workgroup is resident at once: position -> tile chosen for even CU totals
-  const int code = order.code[blockIdx.x >> 3];
-  const int bh = (code >> 16) * 8 + (blockIdx.x & 7);
-  const int qtile = code & 0xffff;
-  if (bh >= BH) return;
+  int bh, qtile;
+  if (order.code[0] >= 0) {
+    // every workgroup is resident at once: position -> tile chosen for even CU totals
+    const int code = order.code[blockIdx.x >> 3];
+    bh = (code >> 16) * 8 + (blockIdx.x & 7);
+    qtile = code & 0xffff;
+    if (bh >= BH) return;
+  } else {  // no table: each XCD's list longest first, handed out by the dispatcher
+    int rank;
+    if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
+    qtile = n_qtiles - 1 - rank;
+  }
   [[maybe_unused]] const int trace_row = blockIdx.x;
   DEERS_TRACE_POINT(0);
   const int b = bh / p.H, h = bh % p.H;
@@ -650,17 +657,19 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
 // lands on CU p % cus_per_xcd when the dispatcher fills an empty chip, so positions p,
 // p + cus, p + 2 cus share a CU and its issue ports: tiles are dealt longest first to the
 // CU with the smallest total that still has a free slot.  Returns nullptr when the tiles
-// do not all fit (then the dispatcher's own longest-first hand-out is the better order)
-// or fit the pipelined kernel's two workgroups per CU as well.  Built at the first launch
-// of a geometry and kept on the host for the life of the process; no device memory.
+// do not all fit (then the dispatcher's own longest-first hand-out is the better order).
+// *use_resident_kernel tells whether the launch is large enough for the plain kernel at
+// all.  Built at the first launch of a geometry and kept on the host for the life of the
+// process; no device memory.
 template <int D>
-static const TileOrder* resident_order(int heads_per_xcd, int T) {
+static const TileOrder* resident_order(int heads_per_xcd, int T, bool* use_resident_kernel) {
   struct Key {
     int dev, heads, T;
     bool operator<(const Key& o) const { return std::tie(dev, heads, T) < std::tie(o.dev, o.heads, o.T); }
   };
   struct Entry {
-    bool usable = false;
+    bool usable = false;    // the table is filled in
+    bool resident = false;  // the launch is large enough for the plain kernel
     TileOrder order{};
   };
   static std::map<Key, Entry> cache;  // launches are serialised by the caller
@@ -668,8 +677,12 @@ static const TileOrder* resident_order(int heads_per_xcd, int T) {
   (void)hipGetDevice(&dev);
   const Key key{dev, heads_per_xcd, T};
   auto it = cache.find(key);
-  if (it != cache.end()) return it->second.usable ? &it->second.order : nullptr;
+  if (it != cache.end()) {
+    *use_resident_kernel = it->second.resident;
+    return it->second.usable ? &it->second.order : nullptr;
+  }
   Entry& entry = cache[key];
+  *use_resident_kernel = false;
   int cus = 0, per_cu = 0;
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_fwd_f16_resident_kernel<D>, 256,
@@ -677,8 +690,10 @@ static const TileOrder* resident_order(int heads_per_xcd, int T) {
   const int n_cu = std::max(cus / 8, 1);
   const int n_qtiles = (T + kFwdBM - 1) / kFwdBM;
   const int n_items = heads_per_xcd * n_qtiles;
-  if (per_cu <= 2 || n_items <= 2 * n_cu || n_items > n_cu * per_cu || n_items > kMaxResidentTiles)
-    return nullptr;
+  // launches that fit the pipelined kernel's two workgroups per CU are faster there
+  entry.resident = per_cu > 2 && n_items > 2 * n_cu;
+  *use_resident_kernel = entry.resident;
+  if (!entry.resident || n_items > n_cu * per_cu || n_items > kMaxResidentTiles) return nullptr;
   std::vector<long> load(n_cu, 0);
   std::vector<int> used(n_cu, 0);
   std::vector<char> filled((size_t)n_items, 0);
@@ -716,13 +731,21 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
   }
   LaunchScope scope("attn_fwd_f16", stream);
   if constexpr (D <= 64) {
-    // More tiles than the pipelined kernel holds at once (two workgroups per CU) but no
-    // more than the three-per-CU kernel does: every workgroup is resident from the start,
-    // placed for even CU totals, and nothing is left to a tail of late, short workgroups
-    // (8x12x1024x64: 32.2 -> 30.0 us; 4x12x2048x64: 49.5 -> 48.2 us; 8x12x1024x32, where
-    // four workgroups fit: 22.9 -> 20.6 us).  Smaller and larger launches are as fast or
-    // faster on the pipelined kernel.
-    if (const TileOrder* order = resident_order<D>(heads_per_xcd, p.T)) {
+    // More tiles than the pipelined kernel holds at once (two workgroups per CU): the plain
+    // kernel at three or four workgroups per CU.  While they all fit, every workgroup is
+    // resident from the start, placed for even CU totals, and nothing is left to a tail of
+    // late, short workgroups (8x12x1024x64: 32.2 -> 27.4 us; 8x12x1024x32: 22.9 -> 20.8 us);
+    // beyond that the dispatcher hands out each XCD's list longest first (32x12x1024x64:
+    // 114.4 -> 95.1 us; 4x12x4096x64: 171 -> 159 us).  Smaller launches are faster on the
+    // pipelined kernel (2x12x1024x64: 20.1 against 21.3 us).
+    bool use_resident = false;
+    const TileOrder* table = resident_order<D>(heads_per_xcd, p.T, &use_resident);
+    static const TileOrder kNoTable = [] {
+      TileOrder t{};
+      t.code[0] = -1;
+      return t;
+    }();
+    if (const TileOrder* order = use_resident ? (table ? table : &kNoTable) : nullptr) {
       hipLaunchKernelGGL(attn_fwd_f16_resident_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
                          stream, p, BH, n_qtiles, heads_per_xcd, *order);
       return;
