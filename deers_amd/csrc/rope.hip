@@ -66,7 +66,74 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   }
 }
 
+// One generation step's handling of the new token's projections, in one launch: q and k
+// rotated at the step's position, q to a compact [B,H,D] tensor, k and the unrotated v to
+// row `pos` of their caches.  Inputs are [B,H,D] views by strides {b,h} (thirds of a fused
+// [B,3C] projection row); caches [B,H,cap,D] by strides {b,h,t}.
+struct DecodeQkvParams {
+  const void* q; const void* k; const void* v;
+  const void* cos; const void* sin;  // the position's rows: D/2 elements each
+  void* q_out; void* k_cache; void* v_cache;
+  int64_t in_b, in_h;
+  int64_t c_b, c_h, c_t;
+  int64_t pos;
+  int B, H, D;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void decode_qkv_kernel(DecodeQkvParams p) {
+  typedef typename Vec16<T>::type V;
+  constexpr int N = Vec16<T>::N;
+  const int half_chunks = p.D / 2 / N;
+  const int per_tensor = p.B * p.H * half_chunks;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= 3 * per_tensor) return;
+  const int which = i / per_tensor;  // 0 q, 1 k, 2 v
+  int r = i - which * per_tensor;
+  const int c = r % half_chunks; r /= half_chunks;
+  const int h = r % p.H;
+  const int b = r / p.H;
+  const T* src = (const T*)(which == 0 ? p.q : which == 1 ? p.k : p.v) + b * p.in_b + h * p.in_h + c * N;
+  T* dst = which == 0 ? (T*)p.q_out + ((int64_t)b * p.H + h) * p.D + c * N
+                      : (T*)(which == 1 ? p.k_cache : p.v_cache) + b * p.c_b + h * p.c_h + p.pos * p.c_t + c * N;
+  const V a1 = *(const V*)src, a2 = *(const V*)(src + p.D / 2);
+  if (which == 2) {
+    *(V*)dst = a1;
+    *(V*)(dst + p.D / 2) = a2;
+    return;
+  }
+  const V cs = *(const V*)((const T*)p.cos + c * N);
+  const V sn = *(const V*)((const T*)p.sin + c * N);
+  V o1, o2;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float x1 = (float)a1[e], x2 = (float)a2[e], co = (float)cs[e], si = (float)sn[e];
+    o1[e] = (T)(x1 * co + x2 * si);
+    o2[e] = (T)(x2 * co - x1 * si);
+  }
+  *(V*)dst = o1;
+  *(V*)(dst + p.D / 2) = o2;
+}
+
 }  // namespace
+
+void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* v,
+                       const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
+                       void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
+                       int H, int D, hipStream_t stream) {
+  DecodeQkvParams p{};
+  p.q = q; p.k = k; p.v = v; p.cos = cos_row; p.sin = sin_row;
+  p.q_out = q_out; p.k_cache = k_cache; p.v_cache = v_cache;
+  p.in_b = in_strides[0]; p.in_h = in_strides[1];
+  p.c_b = cache_strides[0]; p.c_h = cache_strides[1]; p.c_t = cache_strides[2];
+  p.pos = pos; p.B = B; p.H = H; p.D = D;
+  const int n16 = dtype_f16 ? 8 : 4;
+  const int total = 3 * B * H * (D / 2 / n16);
+  LaunchScope scope("decode_qkv", stream);
+  if (dtype_f16)
+    hipLaunchKernelGGL((decode_qkv_kernel<half_t>), dim3((total + 255) / 256), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((decode_qkv_kernel<float>), dim3((total + 255) / 256), dim3(256), 0, stream, p);
+}
 
 // x: logical [B,T,H,D] with element strides xs = {b,t,h} (D stride 1); y: [B,H,T,D],
 // compact or with element strides {b,h,t} (a row range of a KV cache).

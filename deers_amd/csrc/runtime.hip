@@ -34,6 +34,10 @@ void launch_add(int dtype_f16, const void* a, const void* b, void* out, size_t n
 void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t stream);
 void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
                          const int64_t* strides, int ndim, void* dst, hipStream_t stream);
+void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* v,
+                       const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
+                       void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
+                       int H, int D, hipStream_t stream);
 void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
                  const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
                  int T, int H, int D, hipStream_t stream);
@@ -1216,10 +1220,10 @@ int deers_rocm_matmul_tune(int on) {
   return DEERS_ROCM_OK;
 }
 
-int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
-                      const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
-                      int64_t batch, int64_t m, int64_t n, int64_t k) {
-  std::lock_guard<std::mutex> lock(g_mu);
+// c = a @ b (accumulate = false) or c += a @ b (true); the caller holds g_mu
+static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+                         const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
+                         int64_t batch, int64_t m, int64_t n, int64_t k, bool accumulate) {
   NEED_INIT();
   if (int rc = check_dtype(dtype)) return rc;
   if (batch < 0 || m < 0 || n < 0 || k < 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX ||
@@ -1228,6 +1232,7 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
   if (batch == 0 || m == 0 || n == 0) return DEERS_ROCM_OK;
   if (!a || !b || !c) return fail(DEERS_ROCM_ERR_ARG, "matmul: null pointer");
   if (k == 0) {  // empty sum
+    if (accumulate) return DEERS_ROCM_OK;
     deers::launch_fill(dtype == DEERS_ROCM_F16, c, (size_t)(batch * m * n), 0.f, g_rt.stream);
     HIP_TRY(hipGetLastError());
     return DEERS_ROCM_OK;
@@ -1258,7 +1263,7 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
   // row-major [rows x cols] matrix with unit column stride is, read column-major, its
   // own transpose with leading dimension = row stride.
   const rocblas_datatype ty = dtype == DEERS_ROCM_F16 ? rocblas_datatype_f16_r : rocblas_datatype_f32_r;
-  const float alpha = 1.f, beta = 0.f;
+  const float alpha = 1.f, beta = accumulate ? 1.f : 0.f;
   const rocblas_operation op_b = b_t ? rocblas_operation_transpose : rocblas_operation_none;
   const rocblas_operation op_a = a_t ? rocblas_operation_transpose : rocblas_operation_none;
   auto run = [&](int solution) {
@@ -1274,7 +1279,7 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
     auto hit = g_rt.gemm_choice.find(key);
     if (hit != g_rt.gemm_choice.end()) {
       solution = hit->second;
-    } else {
+    } else if (!accumulate) {  // the trial runs would add into c again and again
       // Times the default and every listed kernel on the caller's own operands (the
       // output is overwritten by the real call below): one warm-up and one timed run
       // each, a second timed run for those within 20 % of the best so far.
@@ -1333,6 +1338,20 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
                 rocblas_status_to_string(st));
   return DEERS_ROCM_OK;
 }
+
+int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+                      const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
+                      int64_t batch, int64_t m, int64_t n, int64_t k) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, batch, m, n, k, false);
+}
+
+int deers_rocm_matmul_acc(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+                          const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
+                          int64_t batch, int64_t m, int64_t n, int64_t k) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, batch, m, n, k, true);
+}
 #pragma clang diagnostic pop
 
 // ---- rotary embedding fused with the head split / merge ----
@@ -1387,6 +1406,35 @@ int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides, cons
   }
   deers::launch_rope(dtype == DEERS_ROCM_F16, false, x, st, cos, sin, y, y_strides, (int)B, (int)T,
                      (int)H, (int)D, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_decode_qkv(int dtype, const void* q, const void* k, const void* v,
+                          const int64_t* in_strides, const void* cos_row, const void* sin_row,
+                          void* q_out, void* k_cache, void* v_cache, const int64_t* cache_strides,
+                          int64_t pos, int64_t capacity, int64_t B, int64_t H, int64_t D) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (D != 32 && D != 64 && D != 128) return fail(DEERS_ROCM_ERR_ARG, "decode_qkv: head width %lld not in {32, 64, 128}", (long long)D);
+  if (B < 0 || H < 0 || B * H > (int64_t)1 << 24) return fail(DEERS_ROCM_ERR_ARG, "decode_qkv: bad batch or head count");
+  if (pos < 0 || pos >= capacity) return fail(DEERS_ROCM_ERR_ARG, "decode_qkv: position %lld outside the cache capacity %lld", (long long)pos, (long long)capacity);
+  if (B == 0 || H == 0) return DEERS_ROCM_OK;
+  if (!q || !k || !v || !in_strides || !cos_row || !sin_row || !q_out || !k_cache || !v_cache || !cache_strides)
+    return fail(DEERS_ROCM_ERR_ARG, "decode_qkv: null pointer");
+  const int64_t per16 = dtype == DEERS_ROCM_F16 ? 8 : 4;
+  for (int d = 0; d < 2; ++d)
+    if (in_strides[d] < 0 || in_strides[d] % per16)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "decode_qkv: input strides must be non-negative multiples of 16 bytes");
+  for (int d = 0; d < 3; ++d)
+    if (cache_strides[d] < 0 || cache_strides[d] % per16)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "decode_qkv: cache strides must be non-negative multiples of 16 bytes");
+  const void* ptrs[8] = {q, k, v, cos_row, sin_row, q_out, k_cache, v_cache};
+  for (const void* ptr : ptrs)
+    if ((uintptr_t)ptr & 15) return fail(DEERS_ROCM_ERR_LAYOUT, "decode_qkv: pointers must be 16-byte aligned");
+  deers::launch_decode_qkv(dtype == DEERS_ROCM_F16, q, k, v, in_strides, cos_row, sin_row, q_out, k_cache,
+                           v_cache, cache_strides, pos, (int)B, (int)H, (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -36,6 +36,14 @@ Tensor MLP::forward(const Tensor& x) const {
   return y.matmul(down_).reshape({B, T, C});
 }
 
+void MLP::forward_add_into(const Tensor& x, const Tensor& residual) const {
+  NoGradGuard no_grad;
+  if (x.layout().ndim() != 3) throw std::logic_error("MLP expects input shape [B, T, C]");
+  const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
+  const Tensor y = relu_sq(x.reshape({B * T, C}).matmul(up_));  // [B*T, H]
+  matmul_add_into(y, down_, residual.reshape({B * T, C}));
+}
+
 Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
     : attn_(std::move(attn)), mlp_(std::move(mlp)), eps_(eps) {}
 
@@ -46,8 +54,12 @@ Tensor Block::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) con
 
 Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const {
   NoGradGuard no_grad;
-  const Tensor h = x_t.add(attn_.decode_step(rms_norm(x_t, eps_), cache, cos, sin));
-  return h.add(mlp_.forward(rms_norm(h, eps_)));
+  // the residual stream is updated in place: both additions ride on the last product of
+  // their branch (x_t's storage is overwritten; inference only)
+  const Tensor h = x_t.compact();
+  attn_.decode_step(rms_norm(h, eps_), cache, cos, sin, &h);
+  mlp_.forward_add_into(rms_norm(h, eps_), h);
+  return h;
 }
 
 std::vector<Tensor> Block::parameters() const {

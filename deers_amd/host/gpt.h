@@ -28,6 +28,9 @@ class MLP {
  public:
   MLP(Tensor up_proj, Tensor down_proj);
   Tensor forward(const Tensor& x) const;  // [B,T,C] -> [B,T,C]
+  // residual ([B,T,C], compact) += forward(x), the addition riding on the down projection
+  // (inference: the residual's storage is updated in place)
+  void forward_add_into(const Tensor& x, const Tensor& residual) const;
   std::vector<Tensor> parameters() const { return {up_, down_}; }
 
  private:
@@ -40,6 +43,7 @@ class Block {
   Block(CausalSelfAttention attn, MLP mlp, double eps);
   Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
   // One generated position: x_t [B,1,C] at position cache.len (inference, no autograd).
+  // x_t's storage is overwritten with the result when x_t is compact.
   Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
   std::vector<Tensor> parameters() const;  // attention, then MLP
 

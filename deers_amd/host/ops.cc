@@ -509,7 +509,7 @@ KvCache KvCache::create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType
 }
 
 Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos,
-                                        const Tensor& sin) const {
+                                        const Tensor& sin, const Tensor* residual) const {
   NoGradGuard no_grad;
   if (x_t.layout().ndim() != 3 || x_t.shape()[1] != 1)
     throw std::logic_error("decode_step expects input shape [B, 1, C]");
@@ -537,21 +537,39 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   const Tensor cc = cos.compact(), sc = sin.compact();
   const char* cos_t = (const char*)cc.data() + pos * (D / 2) * el;
   const char* sin_t = (const char*)sc.data() + pos * (D / 2) * el;
-  const int64_t x_strides[4] = {3 * C, 3 * C, D, 1};                 // [B,1,H,D] inside a [B, 3C] row
-  const int64_t cache_strides[4] = {H * cap * D, cap * D, D, 1};     // [B,H,1,D] at one cache row
+  // rotate q and k at this position, append k and v to the caches: one launch
+  const int64_t in_strides[2] = {3 * C, D};                          // [B,H,D] inside a [B, 3C] row
+  const int64_t kv_strides[3] = {H * cap * D, cap * D, D};
   Tensor qh = empty({B, H, D}, x_t.dtype(), true);
-  check(deers_rocm_rope_fwd(dt, q_data, x_strides, cos_t, sin_t, qh.data(), nullptr, B, 1, H, D));
-  check(deers_rocm_rope_fwd(dt, k_data, x_strides, cos_t, sin_t,
-                            (char*)cache.k.data() + pos * D * el, cache_strides, B, 1, H, D));
-  const int64_t shape[3] = {B, H, D}, v_src[3] = {3 * C, D, 1}, v_dst[3] = {H * cap * D, cap * D, 1};
-  check(deers_rocm_copy_view(dt, v_data, v_src, (char*)cache.v.data() + pos * D * el, v_dst, shape, 3));
+  check(deers_rocm_decode_qkv(dt, q_data, k_data, v_data, in_strides, cos_t, sin_t, qh.data(),
+                              cache.k.data(), cache.v.data(), kv_strides, pos, cap, B, H, D));
   cache.len = pos + 1;
   Tensor o = empty({B, H * D}, x_t.dtype(), true);
-  const int64_t kv_strides[3] = {H * cap * D, cap * D, D};
   const double scale = 1.0 / std::sqrt((double)D);
   check(deers_rocm_attn_decode(dt, qh.data(), cache.k.data(), cache.v.data(), kv_strides, o.data(), B,
                                H, cache.len, D, (float)scale));
+  if (residual) {
+    matmul_add_into(o, wo_, residual->reshape({B, C}));
+    return *residual;
+  }
   return o.matmul(wo_).reshape({B, 1, C});
+}
+
+void matmul_add_into(const Tensor& a, const Tensor& b, const Tensor& acc) {
+  NoGradGuard no_grad;
+  Tensor ac = a, bc = b;
+  int64_t ars, acs, abs_, brs, bcs, bbs;
+  if (!gemm_view(ac, &ars, &acs, &abs_)) { ac = ac.detach().compact(); gemm_view(ac, &ars, &acs, &abs_); }
+  if (!gemm_view(bc, &brs, &bcs, &bbs)) { bc = bc.detach().compact(); gemm_view(bc, &brs, &bcs, &bbs); }
+  const size_t nd = ac.layout().ndim();
+  const int64_t m = ac.shape()[nd - 2], k = ac.shape()[nd - 1], n = bc.shape()[nd - 1];
+  int64_t batch = 1;
+  for (size_t d = 0; d + 2 < nd; ++d) batch *= ac.shape()[d];
+  if (!acc.is_compact() || (int64_t)acc.layout().size() != batch * m * n || acc.dtype() != ac.dtype())
+    throw std::logic_error("matmul_add_into: the accumulator must be a compact tensor of the product's shape and type");
+  if (backed(ac))
+    check(deers_rocm_matmul_acc((int)ac.dtype(), ac.data(), ars, acs, abs_, bc.data(), brs, bcs, bbs,
+                                const_cast<void*>(acc.data()), batch, m, n, k));
 }
 
 Tensor attention_decode(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache) {

@@ -230,6 +230,10 @@ Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
 // Keys (rotated) and values of the tokens seen so far, [B,H,L_cap,D]; rows [0,len)
 // are valid.  The reference keeps no cache and re-runs the whole window per generated
 // token (examples/tinystories_train.rs:250-276).
+// acc += a @ b in one launch; acc compact, of the product's shape and type.  Inference
+// helper: nothing is recorded for autograd, the accumulator's storage is updated in place.
+void matmul_add_into(const Tensor& a, const Tensor& b, const Tensor& acc);
+
 struct KvCache {
   Tensor k, v;
   // [C, 3C] = (Wq | Wk | Wv), packed by the first decode_step that uses this cache so a
@@ -249,7 +253,10 @@ class CausalSelfAttention {
   // cache.len; its rotated key and its value are appended to the cache and the query
   // attends to all cache.len+1 positions through the decode kernel.  Returns [B,1,C],
   // equal to row cache.len of forward() on the whole prefix.
-  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
+  // With `residual` ([B,1,C], compact) the output projection is added into it in place
+  // (one launch for `residual + attn(x_t)`) and it is returned.
+  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,
+                     const Tensor* residual = nullptr) const;
   std::vector<Tensor> parameters() const { return {wq_, wk_, wv_, wo_}; }
 
  private:

@@ -370,6 +370,25 @@ def matmul_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
         i64(k)))
 
 
+def matmul_acc_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
+    """deers_rocm_matmul_acc: c[batch,m,n] += a @ b; strides are (row, col, batch) in elements."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_matmul_acc(
+        ctypes.c_int(dtype_code(dtype)), a, i64(a_strides[0]), i64(a_strides[1]), i64(a_strides[2]),
+        b, i64(b_strides[0]), i64(b_strides[1]), i64(b_strides[2]), c, i64(batch), i64(m), i64(n),
+        i64(k)))
+
+
+def decode_qkv_raw(dtype, q, k, v, in_strides, cos_row, sin_row, q_out, k_cache, v_cache, cache_strides,
+                   pos, capacity, B, H, D):
+    """deers_rocm_decode_qkv: rotate q, k at `pos`; q -> q_out [B,H,D]; k, v -> row pos of the caches."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_decode_qkv(
+        ctypes.c_int(dtype_code(dtype)), q, k, v, (i64 * 2)(*[int(x) for x in in_strides]), cos_row,
+        sin_row, q_out, k_cache, v_cache, (i64 * 3)(*[int(x) for x in cache_strides]), i64(pos),
+        i64(capacity), i64(B), i64(H), i64(D)))
+
+
 def rope_fwd_raw(dtype, x, cos, sin, y, B, T, H, D, x_strides=None, y_strides=None):
     """deers_rocm_rope_fwd: x logical [B,T,H,D] -> y [B,H,T,D] (compact unless y_strides)."""
     _check(load().deers_rocm_rope_fwd(

@@ -400,6 +400,16 @@ int deers_rocm_matmul(int dtype,
                       const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
                       const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
                       void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
+/* c += a @ b, same operand rules; c holds the other addend on entry.  One launch for
+ * the block's residual connections `x + attn(..)` and `x + mlp(..)`
+ * (src/models/gpt.rs:237-239: a matmul followed by a binary add in the reference) and
+ * for `GradientStore::accumulate` of a matmul's gradient (src/backprop.rs:101-112).  The
+ * sum is formed in f32 inside the product's accumulator and rounded once, where the
+ * reference rounds the product and then the sum (f16: at most one ulp apart). */
+int deers_rocm_matmul_acc(int dtype,
+                          const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
+                          const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
+                          void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
 /* Off by default.  When on, the first matmul of each distinct problem (sizes, strides,
  * transposes, batch) times every kernel the BLAS offers for it on the caller's operands
  * and later calls of that problem use the fastest; the library's own pick is a heuristic
@@ -424,6 +434,19 @@ int deers_rocm_matmul_tune(int on);
 int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides,
                         const void* cos, const void* sin, void* y, const int64_t* y_strides,
                         int64_t B, int64_t T, int64_t H, int64_t D);
+
+/* One generation step's handling of the new token's q, k, v in one launch: q and k rotated
+ * at the step's position (cos_row / sin_row: the D/2 table entries of that position), q to
+ * compact q_out [B,H,D], the rotated k and the unrotated v to row `pos` of their caches.
+ * q, k, v: [B,H,D] by element strides in_strides = {b, h} (D stride 1; e.g. the thirds of a
+ * fused [B, 3C] projection row); caches [B,H,capacity,D] by cache_strides = {b, h, t}.
+ * Replaces two deers_rocm_rope_fwd and one deers_rocm_copy_view per block and step.  The
+ * reference has no KV cache (examples/tinystories_train.rs:250-276 re-runs the window);
+ * the rotation is that of src/models/gpt.rs:49-73. */
+int deers_rocm_decode_qkv(int dtype, const void* q, const void* k, const void* v,
+                          const int64_t* in_strides, const void* cos_row, const void* sin_row,
+                          void* q_out, void* k_cache, void* v_cache, const int64_t* cache_strides,
+                          int64_t pos, int64_t capacity, int64_t B, int64_t H, int64_t D);
 
 /* Backward of the above (Permute::backward then the element-wise backward bodies,
  * src/ops.rs:687-727, 130-260): dx (compact [B,T,H,D]) from dy logical [B,H,T,D]

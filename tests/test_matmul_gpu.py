@@ -108,3 +108,27 @@ def test_matmul_with_kernel_tuning_gives_the_same_product(dtype, tol):
                 assert np.max(np.abs(got.astype(np.float64) - want)) <= tol
     finally:
         rocm.matmul_tune(False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float16, 2e-2), (np.float32, 1e-4)])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 32, 768, 768), (2, 7, 33, 64), (1, 5, 3, 1)])
+def test_matmul_acc_adds_the_product_into_c(dtype, tol, batch, m, n, k):
+    """deers_rocm_matmul_acc: c += a @ b (the residual add of src/models/gpt.rs:237-239 riding on
+    the projection), against the oracle's product plus the addend."""
+    rng = np.random.default_rng(batch * 1000 + m)
+    a = rng.standard_normal((batch, m, k)).astype(dtype)
+    b = rng.standard_normal((batch, k, n)).astype(dtype)
+    c0 = rng.standard_normal((batch, m, n)).astype(dtype)
+    da, db, dc = (rocm.DeviceBuffer.from_numpy(x) for x in (a, b, c0))
+    rocm.matmul_acc_raw(dtype, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dc.ptr, batch, m, n, k)
+    want = oracle.matmul(a.astype(np.float32), b.astype(np.float32)) + c0.astype(np.float32)
+    scale = max(1.0, float(np.abs(want).max()))
+    assert np.abs(dc.numpy().astype(np.float32) - want).max() <= tol * scale
+    # twice more: the accumulator keeps growing by the same product
+    rocm.matmul_acc_raw(dtype, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dc.ptr, batch, m, n, k)
+    want2 = want + oracle.matmul(a.astype(np.float32), b.astype(np.float32))
+    assert np.abs(dc.numpy().astype(np.float32) - want2).max() <= 2 * tol * max(1.0, float(np.abs(want2).max()))
+    # k = 0 leaves c alone
+    rocm.matmul_acc_raw(dtype, da.ptr, (1, 1, 1), db.ptr, (n, 1, 1), dc.ptr, batch, m, n, 0)
+    assert np.abs(dc.numpy().astype(np.float32) - want2).max() <= 2 * tol * max(1.0, float(np.abs(want2).max()))

@@ -137,3 +137,52 @@ def test_rope_appends_rotated_keys_into_a_cache_and_copy_view_scatters_values():
     assert np.array_equal(gotv[:, :, :pos], cache0[:, :, :pos])
     with pytest.raises(rocm.RocmError):
         rocm.copy_view_raw(np.float16, dv.ptr, (1,) * 7, dvc.ptr, (1,) * 7, (1,) * 7)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("B,H,D", [(2, 3, 64), (32, 12, 64), (1, 5, 32), (3, 2, 128)])
+def test_decode_qkv_is_two_ropes_and_a_copy_in_one_launch(dtype, B, H, D):
+    """deers_rocm_decode_qkv against the separate entry points it replaces (same bits): q and k
+    rotated at `pos` from the thirds of a fused [B, 3C] projection row, k and v written to row
+    `pos` of [B,H,cap,D] caches, everything else untouched."""
+    import ctypes
+    cap, pos, C = 11, 7, H * D
+    el = np.dtype(dtype).itemsize
+    _, _, cos, sin = _inputs(1, cap, 1, D, dtype, 31)           # tables [cap, D/2]
+    qkv = synth.normal((B, 3 * C), synth.tensor_seed(31, "decode", "qkv"), 1.0).astype(dtype)
+    kc0 = synth.normal((B, H, cap, D), synth.tensor_seed(31, "decode", "kc"), 1.0).astype(dtype)
+    vc0 = synth.normal((B, H, cap, D), synth.tensor_seed(31, "decode", "vc"), 1.0).astype(dtype)
+    dqkv, dc, ds = (rocm.DeviceBuffer.from_numpy(a) for a in (qkv, cos, sin))
+    at = lambda buf, elems: ctypes.c_void_p(buf.ptr.value + elems * el)
+    cos_row, sin_row = at(dc, pos * (D // 2)), at(ds, pos * (D // 2))
+    kv_strides = (H * cap * D, cap * D, D)
+    # fused
+    q1 = rocm.DeviceBuffer((B, H, D), dtype)
+    k1, v1 = rocm.DeviceBuffer.from_numpy(kc0), rocm.DeviceBuffer.from_numpy(vc0)
+    rocm.decode_qkv_raw(dtype, at(dqkv, 0), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                        q1.ptr, k1.ptr, v1.ptr, kv_strides, pos, cap, B, H, D)
+    # separate
+    q2 = rocm.DeviceBuffer((B, H, D), dtype)
+    k2, v2 = rocm.DeviceBuffer.from_numpy(kc0), rocm.DeviceBuffer.from_numpy(vc0)
+    xs = (3 * C, 3 * C, D, 1)
+    rocm.rope_fwd_raw(dtype, at(dqkv, 0), cos_row, sin_row, q2.ptr, B, 1, H, D, x_strides=xs)
+    rocm.rope_fwd_raw(dtype, at(dqkv, C), cos_row, sin_row, at(k2, pos * D), B, 1, H, D, x_strides=xs,
+                      y_strides=(H * cap * D, cap * D, D, 1))
+    rocm.copy_view_raw(dtype, at(dqkv, 2 * C), (3 * C, D, 1), at(v2, pos * D), (H * cap * D, cap * D, 1),
+                       (B, H, D))
+    assert np.array_equal(q1.numpy(), q2.numpy())
+    assert np.array_equal(k1.numpy(), k2.numpy())
+    assert np.array_equal(v1.numpy(), v2.numpy())
+    # and against the oracle's rotation of the same rows
+    want_q = oracle.rope_apply(qkv[:, :C].reshape(B, 1, H, D), cos[pos:pos + 1], sin[pos:pos + 1], dtype=dtype)
+    tol = 5e-3 if dtype == np.float16 else 1e-5
+    assert np.abs(q1.numpy().astype(np.float32) - want_q.reshape(B, H, D).astype(np.float32)).max() <= tol
+    assert np.array_equal(v1.numpy()[:, :, pos], qkv[:, 2 * C:].reshape(B, H, D))
+    assert np.array_equal(k1.numpy()[:, :, :pos], kc0[:, :, :pos]) and np.array_equal(k1.numpy()[:, :, pos + 1:], kc0[:, :, pos + 1:])
+    with pytest.raises(rocm.RocmError):
+        rocm.decode_qkv_raw(dtype, at(dqkv, 0), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                            q1.ptr, k1.ptr, v1.ptr, kv_strides, cap, cap, B, H, D)   # position past the cache
+    with pytest.raises(rocm.RocmError):
+        rocm.decode_qkv_raw(dtype, at(dqkv, 1), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                            q1.ptr, k1.ptr, v1.ptr, kv_strides, pos, cap, B, H, D)   # misaligned q
