@@ -12,6 +12,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <unordered_map>
 #include <mutex>
@@ -34,6 +35,13 @@ void launch_add(int dtype_f16, const void* a, const void* b, void* out, size_t n
 void launch_neg(int dtype_f16, const void* a, void* out, size_t n, hipStream_t stream);
 void launch_copy_strided(int dtype_f16, const void* src, const int64_t* shape,
                          const int64_t* strides, int ndim, void* dst, hipStream_t stream);
+bool skinny_gemm_takes(int64_t m, int64_t n, int64_t k, int64_t ldx, int64_t ldw, int64_t ldy,
+                       const void* x, const void* w, const void* y);
+int skinny_gemm_splits(int64_t n, int64_t k);
+size_t skinny_gemm_workspace_bytes(int64_t n, int splits);
+void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
+                            int m, int n, int k, bool accumulate, int splits, float* partial,
+                            int* counters, hipStream_t stream);
 void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* v,
                        const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
                        void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
@@ -102,6 +110,7 @@ struct Runtime {
   // next synchronising call after one of them has been launched
   int* index_flag = nullptr;
   bool index_flag_armed = false;
+  int* skinny_counters = nullptr;  // arrival counters of the few-rows GEMM's K splits (all zero between launches)
   // Block cache behind deers_rocm_alloc / _free.  Every kernel and copy of this library
   // runs on `stream`, in order, so a block handed back by free can be handed out again
   // without waiting for the device: whatever still reads it was enqueued earlier than
@@ -1220,6 +1229,8 @@ int deers_rocm_matmul_tune(int on) {
   return DEERS_ROCM_OK;
 }
 
+constexpr int kSkinnyCounters = 4096;  // column blocks a K-split launch of the few-rows GEMM may have
+
 // c = a @ b (accumulate = false) or c += a @ b (true); the caller holds g_mu
 static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
                          const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
@@ -1253,6 +1264,26 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
                 "matmul: each operand needs a unit row or column stride and non-overlapping "
                 "lines (a %lld,%lld b %lld,%lld); compact the tensor first",
                 (long long)a_rs, (long long)a_cs, (long long)b_rs, (long long)b_cs);
+  // a few rows against a weight matrix (a generation step's projections): one streaming
+  // pass over the weights instead of a library GEMM
+  if (dtype == DEERS_ROCM_F16 && batch == 1 && !a_t && !b_t &&
+      deers::skinny_gemm_takes(m, n, k, lda, ldb, n, a, b, c)) {
+    int splits = deers::skinny_gemm_splits(n, k);
+    void* ws = nullptr;
+    if (splits > 1 && (n + 31) / 32 > kSkinnyCounters) splits = 1;
+    if (splits > 1) {
+      if (int rc = workspace(deers::skinny_gemm_workspace_bytes(n, splits), &ws)) return rc;
+      if (!g_rt.skinny_counters) {  // zero once; the kernel leaves every counter at zero
+        HIP_TRY(hipMalloc(&g_rt.skinny_counters, kSkinnyCounters * sizeof(int)));
+        HIP_TRY(hipMemsetAsync(g_rt.skinny_counters, 0, kSkinnyCounters * sizeof(int), g_rt.stream));
+      }
+    }
+    deers::LaunchScope scope("matmul", g_rt.stream);
+    deers::launch_skinny_gemm_f16(a, lda, b, ldb, c, n, (int)m, (int)n, (int)k, accumulate, splits,
+                                  (float*)ws, g_rt.skinny_counters, g_rt.stream);
+    HIP_TRY(hipGetLastError());
+    return DEERS_ROCM_OK;
+  }
   if (!g_rt.blas) {
     if (rocblas_create_handle(&g_rt.blas) != rocblas_status_success)
       return fail(DEERS_ROCM_ERR_HIP, "rocblas_create_handle failed");

@@ -132,3 +132,39 @@ def test_matmul_acc_adds_the_product_into_c(dtype, tol, batch, m, n, k):
     # k = 0 leaves c alone
     rocm.matmul_acc_raw(dtype, da.ptr, (1, 1, 1), db.ptr, (n, 1, 1), dc.ptr, batch, m, n, 0)
     assert np.abs(dc.numpy().astype(np.float32) - want2).max() <= 2 * tol * max(1.0, float(np.abs(want2).max()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(32, 768, 768), (32, 3072, 768), (32, 768, 3072), (7, 2304, 768),
+                                   (1, 768, 256), (32, 776, 512), (5, 8, 256), (31, 40, 1024)])
+def test_few_rows_against_a_weight_matrix_take_the_streaming_kernel(m, n, k):
+    """f16 products with at most 32 rows, K a multiple of 256 and N a multiple of 8 (a generation
+    step's projections) run on the library's own one-pass kernel instead of the BLAS: same
+    contract (f32 accumulation, one rounding), checked against the oracle, with and without the
+    addend, through a strided x (rows of a wider buffer) as well."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    a = rng.standard_normal((1, m, k)).astype(np.float16)
+    b = (rng.standard_normal((1, k, n)) / np.sqrt(k)).astype(np.float16)
+    want = oracle.matmul(a.astype(np.float32), b.astype(np.float32))
+    got = _run(a, b, np.float16)
+    assert np.abs(got.astype(np.float32) - want).max() <= 4e-3 * max(1.0, float(np.abs(want).max()))
+    # y += x @ W, the addend added in f32 before the single rounding
+    c0 = rng.standard_normal((1, m, n)).astype(np.float16)
+    da, db, dc = (rocm.DeviceBuffer.from_numpy(x) for x in (a, b, c0))
+    rocm.matmul_acc_raw(np.float16, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dc.ptr, 1, m, n, k)
+    want_acc = want + c0.astype(np.float32)
+    assert np.abs(dc.numpy().astype(np.float32) - want_acc).max() <= 4e-3 * max(1.0, float(np.abs(want_acc).max()))
+    assert np.array_equal(dc.numpy(), (want_acc.astype(np.float16))) or \
+        np.abs(dc.numpy().astype(np.float32) - want_acc.astype(np.float16).astype(np.float32)).max() <= 2e-3 * max(1.0, float(np.abs(want_acc).max()))
+    # x as the middle third of a [m, 3k] buffer (row stride 3k)
+    wide = rng.standard_normal((m, 3 * k)).astype(np.float16)
+    dw = rocm.DeviceBuffer.from_numpy(wide)
+    import ctypes
+    dc2 = rocm.DeviceBuffer((1, m, n), np.float16)
+    rocm.matmul_raw(np.float16, ctypes.c_void_p(dw.ptr.value + k * 2), (3 * k, 1, 0), db.ptr, (n, 1, k * n),
+                    dc2.ptr, 1, m, n, k)
+    want2 = oracle.matmul(wide[None, :, k:2 * k].astype(np.float32), b.astype(np.float32))
+    assert np.abs(dc2.numpy().astype(np.float32) - want2).max() <= 4e-3 * max(1.0, float(np.abs(want2).max()))
+    # bit-reproducible
+    got2 = _run(a, b, np.float16)
+    assert np.array_equal(got, got2)
