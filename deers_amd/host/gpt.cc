@@ -62,6 +62,14 @@ Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, 
   return h;
 }
 
+Tensor Block::prefill(const Tensor& x, KvCache& cache, const Tensor& cos, const Tensor& sin) const {
+  NoGradGuard no_grad;
+  const Tensor h = x.compact();
+  attn_.prefill(rms_norm(h, eps_), cache, cos, sin, &h);
+  mlp_.forward_add_into(rms_norm(h, eps_), h);
+  return h;
+}
+
 std::vector<Tensor> Block::parameters() const {
   std::vector<Tensor> p = attn_.parameters();
   for (const Tensor& t : mlp_.parameters()) p.push_back(t);
@@ -163,6 +171,23 @@ Tensor GPT::decode_step(const Tensor& idx_t, std::vector<KvCache>& caches) const
   return x.reshape({B, config_.n_embd}).matmul(lm_head_).reshape({B, 1, config_.vocab_size});
 }
 
+Tensor GPT::prefill(const Tensor& idx, std::vector<KvCache>& caches) const {
+  NoGradGuard no_grad;
+  if (idx.layout().ndim() != 2) throw std::logic_error("prefill expects token ids with shape [B, T]");
+  if ((int64_t)caches.size() != config_.n_layer) throw std::logic_error("prefill: one cache per block");
+  const int64_t B = idx.shape()[0], T = idx.shape()[1], C = config_.n_embd;
+  Tensor x = wte_.forward(idx);  // [B, T, C]
+  for (size_t l = 0; l < blocks_.size(); ++l) x = blocks_[l].prefill(x, caches[l], cos_, sin_);
+  // only the last position's logits are needed: its rows out of the residual stream first
+  Tensor last(std::make_shared<RocmStorage>((size_t)(B * C), x.dtype(), true), Layout({B, C}), false, nullptr);
+  const int64_t shape[2] = {B, C}, src[2] = {T * C, 1}, dst[2] = {C, 1};
+  const size_t el = size_in_bytes(x.dtype());
+  check(deers_rocm_copy_view((int)x.dtype(), (const char*)x.data() + (T - 1) * C * el, src, last.data(), dst,
+                             shape, 2));
+  last = rms_norm(last, config_.rms_norm_eps);
+  return last.matmul(lm_head_).reshape({B, 1, config_.vocab_size});
+}
+
 std::vector<int64_t> GPT::generate_greedy(const std::vector<int64_t>& prompt, int64_t batch,
                                           int64_t n_new) const {
   if (batch < 1 || prompt.empty() || prompt.size() % (size_t)batch)
@@ -170,30 +195,19 @@ std::vector<int64_t> GPT::generate_greedy(const std::vector<int64_t>& prompt, in
   NoGradGuard no_grad;
   const int64_t t0 = (int64_t)prompt.size() / batch, total = t0 + n_new, V = config_.vocab_size;
   std::vector<KvCache> caches = new_caches(batch, total);
-  // the prompt goes up once, position-major, so that every step's ids are one contiguous
-  // [batch] slice; after it each step's ids are the previous step's argmax, picked on the
-  // device: nothing in the loop waits for the host
-  std::vector<int64_t> by_pos((size_t)(t0 * batch));
-  for (int64_t b = 0; b < batch; ++b)
-    for (int64_t t = 0; t < t0; ++t) by_pos[t * batch + b] = prompt[b * t0 + t];
-  const Tensor prompt_dev = Tensor::from_host(by_pos.data(), {t0 * batch}, DType::I64);
+  // the prompt goes through the batched forward once; after it each step's ids are the
+  // previous step's argmax, picked on the device: nothing in the loop waits for the host
   std::vector<Tensor> picked;  // one [batch] id tensor per generated position
-  for (int64_t t = 0; t < total - 1; ++t) {
-    Tensor ids_t;
-    if (t < t0) {
-      // a [batch, 1] tensor of its own (layouts with an offset do not count as compact)
-      auto st = std::make_shared<RocmStorage>((size_t)batch, DType::I64, true);
-      ids_t = Tensor(st, Layout({batch, 1}), false, nullptr);
-      check(deers_rocm_dtod(ids_t.data(), (const char*)prompt_dev.data() + t * batch * 8, (size_t)batch * 8));
-    } else {
-      ids_t = Tensor(picked.back().storage(), Layout({batch, 1}), false, nullptr);
-    }
-    const Tensor logits = decode_step(ids_t, caches);  // [batch, 1, V], compact
-    if (t + 1 < t0) continue;                           // still inside the prompt
+  auto pick = [&](const Tensor& logits) {  // [batch, 1, V], compact
     auto st = std::make_shared<RocmStorage>((size_t)batch, DType::I64, true);
     Tensor next(st, Layout({batch}), false, nullptr);
     check(deers_rocm_argmax_rows((int)logits.dtype(), logits.data(), (int64_t*)next.data(), batch, V));
     picked.push_back(next);
+  };
+  if (n_new > 0) pick(prefill(Tensor::from_host(prompt.data(), {batch, t0}, DType::I64), caches));
+  for (int64_t t = t0; t < total - 1; ++t) {
+    const Tensor ids_t(picked.back().storage(), Layout({batch, 1}), false, nullptr);
+    pick(decode_step(ids_t, caches));
   }
   std::vector<int64_t> out((size_t)(batch * total));
   for (int64_t b = 0; b < batch; ++b)

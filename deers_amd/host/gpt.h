@@ -45,6 +45,9 @@ class Block {
   // One generated position: x_t [B,1,C] at position cache.len (inference, no autograd).
   // x_t's storage is overwritten with the result when x_t is compact.
   Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
+  // The whole prompt x [B,T,C] into an empty cache (inference); x's storage is overwritten
+  // like decode_step's.
+  Tensor prefill(const Tensor& x, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
   std::vector<Tensor> parameters() const;  // attention, then MLP
 
  private:
@@ -82,8 +85,13 @@ class GPT {
   // idx_t I64 [B,1], the token at position caches[0].len -> logits [B,1,V]; equal to row
   // caches[0].len of forward() on the whole prefix.  Inference only.
   Tensor decode_step(const Tensor& idx_t, std::vector<KvCache>& caches) const;
-  // Greedy continuation of a prompt (host-side I64 [B, T0], row-major): feeds the prompt
-  // token by token, then appends n_new argmax tokens.  Returns [B, T0 + n_new] on the host.
+  // The prompt in one pass: idx I64 [B,T0] into empty caches -> logits [B,1,V] of the last
+  // prompt position (row T0-1 of forward()); afterwards caches[l].len == T0 and decode_step
+  // continues from there.  Inference only.
+  Tensor prefill(const Tensor& idx, std::vector<KvCache>& caches) const;
+  // Greedy continuation of a prompt (host-side I64 [B, T0], row-major): the prompt goes
+  // through prefill, then n_new argmax tokens are appended one decode_step at a time.
+  // Returns [B, T0 + n_new] on the host.
   std::vector<int64_t> generate_greedy(const std::vector<int64_t>& prompt, int64_t batch,
                                        int64_t n_new) const;
   const GPTConfig& config() const { return config_; }

@@ -582,11 +582,35 @@ static int run_generate(const std::string& dir) {
   bool threw = false;
   try { model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), caches); } catch (const std::logic_error&) { threw = true; }
   EXPECT(threw);  // the caches are full
-  // greedy continuation of the first T0 = T/2 tokens
   const int64_t t0 = T / 2;
   std::vector<int64_t> prompt((size_t)(B * t0));
   for (int64_t b = 0; b < B; ++b)
     for (int64_t t = 0; t < t0; ++t) prompt[b * t0 + t] = h_ids[b * T + t];
+  // the first T0 = T/2 tokens in one prefill pass, the others step by step from there
+  {
+    std::vector<KvCache> c2 = model.new_caches(B, T);
+    Tensor lp = model.prefill(Tensor::from_host(prompt.data(), {B, t0}, DType::I64), c2);
+    EXPECT((lp.shape() == std::vector<int64_t>{B, 1, V}) && !lp.requires_grad());
+    for (const KvCache& c : c2) EXPECT(c.len == t0);
+    dump(lp, dir + "/logits_prefill.bin");
+    dump(c2.back().k, dir + "/k_cache_prefill.bin");
+    dump(c2.back().v, dir + "/v_cache_prefill.bin");
+    dump(caches.back().k, dir + "/k_cache_steps.bin");
+    dump(caches.back().v, dir + "/v_cache_steps.bin");
+    std::vector<char> rest((size_t)(B * (T - t0) * V) * 2);
+    for (int64_t t = t0; t < T; ++t) {
+      for (int64_t b = 0; b < B; ++b) cur[b] = h_ids[b * T + t];
+      Tensor l = model.decode_step(Tensor::from_host(cur.data(), {B, 1}, DType::I64), c2);
+      l.to_host(one.data());
+      for (int64_t b = 0; b < B; ++b)
+        std::memcpy(rest.data() + ((b * (T - t0) + (t - t0)) * V) * 2, one.data() + (b * V) * 2, (size_t)V * 2);
+    }
+    write_file(dir + "/logits_after_prefill.bin", rest.data(), rest.size());
+    threw = false;
+    try { model.prefill(Tensor::from_host(prompt.data(), {B, t0}, DType::I64), c2); } catch (const std::logic_error&) { threw = true; }
+    EXPECT(threw);  // prefill wants empty caches
+  }
+  // greedy continuation of the same prompt
   std::vector<int64_t> gen = model.generate_greedy(prompt, B, n_new);
   EXPECT((int64_t)gen.size() == B * (t0 + n_new));
   write_file(dir + "/generated.bin", gen.data(), gen.size() * 8);

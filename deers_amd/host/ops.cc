@@ -508,6 +508,64 @@ KvCache KvCache::create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType
   return c;
 }
 
+const Tensor& CausalSelfAttention::packed_qkv(KvCache& cache) const {
+  if (!cache.wqkv.defined()) {
+    const int64_t C = n_head_ * head_dim_;
+    const size_t el = size_in_bytes(wq_.dtype());
+    cache.wqkv = empty({C, 3 * C}, wq_.dtype(), true);
+    const Tensor* w[3] = {&wq_, &wk_, &wv_};
+    for (int i = 0; i < 3; ++i) {
+      const Tensor wc = w[i]->compact();
+      const int64_t wshape[2] = {C, C}, src[2] = {C, 1}, dst[2] = {3 * C, 1};
+      check(deers_rocm_copy_view((int)wq_.dtype(), wc.data(), src, (char*)cache.wqkv.data() + i * C * el, dst,
+                                 wshape, 2));
+    }
+  }
+  return cache.wqkv;
+}
+
+Tensor CausalSelfAttention::prefill(const Tensor& x, KvCache& cache, const Tensor& cos,
+                                    const Tensor& sin, const Tensor* residual) const {
+  NoGradGuard no_grad;
+  if (x.layout().ndim() != 3) throw std::logic_error("prefill expects input shape [B, T, C]");
+  if (cache.len != 0) throw std::logic_error("prefill: the KV cache must be empty");
+  const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2], H = n_head_, D = head_dim_;
+  const int64_t cap = cache.capacity;
+  if (C != H * D) throw std::logic_error("input channel size must match attention width");
+  if (T < 1 || T > cap) throw std::logic_error("prefill: the prompt does not fit the KV cache");
+  if (T > cos.shape()[1]) throw std::logic_error("prefill: prompt longer than the RoPE tables");
+  const int dt = (int)x.dtype();
+  const size_t el = size_in_bytes(x.dtype());
+  const Tensor qkv = x.reshape({B * T, C}).matmul(packed_qkv(cache));  // [B*T, 3C]
+  const char* q_data = (const char*)qkv.data();
+  const char* k_data = q_data + C * el;
+  const char* v_data = q_data + 2 * C * el;
+  const Tensor cc = cos.compact(), sc = sin.compact();  // rows [0,T) of the tables are used
+  // q, k, v as [B,T,H,D] views of the fused projection rows
+  const int64_t bthd[4] = {T * 3 * C, 3 * C, D, 1};
+  const int64_t cache_bhtd[4] = {H * cap * D, cap * D, D, 1};
+  Tensor qh = empty({B, H, T, D}, x.dtype(), true);
+  check(deers_rocm_rope_fwd(dt, q_data, bthd, cc.data(), sc.data(), qh.data(), nullptr, B, T, H, D));
+  // rotated keys straight into rows [0,T) of the cache, values beside them
+  check(deers_rocm_rope_fwd(dt, k_data, bthd, cc.data(), sc.data(), cache.k.data(), cache_bhtd, B, T, H, D));
+  const int64_t shape_bhtd[4] = {B, H, T, D}, v_bhtd[4] = {T * 3 * C, D, 3 * C, 1};
+  check(deers_rocm_copy_view(dt, v_data, v_bhtd, cache.v.data(), cache_bhtd, shape_bhtd, 4));
+  cache.len = T;
+  // the fused causal forward reads keys and values from the cache and writes the merged
+  // heads [B,T,H*D] directly (its output taken as a [B,H,T,D] view of that buffer)
+  Tensor y = empty({B * T, C}, x.dtype(), true);
+  Tensor lse = empty({B, H, T}, DType::F32, true);
+  const int64_t y_bhtd[4] = {T * C, D, C, 1};
+  const double scale = 1.0 / std::sqrt((double)D);
+  check(deers_rocm_attn_fwd(dt, qh.data(), nullptr, cache.k.data(), cache_bhtd, cache.v.data(), cache_bhtd,
+                            y.data(), y_bhtd, (float*)lse.data(), B, H, T, D, (float)scale));
+  if (residual) {
+    matmul_add_into(y, wo_, residual->reshape({B * T, C}));
+    return *residual;
+  }
+  return y.matmul(wo_).reshape({B, T, C});
+}
+
 Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos,
                                         const Tensor& sin, const Tensor* residual) const {
   NoGradGuard no_grad;
@@ -520,16 +578,7 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   const int dt = (int)x_t.dtype();
   const size_t el = size_in_bytes(x_t.dtype());
   const Tensor x_flat = x_t.reshape({B, C});
-  if (!cache.wqkv.defined()) {
-    cache.wqkv = empty({C, 3 * C}, x_t.dtype(), true);
-    const Tensor* w[3] = {&wq_, &wk_, &wv_};
-    for (int i = 0; i < 3; ++i) {
-      const Tensor wc = w[i]->compact();
-      const int64_t wshape[2] = {C, C}, src[2] = {C, 1}, dst[2] = {3 * C, 1};
-      check(deers_rocm_copy_view(dt, wc.data(), src, (char*)cache.wqkv.data() + i * C * el, dst, wshape, 2));
-    }
-  }
-  const Tensor qkv = x_flat.matmul(cache.wqkv);  // [B, 3C]: q | k | v, each [B, H*D]
+  const Tensor qkv = x_flat.matmul(packed_qkv(cache));  // [B, 3C]: q | k | v, each [B, H*D]
   const char* q_data = (const char*)qkv.data();
   const char* k_data = q_data + C * el;
   const char* v_data = q_data + 2 * C * el;

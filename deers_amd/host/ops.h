@@ -257,9 +257,17 @@ class CausalSelfAttention {
   // (one launch for `residual + attn(x_t)`) and it is returned.
   Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,
                      const Tensor* residual = nullptr) const;
+  // The whole prompt at once (inference, no autograd): x [B,T,C] at positions [0,T) of an
+  // empty cache.  Rotated keys and values go to rows [0,T) of the cache, the fused causal
+  // forward reads them from there; returns [B,T,C] equal to forward() (same kernels), and
+  // leaves the cache as T decode_steps would (to the rounding of the projection GEMMs).
+  // `residual` ([B,T,C], compact) as in decode_step.
+  Tensor prefill(const Tensor& x, KvCache& cache, const Tensor& cos, const Tensor& sin,
+                 const Tensor* residual = nullptr) const;
   std::vector<Tensor> parameters() const { return {wq_, wk_, wv_, wo_}; }
 
  private:
+  const Tensor& packed_qkv(KvCache& cache) const;  // packs (Wq | Wk | Wv) at first use
   int64_t n_head_, head_dim_;
   Tensor wq_, wk_, wv_, wo_;
 };

@@ -288,7 +288,8 @@ def test_host_gpt_training_step_matches_oracle(tmp_path, cfg, B, T):
 def test_host_gpt_generation_with_kv_caches(tmp_path):
     """An f16 GPT generating through per-block KV caches: every decode step's logits equal
     the matching row of the full causal forward (device) and the f32 oracle on the same
-    f16 weights; the greedy continuation picks the teacher-forced argmax at every position."""
+    f16 weights; a prompt taken through prefill leaves the same logits and caches as its tokens
+    one by one; the greedy continuation picks the teacher-forced argmax at every position."""
     from oracle import gpt as ogpt
     from test_oracle_gpt import make_weights
     cfg = dict(vocab_size=300, sequence_len=48, n_layer=2, n_head=2, n_embd=128, mlp_hidden_dim=256,
@@ -314,8 +315,21 @@ def test_host_gpt_generation_with_kv_caches(tmp_path):
     assert np.abs(full - want).max() <= 2e-2 * scale
     assert np.abs(steps - want).max() <= 2e-2 * scale
     assert np.abs(steps - full).max() <= 2e-2 * scale
-    # greedy continuation
+    # the first half through prefill, the second half step by step from its caches
     t0 = T // 2
+    pre = np.fromfile(tmp_path / "logits_prefill.bin", dtype=np.float16).reshape(B, V).astype(np.float32)
+    assert np.abs(pre - want[:, t0 - 1]).max() <= 2e-2 * scale
+    assert np.abs(pre - full[:, t0 - 1]).max() <= 2e-2 * scale
+    rest = np.fromfile(tmp_path / "logits_after_prefill.bin", dtype=np.float16).reshape(B, T - t0, V)
+    assert np.abs(rest.astype(np.float32) - want[:, t0:]).max() <= 2e-2 * scale
+    H, D = cfg["n_head"], cfg["n_embd"] // cfg["n_head"]
+    for name in ("k", "v"):
+        a = np.fromfile(tmp_path / f"{name}_cache_prefill.bin", dtype=np.float16).reshape(B, H, T, D)
+        b = np.fromfile(tmp_path / f"{name}_cache_steps.bin", dtype=np.float16).reshape(B, H, T, D)
+        a, b = a.astype(np.float32), b.astype(np.float32)
+        assert np.abs(a[:, :, :t0] - b[:, :, :t0]).max() <= 2e-2 * max(1.0, np.abs(b).max()), name
+        assert np.abs(b[:, :, :t0]).max() > 0
+    # greedy continuation
     gen = np.fromfile(tmp_path / "generated.bin", dtype=np.int64).reshape(B, t0 + n_new)
     assert np.array_equal(gen[:, :t0], ids[:, :t0])
     assert gen.min() >= 0 and gen.max() < V
