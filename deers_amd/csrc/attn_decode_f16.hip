@@ -16,6 +16,13 @@
 //   With one split per head (enough heads to give every CU a workgroup) the
 //   workgroup writes the f16 output itself; otherwise a second tiny kernel merges
 //   the splits in split order.
+//
+//   Append form (a generation step): instead of a ready query the kernel takes the new
+//   token's q, k, v projections, rotates q and k at the token's position (the
+//   arithmetic of decode_qkv_kernel: f32, one rounding to f16), writes k and v to cache
+//   row L and attends over rows [0, L] -- rows [0, L) streamed from the cache, row L from
+//   the registers that hold it, so nothing written by this launch is read back from
+//   memory.  One launch per block and step instead of two.
 #include "common.h"
 
 namespace deers {
@@ -36,7 +43,28 @@ int decode_pick_splits(int64_t BH, int64_t L, int* chunk) {
   return splits;
 }
 
+// The thread's 8 columns (8*part ..) of rotate_half RoPE applied to one [D] row: columns
+// below D/2 are x1*cos + x2*sin, the others x2*cos - x1*sin, with x1 / x2 the lower /
+// upper half's elements of the same index (src/models/gpt.rs:49-73).
 template <int D>
+__device__ __forceinline__ half8 rotate_row(const half_t* row, const half_t* cos_row, const half_t* sin_row,
+                                            int part) {
+  constexpr int HALF = D / 2;
+  const int col = 8 * part;
+  const bool upper = col >= HALF;
+  const int c = upper ? col - HALF : col;
+  const half8 a1 = *(const half8*)(row + c), a2 = *(const half8*)(row + c + HALF);
+  const half8 cs = *(const half8*)(cos_row + c), sn = *(const half8*)(sin_row + c);
+  half8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float x1 = (float)a1[e], x2 = (float)a2[e], co = (float)cs[e], si = (float)sn[e];
+    out[e] = upper ? (half_t)(x2 * co - x1 * si) : (half_t)(x1 * co + x2 * si);
+  }
+  return out;
+}
+
+template <int D, bool APPEND>
 __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
   constexpr int LPR = D / 8;        // lanes per cache row
   constexpr int GROUPS = 256 / LPR; // row groups per workgroup
@@ -53,7 +81,22 @@ __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
 
   const half_t* K = (const half_t*)p.k + b * p.skb + h * p.skh + 8 * part;
   const half_t* V = (const half_t*)p.v + b * p.skb + h * p.skh + 8 * part;
-  const half8 qh = *(const half8*)((const half_t*)p.q + (int64_t)bh * D + 8 * part);
+  half8 qh;
+  half8 k_new = {0, 0, 0, 0, 0, 0, 0, 0}, v_new = {0, 0, 0, 0, 0, 0, 0, 0};
+  // the new row is handled by one lane group of the last split
+  const bool owns_new_row = APPEND && grp == 0 && split == p.splits - 1;
+  if constexpr (APPEND) {
+    const int64_t in_off = b * p.in_b + h * p.in_h;
+    qh = rotate_row<D>((const half_t*)p.q_in + in_off, (const half_t*)p.cos_row, (const half_t*)p.sin_row, part);
+    if (owns_new_row) {
+      k_new = rotate_row<D>((const half_t*)p.k_in + in_off, (const half_t*)p.cos_row, (const half_t*)p.sin_row, part);
+      v_new = *(const half8*)((const half_t*)p.v_in + in_off + 8 * part);
+      *(half8*)(const_cast<half_t*>(K) + (int64_t)p.L * p.skl) = k_new;
+      *(half8*)(const_cast<half_t*>(V) + (int64_t)p.L * p.skl) = v_new;
+    }
+  } else {
+    qh = *(const half8*)((const half_t*)p.q + (int64_t)bh * D + 8 * part);
+  }
   float qf[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) qf[e] = (float)qh[e] * p.scale_log2;
@@ -110,6 +153,21 @@ __global__ __launch_bounds__(256) void attn_decode_f16_kernel(DecodeParams p) {
     m = m_new;
   }
 
+  if (owns_new_row) {  // row L from registers (a whole lane group takes this branch)
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += qf[e] * (float)k_new[e];
+#pragma unroll
+    for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    const float m_new = fmaxf(m, acc);
+    const float alpha = fast_exp2(m - m_new);  // 0 when no cached row was seen (m = -inf)
+    const float pu = fast_exp2(acc - m_new);
+    l = l * alpha + pu;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = o[e] * alpha + pu * (float)v_new[e];
+    m = m_new;
+  }
+
   // ---- merge the row groups of this workgroup (fixed order) ----
   if (part == 0) {
     red_m[grp] = m;
@@ -162,14 +220,17 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(DecodeParams p) {
   ((half_t*)p.o)[(int64_t)bh * D + d] = (half_t)(osum / lsum);
 }
 
-void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream) {
+void launch_attn_decode_f16(const DecodeParams& p, int B, int D, bool append, hipStream_t stream) {
   dim3 grid(p.splits, B * p.H);
   {
-    LaunchScope scope("attn_decode_f16", stream);
-    if (D == 64)
-      hipLaunchKernelGGL(attn_decode_f16_kernel<64>, grid, dim3(256), 0, stream, p);
-    else
-      hipLaunchKernelGGL(attn_decode_f16_kernel<128>, grid, dim3(256), 0, stream, p);
+    LaunchScope scope(append ? "attn_decode_append_f16" : "attn_decode_f16", stream);
+    if (D == 64) {
+      if (append) hipLaunchKernelGGL((attn_decode_f16_kernel<64, true>), grid, dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((attn_decode_f16_kernel<64, false>), grid, dim3(256), 0, stream, p);
+    } else {
+      if (append) hipLaunchKernelGGL((attn_decode_f16_kernel<128, true>), grid, dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((attn_decode_f16_kernel<128, false>), grid, dim3(256), 0, stream, p);
+    }
   }
   if (p.splits > 1) {
     LaunchScope scope("attn_decode_merge", stream);

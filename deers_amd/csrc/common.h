@@ -237,6 +237,12 @@ struct DecodeParams {
   int64_t skb, skh, skl;          // cache strides (elements)
   int H, L, splits, chunk;
   float scale_log2;
+  // append form: the new token's projections [B,H,D] by element strides in_b, in_h, the
+  // D/2 cos / sin entries of its position; its rotated key and its value become cache
+  // row L (the cache holds L rows when the kernel starts) and take part in the softmax
+  const void* q_in; const void* k_in; const void* v_in;
+  const void* cos_row; const void* sin_row;
+  int64_t in_b, in_h;
 };
 
 // Maps a block id (blockIdx.x, or blockIdx.x minus a multiple of 8) to (head, block

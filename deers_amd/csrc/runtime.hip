@@ -27,7 +27,7 @@ void launch_attn_fwd_f16(const FwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_fwd_f32(const FwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream);
-void launch_attn_decode_f16(const DecodeParams& p, int B, int D, hipStream_t stream);
+void launch_attn_decode_f16(const DecodeParams& p, int B, int D, bool append, hipStream_t stream);
 int decode_pick_splits(int64_t BH, int64_t L, int* chunk);
 void launch_fill(int dtype_f16, void* dst, size_t n, float value, hipStream_t stream);
 void launch_add(int dtype_f16, const void* a, const void* b, void* out, size_t n,
@@ -40,8 +40,8 @@ bool skinny_gemm_takes(int64_t m, int64_t n, int64_t k, int64_t ldx, int64_t ldw
 int skinny_gemm_splits(int64_t n, int64_t k);
 size_t skinny_gemm_workspace_bytes(int64_t n, int splits);
 void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
-                            int m, int n, int k, bool accumulate, int splits, float* partial,
-                            int* counters, hipStream_t stream);
+                            int m, int n, int k, bool accumulate, int prologue, float eps, bool packed,
+                            int splits, float* partial, int* counters, hipStream_t stream);
 void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* v,
                        const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
                        void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
@@ -653,7 +653,55 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
   p.part_ml = reinterpret_cast<float*>(static_cast<char*>(ws) + part_o);
   p.H = (int)H; p.L = (int)L; p.splits = splits; p.chunk = chunk;
   p.scale_log2 = (float)((double)scale * 1.4426950408889634);
-  deers::launch_attn_decode_f16(p, (int)B, (int)D, g_rt.stream);
+  deers::launch_attn_decode_f16(p, (int)B, (int)D, false, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_attn_decode_append(int dtype, const void* q, const void* k, const void* v,
+                                  const int64_t* in_strides, const void* cos_row, const void* sin_row,
+                                  void* k_cache, void* v_cache, const int64_t* cache_strides, void* o,
+                                  int64_t pos, int64_t capacity, int64_t B, int64_t H, int64_t D,
+                                  float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (dtype != DEERS_ROCM_F16)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: only DEERS_ROCM_F16 caches are supported");
+  if (B < 1 || H < 1 || B * H > 65535 || capacity > (int64_t(1) << 30))
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: need B,H >= 1, B*H <= 65535, capacity <= 2^30");
+  if (pos < 0 || pos >= capacity)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: position %lld outside the cache capacity %lld",
+                (long long)pos, (long long)capacity);
+  if (D != 64 && D != 128)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: head dim %lld unsupported (64 or 128)", (long long)D);
+  if (!q || !k || !v || !in_strides || !cos_row || !sin_row || !k_cache || !v_cache || !cache_strides || !o)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: null pointer");
+  if (int rc = check_scale(scale)) return rc;
+  for (int d = 0; d < 2; ++d)
+    if (in_strides[d] < 0 || in_strides[d] % 8)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "attn_decode_append: input strides must be non-negative multiples of 16 bytes");
+  for (int d = 0; d < 3; ++d)
+    if (cache_strides[d] < 0 || cache_strides[d] % 8)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "attn_decode_append: cache strides must be non-negative multiples of 16 bytes");
+  const void* ptrs[8] = {q, k, v, cos_row, sin_row, k_cache, v_cache, o};
+  for (const void* ptr : ptrs)
+    if ((uintptr_t)ptr & 15) return fail(DEERS_ROCM_ERR_LAYOUT, "attn_decode_append: pointers must be 16-byte aligned");
+  deers::DecodeParams p{};
+  p.skb = cache_strides[0]; p.skh = cache_strides[1]; p.skl = cache_strides[2];
+  int chunk = 0;
+  const int splits = deers::decode_pick_splits(B * H, pos, &chunk);  // over the rows already cached
+  void* ws = nullptr;
+  const size_t part_o = (size_t)(B * H) * splits * D * sizeof(float);
+  const size_t part_ml = (size_t)(B * H) * splits * 2 * sizeof(float);
+  if (int rc = workspace(part_o + part_ml, &ws)) return rc;
+  p.k = k_cache; p.v = v_cache; p.o = o;
+  p.q_in = q; p.k_in = k; p.v_in = v; p.cos_row = cos_row; p.sin_row = sin_row;
+  p.in_b = in_strides[0]; p.in_h = in_strides[1];
+  p.part_o = static_cast<float*>(ws);
+  p.part_ml = reinterpret_cast<float*>(static_cast<char*>(ws) + part_o);
+  p.H = (int)H; p.L = (int)pos; p.splits = splits; p.chunk = chunk;
+  p.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  deers::launch_attn_decode_f16(p, (int)B, (int)D, true, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }
@@ -1231,6 +1279,27 @@ int deers_rocm_matmul_tune(int on) {
 
 constexpr int kSkinnyCounters = 4096;  // column blocks a K-split launch of the few-rows GEMM may have
 
+// The few-rows GEMM on operands skinny_gemm_takes() accepted; prologue 0 none, 1 rms_norm
+// of x's rows, 2 relu(x)^2.  The caller holds g_mu.
+static int skinny_locked(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t m,
+                         int64_t n, int64_t k, bool accumulate, int prologue, float eps, bool packed) {
+  int splits = prologue == 1 ? 1 : deers::skinny_gemm_splits(n, k);  // row sums of squares need all of K
+  void* ws = nullptr;
+  if (splits > 1 && (n + 31) / 32 > kSkinnyCounters) splits = 1;
+  if (splits > 1) {
+    if (int rc = workspace(deers::skinny_gemm_workspace_bytes(n, splits), &ws)) return rc;
+    if (!g_rt.skinny_counters) {  // zero once; the kernel leaves every counter at zero
+      HIP_TRY(hipMalloc(&g_rt.skinny_counters, kSkinnyCounters * sizeof(int)));
+      HIP_TRY(hipMemsetAsync(g_rt.skinny_counters, 0, kSkinnyCounters * sizeof(int), g_rt.stream));
+    }
+  }
+  deers::LaunchScope scope("matmul", g_rt.stream);
+  deers::launch_skinny_gemm_f16(x, ldx, w, ldw, y, n, (int)m, (int)n, (int)k, accumulate, prologue, eps, packed,
+                                splits, (float*)ws, g_rt.skinny_counters, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
 // c = a @ b (accumulate = false) or c += a @ b (true); the caller holds g_mu
 static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
                          const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
@@ -1267,23 +1336,8 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
   // a few rows against a weight matrix (a generation step's projections): one streaming
   // pass over the weights instead of a library GEMM
   if (dtype == DEERS_ROCM_F16 && batch == 1 && !a_t && !b_t &&
-      deers::skinny_gemm_takes(m, n, k, lda, ldb, n, a, b, c)) {
-    int splits = deers::skinny_gemm_splits(n, k);
-    void* ws = nullptr;
-    if (splits > 1 && (n + 31) / 32 > kSkinnyCounters) splits = 1;
-    if (splits > 1) {
-      if (int rc = workspace(deers::skinny_gemm_workspace_bytes(n, splits), &ws)) return rc;
-      if (!g_rt.skinny_counters) {  // zero once; the kernel leaves every counter at zero
-        HIP_TRY(hipMalloc(&g_rt.skinny_counters, kSkinnyCounters * sizeof(int)));
-        HIP_TRY(hipMemsetAsync(g_rt.skinny_counters, 0, kSkinnyCounters * sizeof(int), g_rt.stream));
-      }
-    }
-    deers::LaunchScope scope("matmul", g_rt.stream);
-    deers::launch_skinny_gemm_f16(a, lda, b, ldb, c, n, (int)m, (int)n, (int)k, accumulate, splits,
-                                  (float*)ws, g_rt.skinny_counters, g_rt.stream);
-    HIP_TRY(hipGetLastError());
-    return DEERS_ROCM_OK;
-  }
+      deers::skinny_gemm_takes(m, n, k, lda, ldb, n, a, b, c))
+    return skinny_locked(a, lda, b, ldb, c, m, n, k, accumulate, 0, 0.f, false);
   if (!g_rt.blas) {
     if (rocblas_create_handle(&g_rt.blas) != rocblas_status_success)
       return fail(DEERS_ROCM_ERR_HIP, "rocblas_create_handle failed");
@@ -1382,6 +1436,23 @@ int deers_rocm_matmul_acc(int dtype, const void* a, int64_t a_rs, int64_t a_cs, 
                           int64_t batch, int64_t m, int64_t n, int64_t k) {
   std::lock_guard<std::mutex> lock(g_mu);
   return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, batch, m, n, k, true);
+}
+
+int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, int64_t ldx, const void* w,
+                             int64_t ldw, void* y, int accumulate, int64_t m, int64_t n, int64_t k) {
+  const bool packed = ldw == DEERS_ROCM_LINEAR_W_PACKED;
+  if (packed) ldw = n;  // for the shape rules below
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (prologue < DEERS_ROCM_LINEAR_PLAIN || prologue > DEERS_ROCM_LINEAR_RELU_SQ)
+    return fail(DEERS_ROCM_ERR_ARG, "decode_linear: unknown prologue %d", prologue);
+  if (!x || !w || !y) return fail(DEERS_ROCM_ERR_ARG, "decode_linear: null pointer");
+  if (dtype != DEERS_ROCM_F16 || !deers::skinny_gemm_takes(m, n, k, ldx, ldw, n, x, w, y))
+    return fail(DEERS_ROCM_ERR_ARG,
+                "decode_linear: f16, 1 <= m <= 32, n %% 8 == 0, k %% 256 == 0, row strides multiples of "
+                "8 elements and 16-byte aligned pointers (m %lld n %lld k %lld)",
+                (long long)m, (long long)n, (long long)k);
+  return skinny_locked(x, ldx, w, ldw, y, m, n, k, accumulate != 0, prologue, eps, packed);
 }
 #pragma clang diagnostic pop
 

@@ -19,6 +19,18 @@
 //          L2, and the one that arrives last (a counter per column block, reset by that
 //          workgroup) adds the S partials in index order: one launch, same bits whoever
 //          is last.
+//   x      optionally transformed on the way in, so that a generation step needs no launch
+//          of its own for them: kSkinnyReluSq squares the positive part of every x element
+//          as it leaves LDS (the MLP's activation, src/models/gpt.rs:196-203; the same
+//          f32 arithmetic and single rounding as the stand-alone kernel); kSkinnyRmsNorm
+//          multiplies row m of the result by (mean(x[m,:]^2) + eps)^-1/2, which is
+//          rms_norm(x) @ W (src/nn.rs:244-251) without the rounding of the normalised row
+//          to f16 in between; the sums of squares are taken from the x tiles the MFMAs
+//          read anyway.  The latter needs a workgroup to see all of K (no split).
+//   W      row-major [K][N], or packed as [N/32 column blocks][K][32]: a workgroup's share of
+//          a row-major W is 64 bytes out of every row, and fetched from HBM (a generation
+//          step cycles through more weights and cache than the last-level cache holds) such
+//          scattered pieces cost 2-3 us per launch more than the same bytes in one run.
 // Shapes: K a multiple of 256 (every wave then owns whole chunks), N a multiple of 8,
 // rows 16-byte aligned; the caller falls back to the library otherwise.
 #include "common.h"
@@ -27,6 +39,7 @@ namespace deers {
 
 namespace {
 
+constexpr int kSkinnyPlain = 0, kSkinnyRmsNorm = 1, kSkinnyReluSq = 2;  // the entry point's codes
 constexpr int kSkWaves = 4;
 constexpr int kSkStepsPerChunk = 4;           // k-steps of 16
 constexpr int kSkRing = 3;                    // chunks per wave in LDS
@@ -35,12 +48,13 @@ constexpr int kSkChunkBytes = kSkStepsPerChunk * kSkStepBytes;
 constexpr int kSkWaveBytes = kSkRing * kSkChunkBytes;
 constexpr int kSkLds = kSkWaves * kSkWaveBytes;  // 96 KB
 
-template <bool ACCUMULATE>
+template <bool ACCUMULATE, int PROLOGUE>
 __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __restrict__ x, int64_t ldx,
                                                               const half_t* __restrict__ W, int64_t ldw,
                                                               half_t* __restrict__ y, int64_t ldy, int M,
                                                               int N, int K, int S, float* __restrict__ partial,
-                                                              int* __restrict__ counters) {
+                                                              int* __restrict__ counters, float eps,
+                                                              int64_t w_block_stride) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -65,7 +79,9 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
   // x tile of a step: lane -> row lane/2 of 32 (clamped to M-1), 16-byte piece lane%2
   const int x_row = min(lane >> 1, M - 1);
   const uint32_t x_lane_off = (uint32_t)((x_row * ldx + 8 * (lane & 1)) * 2);
-  const half_t* w_base = W + n0;
+  // row-major W: the block's 32 columns start 32 elements after the previous block's, rows
+  // ldw apart; packed W ([column block][K][32]): blocks K*32 apart, rows 32 apart
+  const half_t* w_base = W + col_block * w_block_stride;
 
   auto issue = [&](int chunk) {
     const uint32_t dst = lds_wave + (chunk % kSkRing) * kSkChunkBytes;
@@ -80,6 +96,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
   if (n_chunks > 1) issue(1);
 
   floatx16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float sum_sq = 0.f;  // kSkinnyRmsNorm: this lane's share of sum(x[m,:]^2), m = lane % 32
   for (int c = 0; c < n_chunks; ++c) {
     if (c + 2 < n_chunks) {
       issue(c + 2);
@@ -97,7 +114,19 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
       const half8 a = lds_frag_transposed(wt, 32, 0, 0, lane);  // column lane%32; k = 4g..4g+3, 8+4g..
       const half4 b_lo = *(const half4*)(xt + (lane & 31) * 16 + 4 * g);
       const half4 b_hi = *(const half4*)(xt + (lane & 31) * 16 + 8 + 4 * g);
-      acc = mfma_f16(a, __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7), acc);
+      half8 b = __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      if constexpr (PROLOGUE == kSkinnyReluSq) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float r = fmaxf((float)b[e], 0.f);
+          b[e] = (half_t)(r * r);
+        }
+      }
+      if constexpr (PROLOGUE == kSkinnyRmsNorm) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum_sq = fmaf((float)b[e], (float)b[e], sum_sq);
+      }
+      acc = mfma_f16(a, b, acc);
     }
     // the ring slot this chunk sat in is refilled two iterations from now by this same
     // wave, after these reads have returned (the MFMAs above consumed them)
@@ -108,6 +137,8 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
   float* red = (float*)smem;  // [wave][reg][lane]
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
+  float* red_sq = red + kSkWaves * 16 * 64;  // [wave][lane]
+  if constexpr (PROLOGUE == kSkinnyRmsNorm) red_sq[wave * 64 + lane] = sum_sq;
   __syncthreads();
   float s[8];
   const int rp = wave & 1;  // waves 0 and 1 sum and store output columns n0 + 16 rp .. + 15
@@ -118,6 +149,15 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
 #pragma unroll
       for (int w = 1; w < kSkWaves; ++w) t += red[(w * 16 + 8 * rp + e) * 64 + lane];
       s[e] = t;
+    }
+    if constexpr (PROLOGUE == kSkinnyRmsNorm) {
+      // row m's sum of squares: both lane halves of all four waves, in a fixed order
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < kSkWaves; ++w) t += red_sq[w * 64 + (lane & 31)] + red_sq[w * 64 + 32 + (lane & 31)];
+      const float inv = 1.0f / sqrtf(t / (float)K + eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s[e] *= inv;
     }
   }
   if (S > 1) {
@@ -219,25 +259,38 @@ size_t skinny_gemm_workspace_bytes(int64_t n, int splits) {
   return splits > 1 ? (size_t)((n + 31) / 32) * splits * 2 * 64 * 8 * sizeof(float) : 0;
 }
 
-void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
-                            int m, int n, int k, bool accumulate, int splits, float* partial,
-                            int* counters, hipStream_t stream) {
+template <bool ACCUMULATE, int PROLOGUE>
+static void launch_one(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy, int m,
+                       int n, int k, int splits, float* partial, int* counters, float eps, bool packed,
+                       hipStream_t stream) {
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)skinny_gemm_f16_kernel<false>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kSkLds);
-    (void)hipFuncSetAttribute((const void*)skinny_gemm_f16_kernel<true>,
+    (void)hipFuncSetAttribute((const void*)skinny_gemm_f16_kernel<ACCUMULATE, PROLOGUE>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, kSkLds);
     attr_set = true;
   }
   const int col_blocks = (n + 31) / 32;
   const dim3 grid((unsigned)(8 * splits * ((col_blocks + 7) / 8)));
-  if (accumulate)
-    hipLaunchKernelGGL(skinny_gemm_f16_kernel<true>, grid, dim3(256), kSkLds, stream, (const half_t*)x, ldx,
-                       (const half_t*)w, ldw, (half_t*)y, ldy, m, n, k, splits, partial, counters);
-  else
-    hipLaunchKernelGGL(skinny_gemm_f16_kernel<false>, grid, dim3(256), kSkLds, stream, (const half_t*)x, ldx,
-                       (const half_t*)w, ldw, (half_t*)y, ldy, m, n, k, splits, partial, counters);
+  hipLaunchKernelGGL((skinny_gemm_f16_kernel<ACCUMULATE, PROLOGUE>), grid, dim3(256), kSkLds, stream,
+                     (const half_t*)x, ldx, (const half_t*)w, packed ? (int64_t)32 : ldw, (half_t*)y, ldy, m, n, k,
+                     splits, partial, counters, eps, packed ? (int64_t)k * 32 : (int64_t)32);
+}
+
+// prologue: kSkinnyPlain, kSkinnyRmsNorm (splits must be 1) or kSkinnyReluSq; packed: w is
+// [ceil(n/32)][k][32] (each workgroup's columns contiguous) instead of row-major
+void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
+                            int m, int n, int k, bool accumulate, int prologue, float eps, bool packed,
+                            int splits, float* partial, int* counters, hipStream_t stream) {
+#define DEERS_SKINNY_CASE(ACC, PRO)                                                                      \
+  if (accumulate == ACC && prologue == PRO)                                                              \
+    return launch_one<ACC, PRO>(x, ldx, w, ldw, y, ldy, m, n, k, splits, partial, counters, eps, packed, stream);
+  DEERS_SKINNY_CASE(false, kSkinnyPlain)
+  DEERS_SKINNY_CASE(true, kSkinnyPlain)
+  DEERS_SKINNY_CASE(false, kSkinnyRmsNorm)
+  DEERS_SKINNY_CASE(true, kSkinnyRmsNorm)
+  DEERS_SKINNY_CASE(false, kSkinnyReluSq)
+  DEERS_SKINNY_CASE(true, kSkinnyReluSq)
+#undef DEERS_SKINNY_CASE
 }
 
 }  // namespace deers

@@ -36,12 +36,29 @@ Tensor MLP::forward(const Tensor& x) const {
   return y.matmul(down_).reshape({B, T, C});
 }
 
-void MLP::forward_add_into(const Tensor& x, const Tensor& residual) const {
+void MLP::forward_add_into(const Tensor& x, const Tensor& residual, const double* norm_eps,
+                           KvCache* cache) const {
   NoGradGuard no_grad;
   if (x.layout().ndim() != 3) throw std::logic_error("MLP expects input shape [B, T, C]");
   const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
-  const Tensor y = relu_sq(x.reshape({B * T, C}).matmul(up_));  // [B*T, H]
-  matmul_add_into(y, down_, residual.reshape({B * T, C}));
+  const Tensor res = residual.reshape({B * T, C});
+  // [B*T, H] before the activation, which rides on the down projection
+  LinearWeight up, down;
+  if (cache) {
+    if (!cache->step_up.w.defined()) {
+      cache->step_up = LinearWeight::pack(up_);
+      cache->step_down = LinearWeight::pack(down_);
+    }
+    up = cache->step_up;
+    down = cache->step_down;
+  } else {
+    up.w = up_;
+    down.w = down_;
+  }
+  const Tensor u = fused_linear(x.reshape({B * T, C}), up,
+                                norm_eps ? LinearPrologue::RmsNorm : LinearPrologue::Plain,
+                                norm_eps ? *norm_eps : 0.0, nullptr);
+  fused_linear(u, down, LinearPrologue::ReluSq, 0.0, &res);
 }
 
 Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
@@ -57,8 +74,8 @@ Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, 
   // the residual stream is updated in place: both additions ride on the last product of
   // their branch (x_t's storage is overwritten; inference only)
   const Tensor h = x_t.compact();
-  attn_.decode_step(rms_norm(h, eps_), cache, cos, sin, &h);
-  mlp_.forward_add_into(rms_norm(h, eps_), h);
+  attn_.decode_step(h, cache, cos, sin, &h, &eps_);
+  mlp_.forward_add_into(h, h, &eps_, &cache);
   return h;
 }
 

@@ -30,7 +30,12 @@ class MLP {
   Tensor forward(const Tensor& x) const;  // [B,T,C] -> [B,T,C]
   // residual ([B,T,C], compact) += forward(x), the addition riding on the down projection
   // (inference: the residual's storage is updated in place)
-  void forward_add_into(const Tensor& x, const Tensor& residual) const;
+  // With `norm_eps` x is the un-normalised stream and its RMSNorm is folded into the up
+  // projection where one launch can do both (a generation step's few rows).
+  // `cache`, when given, holds (and at first use receives) the two weights in the layout a
+  // generation step streams fastest.
+  void forward_add_into(const Tensor& x, const Tensor& residual, const double* norm_eps = nullptr,
+                        KvCache* cache = nullptr) const;
   std::vector<Tensor> parameters() const { return {up_, down_}; }
 
  private:

@@ -71,6 +71,9 @@ static int run_generate(int argc, char** argv) {
     check(deers_rocm_argmax_rows((int)logits.dtype(), logits.data(), (int64_t*)next.data(), B, cfg.vocab_size));
     logits = model.decode_step(next, caches);
   }
+  // how long the host needed to enqueue the steps: close to the wall time means the loop is
+  // bound by the launch rate, well below it means the device is the limit
+  const double enqueue_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s0).count() / n_new;
   check(deers_rocm_sync());
   const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s0).count() / n_new;
   // a few more steps with every launch bracketed by events: device time per kernel family
@@ -108,9 +111,9 @@ static int run_generate(int argc, char** argv) {
   const double w_bytes = 2.0 * (n_params - cfg.vocab_size * cfg.n_embd);  // every weight but the embedding table
   std::printf("{\"mode\": \"generate\", \"ms_per_token_step\": %.4f, \"tokens_per_s\": %.1f, \"batch\": %lld, "
               "\"context\": %lld, \"new_tokens\": %lld, \"bytes_per_step\": %.0f, \"GB_per_s\": %.1f, "
-              "\"prefill_ms\": %.3f, \"prefill_tokens_per_s\": %.0f, \"kernels\": %s}\n",
+              "\"host_enqueue_ms_per_step\": %.4f, \"prefill_ms\": %.3f, \"prefill_tokens_per_s\": %.0f, \"kernels\": %s}\n",
               ms, 1e3 * B / ms, (long long)B, (long long)t0, (long long)n_new, kv_bytes + w_bytes,
-              (kv_bytes + w_bytes) / (ms * 1e-3) / 1e9, prefill_ms, 1e3 * B * t0 / prefill_ms, kernels.c_str());
+              (kv_bytes + w_bytes) / (ms * 1e-3) / 1e9, enqueue_ms, prefill_ms, 1e3 * B * t0 / prefill_ms, kernels.c_str());
   return 0;
 }
 

@@ -567,7 +567,8 @@ Tensor CausalSelfAttention::prefill(const Tensor& x, KvCache& cache, const Tenso
 }
 
 Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos,
-                                        const Tensor& sin, const Tensor* residual) const {
+                                        const Tensor& sin, const Tensor* residual,
+                                        const double* norm_eps) const {
   NoGradGuard no_grad;
   if (x_t.layout().ndim() != 3 || x_t.shape()[1] != 1)
     throw std::logic_error("decode_step expects input shape [B, 1, C]");
@@ -578,7 +579,14 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   const int dt = (int)x_t.dtype();
   const size_t el = size_in_bytes(x_t.dtype());
   const Tensor x_flat = x_t.reshape({B, C});
-  const Tensor qkv = x_flat.matmul(packed_qkv(cache));  // [B, 3C]: q | k | v, each [B, H*D]
+  // [B, 3C]: q | k | v, each [B, H*D]
+  if (!cache.step_qkv.w.defined()) {
+    cache.step_qkv = LinearWeight::pack(packed_qkv(cache));
+    cache.step_out = LinearWeight::pack(wo_);
+  }
+  const Tensor qkv = fused_linear(x_flat, cache.step_qkv,
+                                  norm_eps ? LinearPrologue::RmsNorm : LinearPrologue::Plain,
+                                  norm_eps ? *norm_eps : 0.0, nullptr);
   const char* q_data = (const char*)qkv.data();
   const char* k_data = q_data + C * el;
   const char* v_data = q_data + 2 * C * el;
@@ -586,22 +594,64 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   const Tensor cc = cos.compact(), sc = sin.compact();
   const char* cos_t = (const char*)cc.data() + pos * (D / 2) * el;
   const char* sin_t = (const char*)sc.data() + pos * (D / 2) * el;
-  // rotate q and k at this position, append k and v to the caches: one launch
   const int64_t in_strides[2] = {3 * C, D};                          // [B,H,D] inside a [B, 3C] row
   const int64_t kv_strides[3] = {H * cap * D, cap * D, D};
-  Tensor qh = empty({B, H, D}, x_t.dtype(), true);
-  check(deers_rocm_decode_qkv(dt, q_data, k_data, v_data, in_strides, cos_t, sin_t, qh.data(),
-                              cache.k.data(), cache.v.data(), kv_strides, pos, cap, B, H, D));
-  cache.len = pos + 1;
+  // rotate q and k at this position, append k and v to the caches, attend over the
+  // cache.len + 1 rows: one launch
   Tensor o = empty({B, H * D}, x_t.dtype(), true);
   const double scale = 1.0 / std::sqrt((double)D);
-  check(deers_rocm_attn_decode(dt, qh.data(), cache.k.data(), cache.v.data(), kv_strides, o.data(), B,
-                               H, cache.len, D, (float)scale));
+  check(deers_rocm_attn_decode_append(dt, q_data, k_data, v_data, in_strides, cos_t, sin_t, cache.k.data(),
+                                      cache.v.data(), kv_strides, o.data(), pos, cap, B, H, D, (float)scale));
+  cache.len = pos + 1;
   if (residual) {
-    matmul_add_into(o, wo_, residual->reshape({B, C}));
+    const Tensor res = residual->reshape({B, C});
+    fused_linear(o, cache.step_out, LinearPrologue::Plain, 0.0, &res);
     return *residual;
   }
-  return o.matmul(wo_).reshape({B, 1, C});
+  return fused_linear(o, cache.step_out, LinearPrologue::Plain, 0.0, nullptr).reshape({B, 1, C});
+}
+
+LinearWeight LinearWeight::pack(const Tensor& w) {
+  NoGradGuard no_grad;
+  if (w.layout().ndim() != 2) throw std::logic_error("LinearWeight: w [K,N]");
+  LinearWeight out;
+  out.w = w.detach().compact();
+  const int64_t K = w.shape()[0], N = w.shape()[1];
+  if (w.dtype() == DType::F16 && N % 32 == 0 && K % 256 == 0 && backed(out.w)) {
+    out.tiles = empty({N / 32, K, 32}, w.dtype(), true);
+    const int64_t shape[3] = {N / 32, K, 32}, src[3] = {32, N, 1}, dst[3] = {32 * K, 32, 1};
+    check(deers_rocm_copy_view((int)w.dtype(), out.w.data(), src, out.tiles.data(), dst, shape, 3));
+  }
+  return out;
+}
+
+Tensor fused_linear(const Tensor& x, const Tensor& w, LinearPrologue f, double eps, const Tensor* acc) {
+  LinearWeight lw;
+  lw.w = w;
+  return fused_linear(x, lw, f, eps, acc);
+}
+
+Tensor fused_linear(const Tensor& x, const LinearWeight& lw, LinearPrologue f, double eps, const Tensor* acc) {
+  NoGradGuard no_grad;
+  const Tensor& w = lw.w;
+  if (x.layout().ndim() != 2 || w.layout().ndim() != 2 || x.shape()[1] != w.shape()[0])
+    throw std::logic_error("fused_linear: x [M,K] and w [K,N]");
+  const int64_t M = x.shape()[0], K = x.shape()[1], N = w.shape()[1];
+  if (acc && (!acc->is_compact() || (int64_t)acc->layout().size() != M * N || acc->dtype() != x.dtype()))
+    throw std::logic_error("fused_linear: the accumulator must be a compact [M,N] tensor of x's type");
+  if (x.dtype() == DType::F16 && w.dtype() == DType::F16 && M >= 1 && M <= 32 && N % 8 == 0 && K % 256 == 0 &&
+      x.is_compact() && w.is_compact() && backed(x)) {
+    Tensor y = acc ? *acc : empty({M, N}, x.dtype(), true);
+    const bool tiled = lw.tiles.defined();
+    check(deers_rocm_decode_linear((int)x.dtype(), (int)f, (float)eps, x.data(), K,
+                                   tiled ? lw.tiles.data() : w.data(), tiled ? DEERS_ROCM_LINEAR_W_PACKED : N,
+                                   const_cast<void*>(y.data()), acc ? 1 : 0, M, N, K));
+    return acc ? acc->reshape({M, N}) : y;
+  }
+  const Tensor fx = f == LinearPrologue::RmsNorm ? rms_norm(x, eps) : f == LinearPrologue::ReluSq ? relu_sq(x) : x;
+  if (!acc) return fx.matmul(w);
+  matmul_add_into(fx, w, acc->reshape({M, N}));
+  return acc->reshape({M, N});
 }
 
 void matmul_add_into(const Tensor& a, const Tensor& b, const Tensor& acc) {

@@ -234,12 +234,33 @@ Tensor causal_self_attention(const Tensor& q, const Tensor& k, const Tensor& v);
 // helper: nothing is recorded for autograd, the accumulator's storage is updated in place.
 void matmul_add_into(const Tensor& a, const Tensor& b, const Tensor& acc);
 
+// f(x) @ w, or acc += f(x) @ w when `acc` is given, for x [M,K] and w [K,N]; f is the
+// weightless RMSNorm over x's rows (src/nn.rs:244-251) or relu(x)^2
+// (src/models/gpt.rs:196-203).  The few rows of a generation step (f16, M <= 32) take one
+// launch (deers_rocm_decode_linear); any other shape runs the separate ops.  Inference
+// helper: nothing is recorded for autograd.
+enum class LinearPrologue { Plain = 0, RmsNorm = 1, ReluSq = 2 };
+Tensor fused_linear(const Tensor& x, const Tensor& w, LinearPrologue f, double eps, const Tensor* acc);
+// A weight [K,N] as generation steps read it: beside the row-major tensor (shared with the
+// model) a copy stored as [N/32][K][32], the layout in which the 32 columns one workgroup of
+// the few-rows kernel streams are contiguous (f16, N % 32 == 0, K % 256 == 0; otherwise
+// `tiles` stays undefined and the row-major tensor is used).
+struct LinearWeight {
+  Tensor w;      // [K,N] row-major
+  Tensor tiles;  // packed copy, or undefined
+  static LinearWeight pack(const Tensor& w);
+};
+Tensor fused_linear(const Tensor& x, const LinearWeight& w, LinearPrologue f, double eps, const Tensor* acc);
+
 struct KvCache {
   Tensor k, v;
   // [C, 3C] = (Wq | Wk | Wv), packed by the first decode_step that uses this cache so a
   // step runs one projection GEMM instead of three; the weights must not change while
   // the cache lives
   Tensor wqkv;
+  // the block's four products of a generation step in the few-rows kernel's layout,
+  // packed by the first decode_step (same proviso)
+  LinearWeight step_qkv, step_out, step_up, step_down;
   int64_t len = 0, capacity = 0;
   static KvCache create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType dtype);
 };
@@ -255,8 +276,10 @@ class CausalSelfAttention {
   // equal to row cache.len of forward() on the whole prefix.
   // With `residual` ([B,1,C], compact) the output projection is added into it in place
   // (one launch for `residual + attn(x_t)`) and it is returned.
+  // With `norm_eps` x_t is the un-normalised residual stream and its RMSNorm happens inside
+  // the projection's launch.
   Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,
-                     const Tensor* residual = nullptr) const;
+                     const Tensor* residual = nullptr, const double* norm_eps = nullptr) const;
   // The whole prompt at once (inference, no autograd): x [B,T,C] at positions [0,T) of an
   // empty cache.  Rotated keys and values go to rows [0,T) of the cache, the fused causal
   // forward reads them from there; returns [B,T,C] equal to forward() (same kernels), and

@@ -193,6 +193,16 @@ def attn_decode_raw(dtype, q, k_cache, v_cache, o, B, H, L, D, scale, kv_strides
         ctypes.c_int64(H), ctypes.c_int64(L), ctypes.c_int64(D), ctypes.c_float(scale)))
 
 
+def attn_decode_append_raw(dtype, q, k, v, in_strides, cos_row, sin_row, k_cache, v_cache, cache_strides,
+                           o, pos, capacity, B, H, D, scale):
+    """deers_rocm_attn_decode_append: rotate q, k at `pos`, append k, v as cache row pos, attend over [0,pos]."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_attn_decode_append(
+        ctypes.c_int(dtype_code(dtype)), q, k, v, (i64 * 2)(*[int(x) for x in in_strides]), cos_row,
+        sin_row, k_cache, v_cache, (i64 * 3)(*[int(x) for x in cache_strides]), o, i64(pos),
+        i64(capacity), i64(B), i64(H), i64(D), ctypes.c_float(scale)))
+
+
 def fill_raw(dtype, dst, n, value):
     _check(load().deers_rocm_fill(ctypes.c_int(dtype_code(dtype)), dst, ctypes.c_size_t(n),
                                   ctypes.c_float(value)))
@@ -377,6 +387,18 @@ def matmul_acc_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
         ctypes.c_int(dtype_code(dtype)), a, i64(a_strides[0]), i64(a_strides[1]), i64(a_strides[2]),
         b, i64(b_strides[0]), i64(b_strides[1]), i64(b_strides[2]), c, i64(batch), i64(m), i64(n),
         i64(k)))
+
+
+LINEAR_PROLOGUES = {"plain": 0, "rms_norm": 1, "relu_sq": 2}
+LINEAR_W_PACKED = -32  # DEERS_ROCM_LINEAR_W_PACKED: pass as ldw for a [n/32][k][32] weight
+
+
+def decode_linear_raw(dtype, prologue, eps, x, ldx, w, ldw, y, accumulate, m, n, k):
+    """deers_rocm_decode_linear: y[m,n] (+)= f(x)[m,k] @ w[k,n], m <= 32, f one of LINEAR_PROLOGUES."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_decode_linear(
+        ctypes.c_int(dtype_code(dtype)), ctypes.c_int(LINEAR_PROLOGUES[prologue]), ctypes.c_float(eps), x,
+        i64(ldx), w, i64(ldw), y, ctypes.c_int(1 if accumulate else 0), i64(m), i64(n), i64(k)))
 
 
 def decode_qkv_raw(dtype, q, k, v, in_strides, cos_row, sin_row, q_out, k_cache, v_cache, cache_strides,

@@ -176,6 +176,21 @@ int deers_rocm_attn_decode(int dtype,
                            void* o,
                            int64_t B, int64_t H, int64_t L, int64_t D, float scale);
 
+/* One generation step of the attention core in one launch: deers_rocm_decode_qkv followed by
+ * deers_rocm_attn_decode.  q, k, v are the new token's projections [B,H,D] by element strides
+ * in_strides = {b, h} (D stride 1); q and k are rotated at the token's position (cos_row /
+ * sin_row: the D/2 table entries of that position, src/models/gpt.rs:49-73), the rotated k and
+ * v become row `pos` of the caches ([B,H,capacity,D] by cache_strides = {b, h, t}; rows
+ * [0,pos) hold the earlier tokens) and o [B,H,D] (compact) is the attention of the rotated q
+ * over rows [0,pos].  Same values as the two separate calls up to the order of the f32
+ * softmax sums (the new row is merged last).  D in {64,128}, f16.  The reference has no KV
+ * cache (examples/tinystories_train.rs:250-276 re-runs the window). */
+int deers_rocm_attn_decode_append(int dtype, const void* q, const void* k, const void* v,
+                                  const int64_t* in_strides, const void* cos_row,
+                                  const void* sin_row, void* k_cache, void* v_cache,
+                                  const int64_t* cache_strides, void* o, int64_t pos,
+                                  int64_t capacity, int64_t B, int64_t H, int64_t D, float scale);
+
 /* ---- element-wise helpers of the storage backend ---------------------------
  * The fused op's contract needs four more things from its backend: the seed of
  * the reverse sweep, gradient accumulation, compaction of strided views, and (for
@@ -410,6 +425,38 @@ int deers_rocm_matmul_acc(int dtype,
                           const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
                           const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
                           void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
+/* y[m,n] (+)= f(x)[m,k] @ w[k,n] for the few rows of a generation step (m <= 32), f16 only,
+ * one streaming pass over w by a kernel of this library; x, w, y row-major with row strides
+ * ldx, ldw and n.  `prologue` picks f:
+ *   DEERS_ROCM_LINEAR_PLAIN     f(x) = x (what deers_rocm_matmul runs for such shapes anyway);
+ *   DEERS_ROCM_LINEAR_RMS_NORM  f(x) = x * (mean(x^2 over the row) + eps)^-1/2, the weightless
+ *                               RMSNorm in front of both branches of a block
+ *                               (src/nn.rs:244-251, src/models/gpt.rs:240-247); the row factor
+ *                               is applied to the f32 sums, so the normalised row is not
+ *                               rounded to f16 in between as it is by deers_rocm_rms_norm_fwd
+ *                               followed by deers_rocm_matmul;
+ *   DEERS_ROCM_LINEAR_RELU_SQ   f(x) = relu(x)^2, the MLP's activation
+ *                               (src/models/gpt.rs:196-203); same bits as
+ *                               deers_rocm_relu_sq_fwd followed by deers_rocm_matmul.
+ * w is row-major with row stride ldw, or, with ldw = DEERS_ROCM_LINEAR_W_PACKED, stored as
+ * [ceil(n/32)][k][32]: element (kk, j) at ((j / 32) * k + kk) * 32 + j % 32, i.e. the 32
+ * columns one workgroup reads are one contiguous run (deers_rocm_copy_view with shape
+ * {n/32, k, 32}, source strides {32, n, 1} and destination strides {32k, 32, 1} packs a
+ * row-major matrix).  Weights that are streamed from HBM every step are 2-3 us per product
+ * faster that way.
+ * accumulate != 0 adds into y (a residual stream updated in place).  Shapes it does not take
+ * (n % 8, k % 256, unaligned rows, m > 32, another dtype) return DEERS_ROCM_ERR_ARG and
+ * launch nothing: the caller then runs the separate entry points.  No counterpart in the
+ * reference, whose sampling loop re-runs the whole window
+ * (examples/tinystories_train.rs:250-276). */
+#define DEERS_ROCM_LINEAR_PLAIN 0
+#define DEERS_ROCM_LINEAR_RMS_NORM 1
+#define DEERS_ROCM_LINEAR_RELU_SQ 2
+#define DEERS_ROCM_LINEAR_W_PACKED (-32)
+int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, int64_t ldx,
+                             const void* w, int64_t ldw, void* y, int accumulate, int64_t m,
+                             int64_t n, int64_t k);
+
 /* Off by default.  When on, the first matmul of each distinct problem (sizes, strides,
  * transposes, batch) times every kernel the BLAS offers for it on the caller's operands
  * and later calls of that problem use the fastest; the library's own pick is a heuristic

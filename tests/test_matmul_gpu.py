@@ -168,3 +168,73 @@ def test_few_rows_against_a_weight_matrix_take_the_streaming_kernel(m, n, k):
     # bit-reproducible
     got2 = _run(a, b, np.float16)
     assert np.array_equal(got, got2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(32, 2304, 768), (32, 3072, 768), (32, 768, 3072), (3, 16, 256),
+                                   (17, 776, 1024)])
+def test_decode_linear_prologues(m, n, k):
+    """deers_rocm_decode_linear: the weightless RMSNorm of src/nn.rs:244-251 and the MLP's
+    relu(x)^2 (src/models/gpt.rs:196-203) folded into the few-rows product.  relu_sq gives the
+    bits of relu_sq_fwd followed by matmul; rms_norm skips the f16 rounding of the normalised
+    row, so it is compared with the f64 evaluation at the f16 tolerance; both with and without
+    the addend."""
+    rng = np.random.default_rng(m + 3 * n + 5 * k)
+    x = (rng.standard_normal((m, k)) * 1.7).astype(np.float16)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float16)
+    y0 = rng.standard_normal((m, n)).astype(np.float16)
+    eps = 1e-5
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    dx, dw = rocm.DeviceBuffer.from_numpy(x), rocm.DeviceBuffer.from_numpy(w)
+
+    def run(prologue, accumulate):
+        dy = rocm.DeviceBuffer.from_numpy(y0.copy())
+        rocm.decode_linear_raw(np.float16, prologue, eps, dx.ptr, k, dw.ptr, n, dy.ptr, accumulate, m, n, k)
+        return dy.numpy()
+
+    # rms_norm: row factor from the definition
+    inv = 1.0 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps)
+    want = (x64 * inv) @ w64
+    for acc in (False, True):
+        ref = want + (y0.astype(np.float64) if acc else 0.0)
+        got = run("rms_norm", acc).astype(np.float64)
+        assert np.abs(got - ref).max() <= 4e-3 * max(1.0, np.abs(ref).max()), acc
+    # relu_sq: same bits as the two separate entry points
+    r = rocm.DeviceBuffer((m, k), np.float16)
+    rocm.relu_sq_fwd_raw(np.float16, dx.ptr, r.ptr, m * k)
+    sep = rocm.DeviceBuffer((m, n), np.float16)
+    rocm.matmul_raw(np.float16, r.ptr, (k, 1, m * k), dw.ptr, (n, 1, k * n), sep.ptr, 1, m, n, k)
+    assert np.array_equal(run("relu_sq", False), sep.numpy())
+    want_r = (np.maximum(x.astype(np.float32), 0) ** 2).astype(np.float16).astype(np.float64) @ w64
+    got = run("relu_sq", True).astype(np.float64)
+    ref = want_r + y0.astype(np.float64)
+    assert np.abs(got - ref).max() <= 4e-3 * max(1.0, np.abs(ref).max())
+    # the packed weight layout [n/32][k][32] gives the same bits as the row-major one
+    if n % 32 == 0:
+        tiles = np.ascontiguousarray(w.reshape(k, n // 32, 32).transpose(1, 0, 2))
+        dt_ = rocm.DeviceBuffer.from_numpy(tiles)
+        for prologue in ("plain", "rms_norm", "relu_sq"):
+            dy = rocm.DeviceBuffer.from_numpy(y0.copy())
+            rocm.decode_linear_raw(np.float16, prologue, eps, dx.ptr, k, dt_.ptr, rocm.LINEAR_W_PACKED, dy.ptr,
+                                   True, m, n, k)
+            assert np.array_equal(dy.numpy(), run(prologue, True)), prologue
+        # and copy_view with the documented strides is the packing
+        packed = rocm.DeviceBuffer((n // 32, k, 32), np.float16)
+        rocm.copy_view_raw(np.float16, dw.ptr, (32, n, 1), packed.ptr, (32 * k, 32, 1), (n // 32, k, 32))
+        assert np.array_equal(packed.numpy(), tiles)
+    # plain = deers_rocm_matmul on the same operands
+    plain = rocm.DeviceBuffer((m, n), np.float16)
+    rocm.matmul_raw(np.float16, dx.ptr, (k, 1, m * k), dw.ptr, (n, 1, k * n), plain.ptr, 1, m, n, k)
+    assert np.array_equal(run("plain", False), plain.numpy())
+
+
+@pytest.mark.gpu
+def test_decode_linear_rejects_what_the_kernel_does_not_take():
+    x = rocm.DeviceBuffer((40, 512), np.float16)
+    w = rocm.DeviceBuffer((512, 64), np.float16)
+    y = rocm.DeviceBuffer((40, 64), np.float16)
+    for m, n, k in ((40, 64, 512), (8, 60, 512), (8, 64, 384)):
+        with pytest.raises(rocm.RocmError):
+            rocm.decode_linear_raw(np.float16, "plain", 0.0, x.ptr, 512, w.ptr, 64, y.ptr, False, m, n, k)
+    with pytest.raises(rocm.RocmError):
+        rocm.decode_linear_raw(np.float32, "plain", 0.0, x.ptr, 512, w.ptr, 64, y.ptr, False, 8, 64, 512)

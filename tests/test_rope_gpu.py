@@ -186,3 +186,47 @@ def test_decode_qkv_is_two_ropes_and_a_copy_in_one_launch(dtype, B, H, D):
     with pytest.raises(rocm.RocmError):
         rocm.decode_qkv_raw(dtype, at(dqkv, 1), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
                             q1.ptr, k1.ptr, v1.ptr, kv_strides, pos, cap, B, H, D)   # misaligned q
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,D,cap,pos", [(2, 3, 64, 11, 7), (1, 2, 64, 5, 0), (3, 2, 128, 300, 299),
+                                           (32, 12, 64, 700, 650), (1, 1, 64, 2100, 2000)])
+def test_attn_decode_append_is_decode_qkv_then_attn_decode(B, H, D, cap, pos):
+    """deers_rocm_attn_decode_append against the two launches it replaces: the caches end up
+    bit-identical (same rotation arithmetic), the attention output agrees to the rounding of the
+    f32 softmax sums (the new row is merged last instead of in stream order) and with the oracle
+    on the same rows.  pos = 0 is the empty cache; the last case splits a head over workgroups."""
+    import ctypes
+    dtype = np.float16
+    C = H * D
+    _, _, cos, sin = _inputs(1, cap, 1, D, dtype, 37)           # tables [cap, D/2]
+    qkv = synth.normal((B, 3 * C), synth.tensor_seed(37 + pos, "append", "qkv"), 1.0).astype(dtype)
+    kc0 = synth.normal((B, H, cap, D), synth.tensor_seed(37 + pos, "append", "kc"), 1.0).astype(dtype)
+    vc0 = synth.normal((B, H, cap, D), synth.tensor_seed(37 + pos, "append", "vc"), 1.0).astype(dtype)
+    dqkv, dc, ds = (rocm.DeviceBuffer.from_numpy(a) for a in (qkv, cos, sin))
+    at = lambda buf, elems: ctypes.c_void_p(buf.ptr.value + elems * 2)
+    cos_row, sin_row = at(dc, pos * (D // 2)), at(ds, pos * (D // 2))
+    kv_strides = (H * cap * D, cap * D, D)
+    scale = rocm.default_scale(D)
+    # one launch
+    k1, v1 = rocm.DeviceBuffer.from_numpy(kc0), rocm.DeviceBuffer.from_numpy(vc0)
+    o1 = rocm.DeviceBuffer((B, H, D), dtype)
+    rocm.attn_decode_append_raw(dtype, at(dqkv, 0), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                                k1.ptr, v1.ptr, kv_strides, o1.ptr, pos, cap, B, H, D, scale)
+    # two launches
+    k2, v2 = rocm.DeviceBuffer.from_numpy(kc0), rocm.DeviceBuffer.from_numpy(vc0)
+    q2, o2 = rocm.DeviceBuffer((B, H, D), dtype), rocm.DeviceBuffer((B, H, D), dtype)
+    rocm.decode_qkv_raw(dtype, at(dqkv, 0), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                        q2.ptr, k2.ptr, v2.ptr, kv_strides, pos, cap, B, H, D)
+    rocm.attn_decode_raw(dtype, q2.ptr, k2.ptr, v2.ptr, o2.ptr, B, H, pos + 1, D, scale, kv_strides=kv_strides)
+    assert np.array_equal(k1.numpy(), k2.numpy())
+    assert np.array_equal(v1.numpy(), v2.numpy())
+    a, b = o1.numpy().astype(np.float32), o2.numpy().astype(np.float32)
+    assert np.abs(a - b).max() <= 2e-3
+    # the oracle on the rows the kernel saw
+    kk, vv, qq = k2.numpy()[:, :, :pos + 1], v2.numpy()[:, :, :pos + 1], q2.numpy()
+    want = oracle.attn_fwd(qq[:, :, None].astype(np.float32), kk.astype(np.float32), vv.astype(np.float32))[:, :, 0]
+    assert np.abs(a - want).max() <= 5e-3
+    with pytest.raises(rocm.RocmError):
+        rocm.attn_decode_append_raw(dtype, at(dqkv, 0), at(dqkv, C), at(dqkv, 2 * C), (3 * C, D), cos_row, sin_row,
+                                    k1.ptr, v1.ptr, kv_strides, o1.ptr, cap, cap, B, H, D, scale)
