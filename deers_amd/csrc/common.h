@@ -245,6 +245,13 @@ struct DecodeParams {
   int64_t in_b, in_h;
 };
 
+// The packed weight ([ceil(n/32)][k][32] f16) of the few-rows product that will follow the
+// one being launched; w == nullptr: none.
+struct SkinnyPrefetch {
+  const void* w = nullptr;
+  int64_t n = 0, k = 0;
+};
+
 // Maps a block id (blockIdx.x, or blockIdx.x minus a multiple of 8) to (head, block
 // rank).  Workgroups are dealt round-robin to the 8 XCDs, so id % 8 is the XCD: every block of one head is given to one XCD
 // (its operands stay in that XCD's L2) and each XCD's list is ordered longest

@@ -41,7 +41,8 @@ int skinny_gemm_splits(int64_t n, int64_t k);
 size_t skinny_gemm_workspace_bytes(int64_t n, int splits);
 void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
                             int m, int n, int k, bool accumulate, int prologue, float eps, bool packed,
-                            int splits, float* partial, int* counters, hipStream_t stream);
+                            int splits, float* partial, int* counters, const SkinnyPrefetch& next,
+                            hipStream_t stream);
 void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* v,
                        const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
                        void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
@@ -110,6 +111,7 @@ struct Runtime {
   // next synchronising call after one of them has been launched
   int* index_flag = nullptr;
   bool index_flag_armed = false;
+  deers::SkinnyPrefetch skinny_next;  // one-shot hint for the next few-rows product (decode_linear_hint)
   int* skinny_counters = nullptr;  // arrival counters of the few-rows GEMM's K splits (all zero between launches)
   // Block cache behind deers_rocm_alloc / _free.  Every kernel and copy of this library
   // runs on `stream`, in order, so a block handed back by free can be handed out again
@@ -1293,9 +1295,11 @@ static int skinny_locked(const void* x, int64_t ldx, const void* w, int64_t ldw,
       HIP_TRY(hipMemsetAsync(g_rt.skinny_counters, 0, kSkinnyCounters * sizeof(int), g_rt.stream));
     }
   }
+  const deers::SkinnyPrefetch next = g_rt.skinny_next;
+  g_rt.skinny_next = deers::SkinnyPrefetch{};  // a hint serves one launch
   deers::LaunchScope scope("matmul", g_rt.stream);
   deers::launch_skinny_gemm_f16(x, ldx, w, ldw, y, n, (int)m, (int)n, (int)k, accumulate, prologue, eps, packed,
-                                splits, (float*)ws, g_rt.skinny_counters, g_rt.stream);
+                                splits, (float*)ws, g_rt.skinny_counters, next, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }
@@ -1338,6 +1342,7 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
   if (dtype == DEERS_ROCM_F16 && batch == 1 && !a_t && !b_t &&
       deers::skinny_gemm_takes(m, n, k, lda, ldb, n, a, b, c))
     return skinny_locked(a, lda, b, ldb, c, m, n, k, accumulate, 0, 0.f, false);
+  g_rt.skinny_next = deers::SkinnyPrefetch{};  // a pending prefetch hint does not outlive this product
   if (!g_rt.blas) {
     if (rocblas_create_handle(&g_rt.blas) != rocblas_status_success)
       return fail(DEERS_ROCM_ERR_HIP, "rocblas_create_handle failed");
@@ -1453,6 +1458,19 @@ int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, 
                 "8 elements and 16-byte aligned pointers (m %lld n %lld k %lld)",
                 (long long)m, (long long)n, (long long)k);
   return skinny_locked(x, ldx, w, ldw, y, m, n, k, accumulate != 0, prologue, eps, packed);
+}
+
+int deers_rocm_decode_linear_hint(const void* next_w_packed, int64_t n, int64_t k) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  g_rt.skinny_next = deers::SkinnyPrefetch{};
+  if (!next_w_packed) return DEERS_ROCM_OK;
+  if (n < 1 || k < 1 || k * 64 > INT32_MAX || (n + 31) / 32 > 65536 || ((uintptr_t)next_w_packed & 15))
+    return fail(DEERS_ROCM_ERR_ARG, "decode_linear_hint: bad shape or unaligned pointer");
+  g_rt.skinny_next.w = next_w_packed;
+  g_rt.skinny_next.n = n;
+  g_rt.skinny_next.k = k;
+  return DEERS_ROCM_OK;
 }
 #pragma clang diagnostic pop
 

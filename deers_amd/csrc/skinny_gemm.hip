@@ -54,9 +54,32 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
                                                               half_t* __restrict__ y, int64_t ldy, int M,
                                                               int N, int K, int S, float* __restrict__ partial,
                                                               int* __restrict__ counters, float eps,
-                                                              int64_t w_block_stride) {
+                                                              int64_t w_block_stride, int main_blocks,
+                                                              const char* __restrict__ next_w,
+                                                              int next_tiles, int next_tile_bytes) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
+  if ((int)blockIdx.x >= main_blocks) {
+    // Prefetch role (workgroups past the product's own, on CUs the product leaves idle):
+    // touch the packed weight of the product that follows, each tile from the XCD whose L2
+    // its consumer will read it through (block id % 8, the same mapping as below), so that
+    // product finds its weights in L2 instead of HBM.  Results are discarded.
+    const int pid = (int)blockIdx.x - main_blocks;  // main_blocks is a multiple of 8
+    const int tile = (pid >> 3) * 8 + (pid & 7);
+    if (tile < next_tiles) {
+      // the same register-free loads as the product's own, all in flight at once; they land
+      // in this wave's LDS ring, where nobody reads them
+      const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
+      const int per_wave = next_tile_bytes / kSkWaves;  // a multiple of 4 KB (K % 256 == 0)
+      const char* src = next_w + (int64_t)tile * next_tile_bytes + (int64_t)pw * per_wave;
+      const uint32_t dst = lds_address(smem) + pw * kSkWaveBytes;
+      for (int i = 0; i < per_wave / 1024; ++i)
+        async_load16_to_lds((const half_t*)(src + i * 1024), (uint32_t)(lane * 16),
+                            dst + (uint32_t)((i % (kSkWaveBytes / 1024)) * 1024));
+      wait_vmcnt<0>();  // the LDS allocation must outlive the writes into it
+    }
+    return;
+  }
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   // block id -> (column block, K split): the S splits of a column block share id % 8
@@ -262,7 +285,7 @@ size_t skinny_gemm_workspace_bytes(int64_t n, int splits) {
 template <bool ACCUMULATE, int PROLOGUE>
 static void launch_one(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy, int m,
                        int n, int k, int splits, float* partial, int* counters, float eps, bool packed,
-                       hipStream_t stream) {
+                       const SkinnyPrefetch& next, hipStream_t stream) {
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
     (void)hipFuncSetAttribute((const void*)skinny_gemm_f16_kernel<ACCUMULATE, PROLOGUE>,
@@ -270,20 +293,24 @@ static void launch_one(const void* x, int64_t ldx, const void* w, int64_t ldw, v
     attr_set = true;
   }
   const int col_blocks = (n + 31) / 32;
-  const dim3 grid((unsigned)(8 * splits * ((col_blocks + 7) / 8)));
+  const int main_blocks = 8 * splits * ((col_blocks + 7) / 8);
+  const int next_tiles = next.w ? (int)((next.n + 31) / 32) : 0;
+  const dim3 grid((unsigned)(main_blocks + 8 * ((next_tiles + 7) / 8)));
   hipLaunchKernelGGL((skinny_gemm_f16_kernel<ACCUMULATE, PROLOGUE>), grid, dim3(256), kSkLds, stream,
                      (const half_t*)x, ldx, (const half_t*)w, packed ? (int64_t)32 : ldw, (half_t*)y, ldy, m, n, k,
-                     splits, partial, counters, eps, packed ? (int64_t)k * 32 : (int64_t)32);
+                     splits, partial, counters, eps, packed ? (int64_t)k * 32 : (int64_t)32, main_blocks,
+                     (const char*)next.w, next_tiles, (int)(next.k * 64));
 }
 
 // prologue: kSkinnyPlain, kSkinnyRmsNorm (splits must be 1) or kSkinnyReluSq; packed: w is
 // [ceil(n/32)][k][32] (each workgroup's columns contiguous) instead of row-major
 void launch_skinny_gemm_f16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
                             int m, int n, int k, bool accumulate, int prologue, float eps, bool packed,
-                            int splits, float* partial, int* counters, hipStream_t stream) {
+                            int splits, float* partial, int* counters, const SkinnyPrefetch& next,
+                            hipStream_t stream) {
 #define DEERS_SKINNY_CASE(ACC, PRO)                                                                      \
   if (accumulate == ACC && prologue == PRO)                                                              \
-    return launch_one<ACC, PRO>(x, ldx, w, ldw, y, ldy, m, n, k, splits, partial, counters, eps, packed, stream);
+    return launch_one<ACC, PRO>(x, ldx, w, ldw, y, ldy, m, n, k, splits, partial, counters, eps, packed, next, stream);
   DEERS_SKINNY_CASE(false, kSkinnyPlain)
   DEERS_SKINNY_CASE(true, kSkinnyPlain)
   DEERS_SKINNY_CASE(false, kSkinnyRmsNorm)

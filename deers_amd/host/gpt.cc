@@ -37,7 +37,7 @@ Tensor MLP::forward(const Tensor& x) const {
 }
 
 void MLP::forward_add_into(const Tensor& x, const Tensor& residual, const double* norm_eps,
-                           KvCache* cache) const {
+                           KvCache* cache, const LinearWeight* after) const {
   NoGradGuard no_grad;
   if (x.layout().ndim() != 3) throw std::logic_error("MLP expects input shape [B, T, C]");
   const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
@@ -57,8 +57,8 @@ void MLP::forward_add_into(const Tensor& x, const Tensor& residual, const double
   }
   const Tensor u = fused_linear(x.reshape({B * T, C}), up,
                                 norm_eps ? LinearPrologue::RmsNorm : LinearPrologue::Plain,
-                                norm_eps ? *norm_eps : 0.0, nullptr);
-  fused_linear(u, down, LinearPrologue::ReluSq, 0.0, &res);
+                                norm_eps ? *norm_eps : 0.0, nullptr, &down);
+  fused_linear(u, down, LinearPrologue::ReluSq, 0.0, &res, after);
 }
 
 Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
@@ -69,13 +69,14 @@ Tensor Block::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) con
   return h.add(mlp_.forward(rms_norm(h, eps_)));
 }
 
-Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const {
+Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,
+                          KvCache* next_cache) const {
   NoGradGuard no_grad;
   // the residual stream is updated in place: both additions ride on the last product of
   // their branch (x_t's storage is overwritten; inference only)
   const Tensor h = x_t.compact();
   attn_.decode_step(h, cache, cos, sin, &h, &eps_);
-  mlp_.forward_add_into(h, h, &eps_, &cache);
+  mlp_.forward_add_into(h, h, &eps_, &cache, next_cache ? &next_cache->step_qkv : nullptr);
   return h;
 }
 
@@ -183,7 +184,8 @@ Tensor GPT::decode_step(const Tensor& idx_t, std::vector<KvCache>& caches) const
   if ((int64_t)caches.size() != config_.n_layer) throw std::logic_error("decode_step: one cache per block");
   const int64_t B = idx_t.shape()[0];
   Tensor x = wte_.forward(idx_t);  // [B, 1, C]
-  for (size_t l = 0; l < blocks_.size(); ++l) x = blocks_[l].decode_step(x, caches[l], cos_, sin_);
+  for (size_t l = 0; l < blocks_.size(); ++l)
+    x = blocks_[l].decode_step(x, caches[l], cos_, sin_, l + 1 < blocks_.size() ? &caches[l + 1] : nullptr);
   x = rms_norm(x, config_.rms_norm_eps);
   return x.reshape({B, config_.n_embd}).matmul(lm_head_).reshape({B, 1, config_.vocab_size});
 }

@@ -34,8 +34,10 @@ class MLP {
   // projection where one launch can do both (a generation step's few rows).
   // `cache`, when given, holds (and at first use receives) the two weights in the layout a
   // generation step streams fastest.
+  // `after`: the weight of the product that follows the down projection (the next block's
+  // packed projection in a generation step), for the prefetch hint.
   void forward_add_into(const Tensor& x, const Tensor& residual, const double* norm_eps = nullptr,
-                        KvCache* cache = nullptr) const;
+                        KvCache* cache = nullptr, const LinearWeight* after = nullptr) const;
   std::vector<Tensor> parameters() const { return {up_, down_}; }
 
  private:
@@ -49,7 +51,10 @@ class Block {
   Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
   // One generated position: x_t [B,1,C] at position cache.len (inference, no autograd).
   // x_t's storage is overwritten with the result when x_t is compact.
-  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin) const;
+  // `next_cache`: the following block's cache (its packed projection is prefetched while this
+  // block's last product runs).
+  Tensor decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,
+                     KvCache* next_cache = nullptr) const;
   // The whole prompt x [B,T,C] into an empty cache (inference); x's storage is overwritten
   // like decode_step's.
   Tensor prefill(const Tensor& x, KvCache& cache, const Tensor& cos, const Tensor& sin) const;

@@ -2,6 +2,7 @@
 #include "ops.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -586,7 +587,7 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   }
   const Tensor qkv = fused_linear(x_flat, cache.step_qkv,
                                   norm_eps ? LinearPrologue::RmsNorm : LinearPrologue::Plain,
-                                  norm_eps ? *norm_eps : 0.0, nullptr);
+                                  norm_eps ? *norm_eps : 0.0, nullptr, &cache.step_out);
   const char* q_data = (const char*)qkv.data();
   const char* k_data = q_data + C * el;
   const char* v_data = q_data + 2 * C * el;
@@ -605,7 +606,7 @@ Tensor CausalSelfAttention::decode_step(const Tensor& x_t, KvCache& cache, const
   cache.len = pos + 1;
   if (residual) {
     const Tensor res = residual->reshape({B, C});
-    fused_linear(o, cache.step_out, LinearPrologue::Plain, 0.0, &res);
+    fused_linear(o, cache.step_out, LinearPrologue::Plain, 0.0, &res, &cache.step_up);
     return *residual;
   }
   return fused_linear(o, cache.step_out, LinearPrologue::Plain, 0.0, nullptr).reshape({B, 1, C});
@@ -631,7 +632,8 @@ Tensor fused_linear(const Tensor& x, const Tensor& w, LinearPrologue f, double e
   return fused_linear(x, lw, f, eps, acc);
 }
 
-Tensor fused_linear(const Tensor& x, const LinearWeight& lw, LinearPrologue f, double eps, const Tensor* acc) {
+Tensor fused_linear(const Tensor& x, const LinearWeight& lw, LinearPrologue f, double eps, const Tensor* acc,
+                    const LinearWeight* next) {
   NoGradGuard no_grad;
   const Tensor& w = lw.w;
   if (x.layout().ndim() != 2 || w.layout().ndim() != 2 || x.shape()[1] != w.shape()[0])
@@ -643,6 +645,8 @@ Tensor fused_linear(const Tensor& x, const LinearWeight& lw, LinearPrologue f, d
       x.is_compact() && w.is_compact() && backed(x)) {
     Tensor y = acc ? *acc : empty({M, N}, x.dtype(), true);
     const bool tiled = lw.tiles.defined();
+    if (next && next->tiles.defined())
+      check(deers_rocm_decode_linear_hint(next->tiles.data(), next->w.shape()[1], next->w.shape()[0]));
     check(deers_rocm_decode_linear((int)x.dtype(), (int)f, (float)eps, x.data(), K,
                                    tiled ? lw.tiles.data() : w.data(), tiled ? DEERS_ROCM_LINEAR_W_PACKED : N,
                                    const_cast<void*>(y.data()), acc ? 1 : 0, M, N, K));

@@ -250,7 +250,10 @@ struct LinearWeight {
   Tensor tiles;  // packed copy, or undefined
   static LinearWeight pack(const Tensor& w);
 };
-Tensor fused_linear(const Tensor& x, const LinearWeight& w, LinearPrologue f, double eps, const Tensor* acc);
+// `next`: the weight of the product that follows this one, if known; its tiles are then
+// pulled into L2 by CUs this launch leaves idle (deers_rocm_decode_linear_hint).
+Tensor fused_linear(const Tensor& x, const LinearWeight& w, LinearPrologue f, double eps, const Tensor* acc,
+                    const LinearWeight* next = nullptr);
 
 struct KvCache {
   Tensor k, v;

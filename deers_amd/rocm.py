@@ -401,6 +401,11 @@ def decode_linear_raw(dtype, prologue, eps, x, ldx, w, ldw, y, accumulate, m, n,
         i64(ldx), w, i64(ldw), y, ctypes.c_int(1 if accumulate else 0), i64(m), i64(n), i64(k)))
 
 
+def decode_linear_hint_raw(next_w_packed, n, k):
+    """deers_rocm_decode_linear_hint: the packed weight of the product after the next one (None clears)."""
+    _check(load().deers_rocm_decode_linear_hint(next_w_packed, ctypes.c_int64(n), ctypes.c_int64(k)))
+
+
 def decode_qkv_raw(dtype, q, k, v, in_strides, cos_row, sin_row, q_out, k_cache, v_cache, cache_strides,
                    pos, capacity, B, H, D):
     """deers_rocm_decode_qkv: rotate q, k at `pos`; q -> q_out [B,H,D]; k, v -> row pos of the caches."""

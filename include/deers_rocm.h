@@ -457,6 +457,15 @@ int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, 
                              const void* w, int64_t ldw, void* y, int accumulate, int64_t m,
                              int64_t n, int64_t k);
 
+/* Optional hint for the NEXT deers_rocm_decode_linear (or few-rows deers_rocm_matmul) launch:
+ * the packed weight (DEERS_ROCM_LINEAR_W_PACKED layout, [ceil(n/32)][k][32] f16) of the product
+ * that will follow it.  Workgroups on CUs that launch leaves idle read that weight once, each
+ * tile through the L2 of the XCD that will consume it, so the following product finds its
+ * weights in L2 instead of HBM.  One-shot: consumed (or dropped) by the next launch; NULL
+ * clears it.  Purely a performance hint: results never depend on it.  No counterpart in the
+ * reference. */
+int deers_rocm_decode_linear_hint(const void* next_w_packed, int64_t n, int64_t k);
+
 /* Off by default.  When on, the first matmul of each distinct problem (sizes, strides,
  * transposes, batch) times every kernel the BLAS offers for it on the caller's operands
  * and later calls of that problem use the fastest; the library's own pick is a heuristic

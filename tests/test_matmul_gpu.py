@@ -1,6 +1,8 @@
 """deers_rocm_matmul (library GEMM behind BackendStorage::matmul) against the CPU oracle's
 gemm_strided restatement and the reference's own integer-valued conformance cases
 (tests/tensor.rs:83-110)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -238,3 +240,36 @@ def test_decode_linear_rejects_what_the_kernel_does_not_take():
             rocm.decode_linear_raw(np.float16, "plain", 0.0, x.ptr, 512, w.ptr, 64, y.ptr, False, m, n, k)
     with pytest.raises(rocm.RocmError):
         rocm.decode_linear_raw(np.float32, "plain", 0.0, x.ptr, 512, w.ptr, 64, y.ptr, False, 8, 64, 512)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,k,n2,k2", [(2304, 768, 768, 768), (768, 3072, 2304, 768), (768, 768, 768, 3072),
+                                       (64, 256, 3072, 768)])
+def test_decode_linear_prefetch_hint_changes_nothing_but_time(n, k, n2, k2):
+    """deers_rocm_decode_linear_hint names the packed weight of the following product; the launch
+    it rides on (split or not) gives the same bits with and without it, the hinted weight is
+    only read, and a hint is used once."""
+    m = 32
+    rng = np.random.default_rng(n + k + n2)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float16)
+    nxt = rng.standard_normal((n2 // 32, k2, 32)).astype(np.float16)
+    dx, dw, dn = (rocm.DeviceBuffer.from_numpy(a) for a in (x, w, nxt))
+    y0 = rng.standard_normal((m, n)).astype(np.float16)
+
+    def run(hint):
+        dy = rocm.DeviceBuffer.from_numpy(y0.copy())
+        if hint:
+            rocm.decode_linear_hint_raw(dn.ptr, n2, k2)
+        rocm.decode_linear_raw(np.float16, "relu_sq", 0.0, dx.ptr, k, dw.ptr, n, dy.ptr, True, m, n, k)
+        return dy.numpy()
+
+    plain = run(False)
+    assert np.array_equal(run(True), plain)
+    assert np.array_equal(run(False), plain)      # the hint did not linger
+    assert np.array_equal(dn.numpy(), nxt)        # and its target is untouched
+    rocm.decode_linear_hint_raw(dn.ptr, n2, k2)
+    rocm.decode_linear_hint_raw(None, 0, 0)       # cleared again
+    assert np.array_equal(run(False), plain)
+    with pytest.raises(rocm.RocmError):
+        rocm.decode_linear_hint_raw(ctypes.c_void_p(dn.ptr.value + 2), n2, k2)   # unaligned
