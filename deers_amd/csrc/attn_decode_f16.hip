@@ -224,17 +224,21 @@ void launch_attn_decode_f16(const DecodeParams& p, int B, int D, bool append, hi
   dim3 grid(p.splits, B * p.H);
   {
     LaunchScope scope(append ? "attn_decode_append_f16" : "attn_decode_f16", stream);
-    if (D == 64) {
-      if (append) hipLaunchKernelGGL((attn_decode_f16_kernel<64, true>), grid, dim3(256), 0, stream, p);
-      else hipLaunchKernelGGL((attn_decode_f16_kernel<64, false>), grid, dim3(256), 0, stream, p);
-    } else {
-      if (append) hipLaunchKernelGGL((attn_decode_f16_kernel<128, true>), grid, dim3(256), 0, stream, p);
-      else hipLaunchKernelGGL((attn_decode_f16_kernel<128, false>), grid, dim3(256), 0, stream, p);
-    }
+#define DEERS_DECODE_CASE(DD, APP) \
+  if (D == DD && append == APP) hipLaunchKernelGGL((attn_decode_f16_kernel<DD, APP>), grid, dim3(256), 0, stream, p);
+    DEERS_DECODE_CASE(32, false)
+    DEERS_DECODE_CASE(32, true)
+    DEERS_DECODE_CASE(64, false)
+    DEERS_DECODE_CASE(64, true)
+    DEERS_DECODE_CASE(128, false)
+    DEERS_DECODE_CASE(128, true)
+#undef DEERS_DECODE_CASE
   }
   if (p.splits > 1) {
     LaunchScope scope("attn_decode_merge", stream);
-    if (D == 64)
+    if (D == 32)
+      hipLaunchKernelGGL(attn_decode_merge_kernel<32>, dim3(B * p.H), dim3(32), 0, stream, p);
+    else if (D == 64)
       hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(B * p.H), dim3(64), 0, stream, p);
     else
       hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(B * p.H), dim3(128), 0, stream, p);

@@ -632,8 +632,8 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
     return fail(DEERS_ROCM_ERR_ARG, "attn_decode: only DEERS_ROCM_F16 caches are supported");
   if (B < 1 || H < 1 || L < 1 || B * H > 65535 || L > (int64_t(1) << 30))
     return fail(DEERS_ROCM_ERR_ARG, "attn_decode: need B,H,L >= 1, B*H <= 65535, L <= 2^30");
-  if (D != 64 && D != 128)
-    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: head dim %lld unsupported (64 or 128)",
+  if (D != 32 && D != 64 && D != 128)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: head dim %lld unsupported (32, 64 or 128)",
                 (long long)D);
   if (!q || !k_cache || !v_cache || !o) return fail(DEERS_ROCM_ERR_ARG, "attn_decode: null pointer");
   if (int rc = check_scale(scale)) return rc;
@@ -674,8 +674,8 @@ int deers_rocm_attn_decode_append(int dtype, const void* q, const void* k, const
   if (pos < 0 || pos >= capacity)
     return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: position %lld outside the cache capacity %lld",
                 (long long)pos, (long long)capacity);
-  if (D != 64 && D != 128)
-    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: head dim %lld unsupported (64 or 128)", (long long)D);
+  if (D != 32 && D != 64 && D != 128)
+    return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: head dim %lld unsupported (32, 64 or 128)", (long long)D);
   if (!q || !k || !v || !in_strides || !cos_row || !sin_row || !k_cache || !v_cache || !cache_strides || !o)
     return fail(DEERS_ROCM_ERR_ARG, "attn_decode_append: null pointer");
   if (int rc = check_scale(scale)) return rc;

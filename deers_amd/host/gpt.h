@@ -87,7 +87,7 @@ class GPT {
   Tensor forward(const Tensor& idx) const;  // I64 [B,T] -> logits [B,T,V]
   std::vector<Tensor> parameters() const;
 
-  // Generation with a KV cache per block (f16 models; head width 64 or 128).  The
+  // Generation with a KV cache per block (f16 models; head width 32, 64 or 128).  The
   // reference has no cache: its sampling loop re-runs the whole window for every new
   // token (examples/tinystories_train.rs:250-276).  Here each token costs one pass over
   // the weights and one streaming pass over the cached keys and values.

@@ -168,7 +168,7 @@ int deers_rocm_attn_bwd(int dtype,
  * (examples/tinystories_train.rs:250-276).
  * q,o: [B,H,D] compact.  k_cache,v_cache: [B,H,L_cap,D] with element strides
  * `kv_strides` = {b,h,l} (NULL: compact with L_cap = L); only rows [0,L) are
- * read.  D in {64,128}. */
+ * read.  D in {32,64,128}. */
 int deers_rocm_attn_decode(int dtype,
                            const void* q,
                            const void* k_cache, const void* v_cache,
@@ -183,7 +183,7 @@ int deers_rocm_attn_decode(int dtype,
  * v become row `pos` of the caches ([B,H,capacity,D] by cache_strides = {b, h, t}; rows
  * [0,pos) hold the earlier tokens) and o [B,H,D] (compact) is the attention of the rotated q
  * over rows [0,pos].  Same values as the two separate calls up to the order of the f32
- * softmax sums (the new row is merged last).  D in {64,128}, f16.  The reference has no KV
+ * softmax sums (the new row is merged last).  D in {32,64,128}, f16.  The reference has no KV
  * cache (examples/tinystories_train.rs:250-276 re-runs the window). */
 int deers_rocm_attn_decode_append(int dtype, const void* q, const void* k, const void* v,
                                   const int64_t* in_strides, const void* cos_row,

@@ -186,7 +186,8 @@ def test_strided_head_interleaved_layout():
 
 
 @pytest.mark.parametrize("B,H,L,D", [(1, 1, 1, 64), (2, 3, 77, 64), (3, 2, 1000, 64),
-                                     (2, 2, 4096, 128), (1, 5, 333, 128)])
+                                     (2, 2, 4096, 128), (1, 5, 333, 128), (1, 1, 1, 32), (4, 6, 500, 32),
+                                     (1, 2, 2100, 32)])
 def test_decode_matches_oracle(B, H, L, D):
     name = f"dec-{B}-{H}-{L}-{D}"
     x = synth.attention_inputs(name, B, H, 1, D, np.float16, base_seed=9, kv_len=L,

@@ -285,17 +285,20 @@ def test_host_gpt_training_step_matches_oracle(tmp_path, cfg, B, T):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("T,n_new,seq_len", [(24, 10, 48), (300, 6, 320)])
-def test_host_gpt_generation_with_kv_caches(tmp_path, T, n_new, seq_len):
+@pytest.mark.parametrize("T,n_new,seq_len,C,H", [(24, 10, 48, 128, 2), (300, 6, 320, 128, 2), (40, 8, 64, 192, 6)])
+def test_host_gpt_generation_with_kv_caches(tmp_path, T, n_new, seq_len, C, H):
     """An f16 GPT generating through per-block KV caches: every decode step's logits equal
     the matching row of the full causal forward (device) and the f32 oracle on the same
     f16 weights; a prompt taken through prefill leaves the same logits and caches as its tokens
     one by one; the greedy continuation picks the teacher-forced argmax at every position."""
     from oracle import gpt as ogpt
     from test_oracle_gpt import make_weights
-    cfg = dict(vocab_size=300, sequence_len=seq_len, n_layer=2, n_head=2, n_embd=128, mlp_hidden_dim=256,
+    cfg = dict(vocab_size=300, sequence_len=seq_len, n_layer=2, n_head=H, n_embd=C, mlp_hidden_dim=2 * C,
                rms_norm_eps=1e-5, rope_base=10000.0)
-    B = 3   # T = 300: the prefilled half spans two 128-row tiles of the fused forward
+    # T = 300: the prefilled half spans two 128-row tiles of the fused forward; C = 192 with 6
+    # heads is the width of the reference's TinyStories model (head width 32; its products do
+    # not fit the few-rows kernel and take the separate norm / GEMM / activation launches)
+    B = 3
     rng = np.random.default_rng(23)
     ids = rng.integers(0, cfg["vocab_size"], (B, T)).astype(np.int64)
     w = [a.astype(np.float16) for a in make_weights(cfg, 29, dtype=np.float32)]

@@ -190,7 +190,8 @@ def test_decode_qkv_is_two_ropes_and_a_copy_in_one_launch(dtype, B, H, D):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,H,D,cap,pos", [(2, 3, 64, 11, 7), (1, 2, 64, 5, 0), (3, 2, 128, 300, 299),
-                                           (32, 12, 64, 700, 650), (1, 1, 64, 2100, 2000)])
+                                           (32, 12, 64, 700, 650), (1, 1, 64, 2100, 2000),
+                                           (4, 6, 32, 40, 17), (1, 1, 32, 2100, 2000)])
 def test_attn_decode_append_is_decode_qkv_then_attn_decode(B, H, D, cap, pos):
     """deers_rocm_attn_decode_append against the two launches it replaces: the caches end up
     bit-identical (same rotation arithmetic), the attention output agrees to the rounding of the
