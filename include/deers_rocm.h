@@ -462,7 +462,9 @@ int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, 
  * that will follow it.  Workgroups on CUs that launch leaves idle read that weight once, each
  * tile through the L2 of the XCD that will consume it, so the following product finds its
  * weights in L2 instead of HBM.  One-shot: consumed (or dropped) by the next launch; NULL
- * clears it.  Purely a performance hint: results never depend on it.  No counterpart in the
+ * clears it.  Purely a performance hint: results never depend on it, but the hinted buffer is
+ * read by that launch, so it must stay allocated until the launch has run (threads that
+ * share the library should pair hint and launch under their own lock).  No counterpart in the
  * reference. */
 int deers_rocm_decode_linear_hint(const void* next_w_packed, int64_t n, int64_t k);
 
