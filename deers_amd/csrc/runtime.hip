@@ -1465,7 +1465,8 @@ int deers_rocm_decode_linear_hint(const void* next_w_packed, int64_t n, int64_t 
   NEED_INIT();
   g_rt.skinny_next = deers::SkinnyPrefetch{};
   if (!next_w_packed) return DEERS_ROCM_OK;
-  if (n < 1 || k < 1 || k * 64 > INT32_MAX || (n + 31) / 32 > 65536 || ((uintptr_t)next_w_packed & 15))
+  if (n < 1 || k < 256 || k % 256 || k * 64 > INT32_MAX || (n + 31) / 32 * (k / 256) > 65536 ||
+      ((uintptr_t)next_w_packed & 15))
     return fail(DEERS_ROCM_ERR_ARG, "decode_linear_hint: bad shape or unaligned pointer");
   g_rt.skinny_next.w = next_w_packed;
   g_rt.skinny_next.n = n;

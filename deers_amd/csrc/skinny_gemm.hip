@@ -47,6 +47,7 @@ constexpr int kSkStepBytes = 2048;            // W tile [16 k x 32 n] + x tile [
 constexpr int kSkChunkBytes = kSkStepsPerChunk * kSkStepBytes;
 constexpr int kSkWaveBytes = kSkRing * kSkChunkBytes;
 constexpr int kSkLds = kSkWaves * kSkWaveBytes;  // 96 KB
+constexpr int kSkPieceBytes = 256 * 64;          // prefetch unit: 256 rows of a packed tile
 
 template <bool ACCUMULATE, int PROLOGUE>
 __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __restrict__ x, int64_t ldx,
@@ -64,14 +65,19 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(const half_t* __re
     // touch the packed weight of the product that follows, each tile from the XCD whose L2
     // its consumer will read it through (block id % 8, the same mapping as below), so that
     // product finds its weights in L2 instead of HBM.  Results are discarded.
+    // A tile of K rows (64 bytes each) is cut into pieces of 256 rows, one workgroup each,
+    // so that a long K does not make the prefetch outlast the product it rides on.
     const int pid = (int)blockIdx.x - main_blocks;  // main_blocks is a multiple of 8
-    const int tile = (pid >> 3) * 8 + (pid & 7);
+    const int pieces = next_tile_bytes / kSkPieceBytes;
+    const int q = pid >> 3;
+    const int tile = (q / pieces) * 8 + (pid & 7), piece = q % pieces;
     if (tile < next_tiles) {
       // the same register-free loads as the product's own, all in flight at once; they land
       // in this wave's LDS ring, where nobody reads them
       const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
-      const int per_wave = next_tile_bytes / kSkWaves;  // a multiple of 4 KB (K % 256 == 0)
-      const char* src = next_w + (int64_t)tile * next_tile_bytes + (int64_t)pw * per_wave;
+      const int per_wave = kSkPieceBytes / kSkWaves;  // 4 KB
+      const char* src = next_w + (int64_t)tile * next_tile_bytes + (int64_t)piece * kSkPieceBytes +
+                        (int64_t)pw * per_wave;
       const uint32_t dst = lds_address(smem) + pw * kSkWaveBytes;
       for (int i = 0; i < per_wave / 1024; ++i)
         async_load16_to_lds((const half_t*)(src + i * 1024), (uint32_t)(lane * 16),
@@ -295,7 +301,8 @@ static void launch_one(const void* x, int64_t ldx, const void* w, int64_t ldw, v
   const int col_blocks = (n + 31) / 32;
   const int main_blocks = 8 * splits * ((col_blocks + 7) / 8);
   const int next_tiles = next.w ? (int)((next.n + 31) / 32) : 0;
-  const dim3 grid((unsigned)(main_blocks + 8 * ((next_tiles + 7) / 8)));
+  const int pieces = next.w ? (int)(next.k / 256) : 0;  // K % 256 == 0 for every weight the kernel takes
+  const dim3 grid((unsigned)(main_blocks + 8 * ((next_tiles + 7) / 8) * pieces));
   hipLaunchKernelGGL((skinny_gemm_f16_kernel<ACCUMULATE, PROLOGUE>), grid, dim3(256), kSkLds, stream,
                      (const half_t*)x, ldx, (const half_t*)w, packed ? (int64_t)32 : ldw, (half_t*)y, ldy, m, n, k,
                      splits, partial, counters, eps, packed ? (int64_t)k * 32 : (int64_t)32, main_blocks,
