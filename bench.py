@@ -88,7 +88,17 @@ def bench_train(steps: int, warmup: int, only: str = "all"):
     prof = rocm.profile_collect()
     rocm.profile_enable(False)
     kernels = {n: {"calls": c, "avg_us": 1e3 * ms / c} for n, (c, ms) in prof.items()}
-    return dict(wall_ms=wall_ms, dev_ms=dev_ms, kernels=kernels)
+
+    # third pass: every step between its own pair of events (median and minimum of a step)
+    timers = [rocm.Timer() for _ in range(steps)]
+    for t in timers:
+        t.start()
+        step()
+        t.stop()
+    rocm.sync()
+    per_step = sorted(1e3 * t.elapsed_ms() for t in timers)
+    step_us = {"median": per_step[len(per_step) // 2], "min": per_step[0]}
+    return dict(wall_ms=wall_ms, dev_ms=dev_ms, kernels=kernels, step_us=step_us)
 
 
 def bench_decode(steps: int, warmup: int, rotate: int = 4):
@@ -531,6 +541,7 @@ def main():
         "frac_mfma_peak": tflops / PEAK_F16_TFLOPS,
         "peak_tflops_f16_dense": PEAK_F16_TFLOPS,
         "wall_ms_per_step": tr["wall_ms"] / args.steps,
+        "step_us_event_pairs": tr["step_us"],
         "kernels": kern,
         "roofline": roofline,
         "decode": {"workload": "decode f16 B=32 H=12 L=4096 D=64 (BASELINE configs[3]), "
