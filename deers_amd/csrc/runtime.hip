@@ -130,6 +130,15 @@ struct Runtime {
 
 Runtime g_rt;
 std::mutex g_mu;
+
+// Device memory that exists without any allocation call: the split partials of
+// deers_rocm_attn_decode_noalloc live here.  Each GPU the library is loaded on holds its
+// own copy until the process ends.  The name below is only a host-side handle: host code
+// uses the address hipGetSymbolAddress returns for the current device (g_scratch_ptr,
+// resolved once in deers_rocm_init), never the name itself.
+constexpr size_t kScratchBytes = 512 * 1024;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+void* g_scratch_ptr = nullptr;  // device address of `scratch` on g_rt.ordinal
 thread_local std::string t_err;
 
 int fail(int code, const char* fmt, ...) {
@@ -308,6 +317,7 @@ int deers_rocm_init(int ordinal) {
                 ordinal);
   HIP_TRY(hipSetDevice(ordinal));
   HIP_TRY(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
+  HIP_TRY(hipGetSymbolAddress(&g_scratch_ptr, HIP_SYMBOL(scratch)));
   g_rt.ordinal = ordinal;
   g_rt.ready = true;
   return DEERS_ROCM_OK;
@@ -623,19 +633,20 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   return DEERS_ROCM_OK;
 }
 
-int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
-                           const int64_t* kv_strides, void* o, int64_t B, int64_t H, int64_t L,
-                           int64_t D, float scale) {
-  std::lock_guard<std::mutex> lock(g_mu);
+// Argument checks and launch shared by deers_rocm_attn_decode (partials in the growing
+// workspace) and deers_rocm_attn_decode_noalloc (partials in the static scratch array).
+static int attn_decode_impl(const char* what, bool no_alloc, int dtype, const void* q,
+                            const void* k_cache, const void* v_cache, const int64_t* kv_strides,
+                            void* o, int64_t B, int64_t H, int64_t L, int64_t D, float scale) {
   NEED_INIT();
   if (dtype != DEERS_ROCM_F16)
-    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: only DEERS_ROCM_F16 caches are supported");
+    return fail(DEERS_ROCM_ERR_ARG, "%s: only DEERS_ROCM_F16 caches are supported", what);
   if (B < 1 || H < 1 || L < 1 || B * H > 65535 || L > (int64_t(1) << 30))
-    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: need B,H,L >= 1, B*H <= 65535, L <= 2^30");
+    return fail(DEERS_ROCM_ERR_ARG, "%s: need B,H,L >= 1, B*H <= 65535, L <= 2^30", what);
   if (D != 32 && D != 64 && D != 128)
-    return fail(DEERS_ROCM_ERR_ARG, "attn_decode: head dim %lld unsupported (32, 64 or 128)",
+    return fail(DEERS_ROCM_ERR_ARG, "%s: head dim %lld unsupported (32, 64 or 128)", what,
                 (long long)D);
-  if (!q || !k_cache || !v_cache || !o) return fail(DEERS_ROCM_ERR_ARG, "attn_decode: null pointer");
+  if (!q || !k_cache || !v_cache || !o) return fail(DEERS_ROCM_ERR_ARG, "%s: null pointer", what);
   if (int rc = check_scale(scale)) return rc;
   deers::DecodeParams p{};
   p.skb = H * L * D; p.skh = L * D; p.skl = D;
@@ -643,13 +654,23 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
   if (p.skb % 8 || p.skh % 8 || p.skl % 8 || (reinterpret_cast<uintptr_t>(k_cache) & 15) ||
       (reinterpret_cast<uintptr_t>(v_cache) & 15) || (reinterpret_cast<uintptr_t>(q) & 15) ||
       (reinterpret_cast<uintptr_t>(o) & 15))
-    return fail(DEERS_ROCM_ERR_LAYOUT, "attn_decode: cache rows, q and o must be 16-byte aligned");
+    return fail(DEERS_ROCM_ERR_LAYOUT, "%s: cache rows, q and o must be 16-byte aligned", what);
   int chunk = 0;
   const int splits = deers::decode_pick_splits(B * H, L, &chunk);
   void* ws = nullptr;
   const size_t part_o = (size_t)(B * H) * splits * D * sizeof(float);
   const size_t part_ml = (size_t)(B * H) * splits * 2 * sizeof(float);
-  if (int rc = workspace(part_o + part_ml, &ws)) return rc;
+  if (no_alloc) {
+    // a head that is not split writes its output itself and touches no scratch
+    if (splits > 1 && part_o + part_ml > kScratchBytes)
+      return fail(DEERS_ROCM_ERR_ARG,
+                  "%s: the split partials of this problem need %zu bytes, the static scratch "
+                  "holds %zu; use deers_rocm_attn_decode",
+                  what, part_o + part_ml, kScratchBytes);
+    ws = g_scratch_ptr;
+  } else {
+    if (int rc = workspace(part_o + part_ml, &ws)) return rc;
+  }
   p.q = q; p.k = k_cache; p.v = v_cache; p.o = o;
   p.part_o = static_cast<float*>(ws);
   p.part_ml = reinterpret_cast<float*>(static_cast<char*>(ws) + part_o);
@@ -658,6 +679,25 @@ int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const 
   deers::launch_attn_decode_f16(p, (int)B, (int)D, false, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
+}
+
+int deers_rocm_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                           const int64_t* kv_strides, void* o, int64_t B, int64_t H, int64_t L,
+                           int64_t D, float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return attn_decode_impl("attn_decode", false, dtype, q, k_cache, v_cache, kv_strides, o, B, H, L,
+                          D, scale);
+}
+
+// The same kernels with the split partials in the file-scope `scratch` array: no
+// hipMalloc / hipFree on any path.  Every split slot that the merge kernel reads is
+// written by the main kernel of the same call first, so nothing needs clearing.
+int deers_rocm_attn_decode_noalloc(int dtype, const void* q, const void* k_cache,
+                                   const void* v_cache, const int64_t* kv_strides, void* o,
+                                   int64_t B, int64_t H, int64_t L, int64_t D, float scale) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return attn_decode_impl("attn_decode_noalloc", true, dtype, q, k_cache, v_cache, kv_strides, o,
+                          B, H, L, D, scale);
 }
 
 int deers_rocm_attn_decode_append(int dtype, const void* q, const void* k, const void* v,

@@ -193,6 +193,14 @@ def attn_decode_raw(dtype, q, k_cache, v_cache, o, B, H, L, D, scale, kv_strides
         ctypes.c_int64(H), ctypes.c_int64(L), ctypes.c_int64(D), ctypes.c_float(scale)))
 
 
+def attn_decode_noalloc_raw(dtype, q, k_cache, v_cache, o, B, H, L, D, scale, kv_strides=None):
+    """deers_rocm_attn_decode_noalloc: attn_decode with the split partials in static device memory."""
+    ks = None if kv_strides is None else (ctypes.c_int64 * 3)(*[int(x) for x in kv_strides])
+    _check(load().deers_rocm_attn_decode_noalloc(
+        ctypes.c_int(dtype_code(dtype)), q, k_cache, v_cache, ks, o, ctypes.c_int64(B),
+        ctypes.c_int64(H), ctypes.c_int64(L), ctypes.c_int64(D), ctypes.c_float(scale)))
+
+
 def attn_decode_append_raw(dtype, q, k, v, in_strides, cos_row, sin_row, k_cache, v_cache, cache_strides,
                            o, pos, capacity, B, H, D, scale):
     """deers_rocm_attn_decode_append: rotate q, k at `pos`, append k, v as cache row pos, attend over [0,pos]."""

@@ -176,6 +176,23 @@ int deers_rocm_attn_decode(int dtype,
                            void* o,
                            int64_t B, int64_t H, int64_t L, int64_t D, float scale);
 
+/* deers_rocm_attn_decode for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical results;
+ * the split partial results live in a fixed 512 KiB device array that is part of the
+ * library image, so the call performs no hipMalloc / hipFree and never grows a
+ * workspace.  A problem whose partials (B*H*splits*(D+2) floats, only when heads are
+ * split over workgroups, i.e. B*H < 256) would not fit is rejected with
+ * DEERS_ROCM_ERR_ARG.  All calls on a device share the one array: calls that overlap
+ * on the device (other streams, other processes' copies aside) would race; the library
+ * stream runs them in order. */
+int deers_rocm_attn_decode_noalloc(int dtype,
+                                   const void* q,
+                                   const void* k_cache, const void* v_cache,
+                                   const int64_t* kv_strides,
+                                   void* o,
+                                   int64_t B, int64_t H, int64_t L, int64_t D, float scale);
+
 /* One generation step of the attention core in one launch: deers_rocm_decode_qkv followed by
  * deers_rocm_attn_decode.  q, k, v are the new token's projections [B,H,D] by element strides
  * in_strides = {b, h} (D stride 1); q and k are rotated at the token's position (cos_row /
