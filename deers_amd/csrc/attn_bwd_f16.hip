@@ -43,10 +43,6 @@ constexpr int kBwdStep = 64;  // rows of the streamed operand per iteration
 
 #define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
-// Hook for a timestamp-tracing build of these kernels; expands to nothing in the library.
-#ifndef DEERS_TRACE_POINT
-#define DEERS_TRACE_POINT(slot)
-#endif
 
 template <int D>
 struct BwdCfg {
@@ -100,8 +96,6 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
   half_t* dV = (half_t*)p.dv + b * p.sdv.b + h * p.sdv.h;
   const float* lse2 = p.lse2 + (int64_t)bh * p.t_pad;
   const float* negdelta = p.negdelta + (int64_t)bh * p.t_pad;
-
-  DEERS_TRACE_POINT(0);
   const int kv0 = kvblk * kBwdBlk;
   const int kvw0 = kv0 + 32 * wave;
   const int kvrow = kvw0 + (lane & 31);
@@ -131,10 +125,16 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     if (qb <= ready_upto) return;
     const int* flag = p.ready + (int64_t)bh * n_blocks + qb;
     // Bounded: a producer cannot be held up by this workgroup (it was dispatched
-    // earlier and waits for nothing), so the bound is never reached in practice; it
-    // only guarantees that every wave leaves the loop.
-    for (int spins = 0; spins < (1 << 20); ++spins) {
-      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) break;
+    // earlier and waits for nothing), so the bound is not reached in practice; it
+    // guarantees that every wave leaves the loop.  A wait that does run out raises the
+    // error word in front of the flags (the statistics it then reads are not valid and
+    // this call's dK / dV are wrong): the host reports it at the next synchronisation.
+    int spins = 0;
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
+      if (++spins >= p.spin_limit) {
+        __hip_atomic_store(p.ready - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
       __builtin_amdgcn_s_sleep(8);
     }
     ready_upto = qb;
@@ -278,7 +278,6 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
       else
         block(no, slot, mb, qb0);
     }
-    DEERS_TRACE_POINT(2 + j - first_tile);
   }
 
   if (kvrow < T) {
@@ -290,7 +289,6 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
       store_block_f16(dvrow + 32 * db, dvacc[db], 1.f, g);
     }
   }
-  DEERS_TRACE_POINT(30);
 }
 
 // ---------------------------------------------------------------------------
@@ -327,8 +325,6 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
   const half_t* V = (const half_t*)p.v + b * p.sv.b + h * p.sv.h;
   const half_t* dO = (const half_t*)p.d_o + b * p.sdo.b + h * p.sdo.h;
   half_t* dQ = (half_t*)p.dq + b * p.sdq.b + h * p.sdq.h;
-
-  DEERS_TRACE_POINT(0);
   const int q0 = qtile * kBwdBlk;
   const int qw0 = q0 + 32 * wave;
   const int qrow = qw0 + (lane & 31);
@@ -485,7 +481,6 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
       else
         block(no, slot, mb, kvb0);
     }
-    DEERS_TRACE_POINT(2 + j);
   }
 
   if (qrow < T) {
@@ -493,7 +488,6 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
 #pragma unroll
     for (int db = 0; db < DB; ++db) store_block_f16(dqrow + 32 * db, dqacc[db], p.scale, g);
   }
-  DEERS_TRACE_POINT(30);
 }
 
 // One launch for the whole backward: the first half of the grid runs the dQ role, the
@@ -504,23 +498,33 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
 // flag before they first touch a query block's statistics.  Against two launches
 // this saves a dispatch and lets the heavy dK/dV blocks start while the light dQ
 // blocks drain.
+//
+// `first_id` is added to blockIdx.x: 0 with a grid of both halves is the single launch;
+// a grid of one half with first_id = 0, then one with first_id = the half's length, runs
+// the two roles as two launches in stream order (the flags are then already set when the
+// second launch starts).  The hand-over inside one launch stores the statistics, drains
+// the stores (vmcnt 0) and sets the flag with relaxed atomics and no cache write-back,
+// which is only enough when producer and consumer share one L2, i.e. one XCD: the host
+// takes the single launch only on a device where workgroup id % 8 is known to be the XCD.
 template <int D>
 __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(BwdParams p, int BH,
                                                               int n_blocks,
-                                                              int heads_per_xcd) {
+                                                              int heads_per_xcd,
+                                                              int first_id) {
   const int per_role = 8 * n_blocks * heads_per_xcd;
-  if ((int)blockIdx.x < per_role)
-    bwd_dq_f16_body<D>(p, BH, n_blocks, heads_per_xcd, blockIdx.x);
+  const int id = (int)blockIdx.x + first_id;
+  if (id < per_role)
+    bwd_dq_f16_body<D>(p, BH, n_blocks, heads_per_xcd, id);
   else
-    bwd_dkdv_f16_body<D>(p, BH, n_blocks, heads_per_xcd, blockIdx.x - per_role);
+    bwd_dkdv_f16_body<D>(p, BH, n_blocks, heads_per_xcd, id - per_role);
 }
 
 template <int D>
-static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
+static void launch_bwd_f16_d(const BwdParams& p, int B, int mode, hipStream_t stream) {
   const int BH = B * p.H;
   const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
   const int heads_per_xcd = (BH + 7) / 8;
-  const dim3 grid(2 * 8 * n_blocks * heads_per_xcd);
+  const int per_role = 8 * n_blocks * heads_per_xcd;
   constexpr size_t lds = BwdCfg<D>::kLdsDkdv > BwdCfg<D>::kLdsDq ? BwdCfg<D>::kLdsDkdv : BwdCfg<D>::kLdsDq;
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
@@ -529,16 +533,38 @@ static void launch_bwd_f16_d(const BwdParams& p, int B, hipStream_t stream) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     attr_set = true;
   }
-  LaunchScope scope("attn_bwd_f16", stream);
-  hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, grid, dim3(256), lds, stream, p, BH, n_blocks,
-                     heads_per_xcd);
+  if (mode == 2) {  // test hook: consumers only, so that their bounded wait runs out
+    LaunchScope scope("attn_bwd_f16_dkdv", stream);
+    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
+                       n_blocks, heads_per_xcd, per_role);
+    return;
+  }
+  if (mode == 1) {
+    LaunchScope scope("attn_bwd_f16", stream);
+    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(2 * per_role), dim3(256), lds, stream, p, BH,
+                       n_blocks, heads_per_xcd, 0);
+    return;
+  }
+  {
+    LaunchScope scope("attn_bwd_f16_dq", stream);
+    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
+                       n_blocks, heads_per_xcd, 0);
+  }
+  {
+    LaunchScope scope("attn_bwd_f16_dkdv", stream);
+    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
+                       n_blocks, heads_per_xcd, per_role);
+  }
 }
 
-void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream) {
+// mode 1: both roles in one grid with the flag hand-over (needs workgroup id % 8 == XCD);
+// mode 0: two launches in stream order; mode 2: only the dK/dV half of the single launch
+// (host-side test of the bounded wait: nobody publishes, every wait runs out).
+void launch_attn_bwd_f16(const BwdParams& p, int B, int D, int mode, hipStream_t stream) {
   switch (D) {
-    case 32: launch_bwd_f16_d<32>(p, B, stream); break;
-    case 64: launch_bwd_f16_d<64>(p, B, stream); break;
-    case 128: launch_bwd_f16_d<128>(p, B, stream); break;
+    case 32: launch_bwd_f16_d<32>(p, B, mode, stream); break;
+    case 64: launch_bwd_f16_d<64>(p, B, mode, stream); break;
+    case 128: launch_bwd_f16_d<128>(p, B, mode, stream); break;
   }
 }
 

@@ -53,10 +53,6 @@ constexpr float kLazyRescale = 8.0f;
 
 #define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
-// Hook for a timestamp-tracing build of this kernel; expands to nothing in the library.
-#ifndef DEERS_TRACE_POINT
-#define DEERS_TRACE_POINT(slot)
-#endif
 
 template <int D>
 struct FwdCfg {
@@ -100,7 +96,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
   half_t* O = (half_t*)p.o + b * p.so.b + h * p.so.h;
 
   [[maybe_unused]] const int trace_row = blockIdx.x;
-  DEERS_TRACE_POINT(0);
   const int q0 = qtile * kFwdBM;
   const int qw0 = q0 + 32 * wave;        // first query row of this wave
   const int qrow = qw0 + (lane & 31);    // this lane's query row
@@ -392,7 +387,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
       pf[i] = pn[i];
     }
     asm volatile("" : "+v"(lsum));
-    DEERS_TRACE_POINT(2 + j);
   };
 
   // ---- S(0): K(0) is the oldest request ----
@@ -404,7 +398,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
     load_k(0, kfr);
     mfma_s(kfr, sa0, sa1);
   }
-  DEERS_TRACE_POINT(1);
 
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
@@ -442,7 +435,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
     for (int db = 0; db < DB; ++db) store_block_f16(orow + 32 * db, oacc[db], inv, g);
     if (g == 0) p.lse[(int64_t)bh * T + qrow] = (m * c + fast_log2(lsum)) * kLn2;
   }
-  DEERS_TRACE_POINT(30);
 }
 
 // Position -> tile table of a launch whose workgroups are all resident at once, passed in
@@ -483,7 +475,6 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
     qtile = n_qtiles - 1 - rank;
   }
   [[maybe_unused]] const int trace_row = blockIdx.x;
-  DEERS_TRACE_POINT(0);
   const int b = bh / p.H, h = bh % p.H;
   const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
   const half_t* K = (const half_t*)p.k + b * p.sk.b + h * p.sk.h;
@@ -546,7 +537,6 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
   float m = -INFINITY, lsum = 0.f;
   const float c = p.scale_log2;
   wait_all_vmem();  // Q fragments (and with them every request so far)
-  DEERS_TRACE_POINT(1);
 
   for (int j = 0; j < n_tiles; ++j) {
     const int kv0 = j * kFwdBN;
@@ -639,7 +629,6 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
       tile_step(std::integral_constant<int, 1>{});
     else
       tile_step(std::integral_constant<int, 2>{});
-    DEERS_TRACE_POINT(2 + j);
   }
   lsum = pair_sum(lsum);
   if (qrow < T) {
@@ -649,7 +638,6 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams
     for (int db = 0; db < DB; ++db) store_block_f16(orow + 32 * db, oacc[db], inv, g);
     if (g == 0) p.lse[(int64_t)bh * T + qrow] = (m * c + fast_log2(lsum)) * kLn2;
   }
-  DEERS_TRACE_POINT(30);
 }
 
 // Builds the TileOrder of a launch whose workgroups are all resident at once (their

@@ -224,7 +224,9 @@ struct BwdParams {
   float* lse2; float* negdelta; int t_pad;
   // ready[bh * n_blocks + q_block] == epoch once the dQ workgroup of that 128-row query
   // block has published its lse2 / negdelta rows (f16 path, single-launch backward)
-  int* ready; int epoch;
+  // ready[-1] is the hand-over error word: set to 1 by a dK/dV workgroup whose bounded
+  // wait for a flag ran out (spin_limit polls), read by the host after the next sync
+  int* ready; int epoch; int spin_limit;
   void* dq; void* dk; void* dv;
   Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
   int H, T;
@@ -274,12 +276,10 @@ __device__ __forceinline__ bool map_block(int block_id, int n_blocks, int heads_
 // blocks ask the instruction arbiter for priority over the short blocks that share
 // their SIMD, which then fill the gaps.
 __device__ __forceinline__ void set_block_priority(int rank, int n_blocks) {
-#ifndef DEERS_NO_BLOCK_PRIORITY
   const int q = (4 * rank) / max(n_blocks, 1);  // 0 = longest quarter
   if (q == 0) __builtin_amdgcn_s_setprio(3);
   else if (q == 1) __builtin_amdgcn_s_setprio(2);
   else if (q == 2) __builtin_amdgcn_s_setprio(1);
-#endif
 }
 
 // Brackets one kernel launch with a hipEvent pair when per-kernel profiling is

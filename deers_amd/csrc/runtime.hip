@@ -25,7 +25,7 @@
 namespace deers {
 void launch_attn_fwd_f16(const FwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_fwd_f32(const FwdParams& p, int B, int D, hipStream_t stream);
-void launch_attn_bwd_f16(const BwdParams& p, int B, int D, hipStream_t stream);
+void launch_attn_bwd_f16(const BwdParams& p, int B, int D, int mode, hipStream_t stream);
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream);
 void launch_attn_decode_f16(const DecodeParams& p, int B, int D, bool append, hipStream_t stream);
 int decode_pick_splits(int64_t BH, int64_t L, int* chunk);
@@ -104,9 +104,21 @@ struct Runtime {
   rocblas_handle blas = nullptr;  // created by the first matmul, bound to `stream`
   // per (head, 128-row query block) publication flags of the single-launch f16
   // backward; a flag equals the current epoch once its rows are published
-  int* bwd_ready = nullptr;
+  int* bwd_ready = nullptr;  // allocation: [error word][flags ...]; kernels get the address of flags[0]
   size_t bwd_ready_len = 0;
   int bwd_epoch = 0;
+  bool bwd_error_armed = false;  // a single-launch backward ran since the error word was last read
+  // Hand-overs between workgroups inside one launch (the f16 backward's row statistics,
+  // the few-rows GEMM's K splits) rely on producer and consumer sharing one XCD's L2,
+  // which the kernels get from "workgroup id % 8 is the XCD".  True only on a device where
+  // that is known to hold (see handover_policy); otherwise the library takes the forms
+  // that need no such hand-over (two launches, unsplit K).
+  bool same_xcd_handover = false;
+  int handover_forced = -1;   // -1: by policy; 0 / 1: forced by deers_rocm_set_handover_mode
+  // test hooks (deers_rocm_debug_bwd_wait): poll bound of the backward's flag wait, and
+  // whether the next single-launch backward leaves out the workgroups that publish
+  int bwd_spin_limit = 1 << 20;
+  int bwd_skip_producers = 0;
   // sticky "an index was out of range" flag that index kernels raise; read back by the
   // next synchronising call after one of them has been launched
   int* index_flag = nullptr;
@@ -163,6 +175,23 @@ int fail(int code, const char* fmt, ...) {
     if (!g_rt.ready)                                                                    \
       return fail(DEERS_ROCM_ERR_NOT_INIT, "deers_rocm_init has not been called");      \
   } while (0)
+
+// The XCD-local hand-overs are taken only on an unpartitioned MI355X with every CU
+// enabled: 256 CUs = 8 XCDs x 32, where the dispatcher deals workgroups round-robin to the
+// XCDs.  A compute partition (fewer CUs per device) or a CU mask changes which XCD a
+// workgroup id lands on.
+int handover_policy(int cu_count, int cu_mask_set) {
+  return (cu_count == 256 && !cu_mask_set) ? DEERS_ROCM_HANDOVER_SAME_XCD
+                                           : DEERS_ROCM_HANDOVER_STREAM_ORDER;
+}
+
+bool cu_mask_in_environment() {
+  for (const char* name : {"ROC_GLOBAL_CU_MASK", "HSA_CU_MASK", "HSA_CU_MASK_SKIP_INIT"}) {
+    const char* v = getenv(name);
+    if (v && *v) return true;
+  }
+  return false;
+}
 
 bool device_is_gfx950(int ordinal) {
   hipDeviceProp_t prop;
@@ -318,6 +347,13 @@ int deers_rocm_init(int ordinal) {
   HIP_TRY(hipSetDevice(ordinal));
   HIP_TRY(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
   HIP_TRY(hipGetSymbolAddress(&g_scratch_ptr, HIP_SYMBOL(scratch)));
+  {
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, ordinal));
+    g_rt.same_xcd_handover =
+        handover_policy(prop.multiProcessorCount, cu_mask_in_environment() ? 1 : 0) ==
+        DEERS_ROCM_HANDOVER_SAME_XCD;
+  }
   g_rt.ordinal = ordinal;
   g_rt.ready = true;
   return DEERS_ROCM_OK;
@@ -340,19 +376,78 @@ int check_index_flag() {
   if (!g_rt.index_flag_armed) return DEERS_ROCM_OK;
   g_rt.index_flag_armed = false;
   int seen = 0;
-  HIP_TRY(hipMemcpy(&seen, g_rt.index_flag, sizeof(int), hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpyAsync(&seen, g_rt.index_flag, sizeof(int), hipMemcpyDeviceToHost, g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
   if (!seen) return DEERS_ROCM_OK;
-  HIP_TRY(hipMemset(g_rt.index_flag, 0, sizeof(int)));
+  // on the library stream, so that the reset is ordered with the kernels that raise the flag
+  HIP_TRY(hipMemsetAsync(g_rt.index_flag, 0, sizeof(int), g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
   return fail(DEERS_ROCM_ERR_INDEX,
               "an index was out of bounds in an index_select / index_add / cross_entropy call "
               "since the last synchronisation (such rows were skipped)");
+}
+
+// After the stream has drained: reports (once) that a dK/dV workgroup of a single-launch
+// backward gave up waiting for its row statistics since the last check.
+int check_handover_error() {
+  if (!g_rt.bwd_error_armed || !g_rt.bwd_ready) return DEERS_ROCM_OK;
+  g_rt.bwd_error_armed = false;
+  int seen = 0;
+  HIP_TRY(hipMemcpyAsync(&seen, g_rt.bwd_ready, sizeof(int), hipMemcpyDeviceToHost, g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  if (!seen) return DEERS_ROCM_OK;
+  HIP_TRY(hipMemsetAsync(g_rt.bwd_ready, 0, sizeof(int), g_rt.stream));
+  HIP_TRY(hipStreamSynchronize(g_rt.stream));
+  return fail(DEERS_ROCM_ERR_HANDOVER,
+              "attn_bwd: a workgroup gave up waiting for another workgroup's row statistics "
+              "in a backward pass since the last synchronisation; dK and dV of that call are "
+              "not valid (deers_rocm_set_handover_mode(DEERS_ROCM_HANDOVER_STREAM_ORDER) "
+              "selects the form without this wait)");
+}
+
+int check_device_flags() {
+  if (int rc = check_index_flag()) return rc;
+  return check_handover_error();
 }
 
 int deers_rocm_sync(void) {
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   HIP_TRY(hipStreamSynchronize(g_rt.stream));
-  return check_index_flag();
+  return check_device_flags();
+}
+
+int deers_rocm_handover_policy(int cu_count, int cu_mask_set) {
+  return handover_policy(cu_count, cu_mask_set);
+}
+
+static bool same_xcd_handover_now() {
+  return g_rt.handover_forced >= 0 ? g_rt.handover_forced == DEERS_ROCM_HANDOVER_SAME_XCD
+                                   : g_rt.same_xcd_handover;
+}
+
+int deers_rocm_handover_mode(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_rt.ready) return -1;
+  return same_xcd_handover_now() ? DEERS_ROCM_HANDOVER_SAME_XCD : DEERS_ROCM_HANDOVER_STREAM_ORDER;
+}
+
+int deers_rocm_set_handover_mode(int mode) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (mode != -1 && mode != DEERS_ROCM_HANDOVER_SAME_XCD && mode != DEERS_ROCM_HANDOVER_STREAM_ORDER)
+    return fail(DEERS_ROCM_ERR_ARG, "set_handover_mode: mode %d is not -1, 0 or 1", mode);
+  g_rt.handover_forced = mode;
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_debug_bwd_wait(int spin_limit, int skip_producers) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (spin_limit < 1) return fail(DEERS_ROCM_ERR_ARG, "debug_bwd_wait: spin_limit must be >= 1");
+  g_rt.bwd_spin_limit = spin_limit;
+  g_rt.bwd_skip_producers = skip_producers ? 1 : 0;
+  return DEERS_ROCM_OK;
 }
 
 const char* deers_rocm_last_error(void) { return t_err.c_str(); }
@@ -443,7 +538,7 @@ int deers_rocm_dtoh(void* dst_host, const void* src_device, size_t bytes) {
   if (!dst_host || !src_device) return fail(DEERS_ROCM_ERR_ARG, "dtoh: null pointer");
   HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, g_rt.stream));
   HIP_TRY(hipStreamSynchronize(g_rt.stream));
-  return check_index_flag();
+  return check_device_flags();
 }
 
 int deers_rocm_dtod(void* dst_device, const void* src_device, size_t bytes) {
@@ -610,14 +705,16 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
         g_rt.bwd_ready = nullptr;
       }
       const size_t want = n_flags > g_rt.bwd_ready_len ? n_flags : g_rt.bwd_ready_len;
-      HIP_TRY(hipMalloc(&g_rt.bwd_ready, want * sizeof(int)));
-      HIP_TRY(hipMemsetAsync(g_rt.bwd_ready, 0, want * sizeof(int), g_rt.stream));
+      HIP_TRY(hipMalloc(&g_rt.bwd_ready, (want + 1) * sizeof(int)));  // [error word][flags]
+      HIP_TRY(hipMemsetAsync(g_rt.bwd_ready, 0, (want + 1) * sizeof(int), g_rt.stream));
       g_rt.bwd_ready_len = want;
       g_rt.bwd_epoch = 0;
     }
-    p.ready = g_rt.bwd_ready;
+    p.ready = g_rt.bwd_ready + 1;
     p.epoch = ++g_rt.bwd_epoch;
+    p.spin_limit = g_rt.bwd_spin_limit;
   }
+  const bool single_launch = same_xcd_handover_now();
   p.lse2 = static_cast<float*>(ws);
   p.negdelta = static_cast<float*>(ws) + B * H * t_pad;
   p.t_pad = (int)t_pad;
@@ -625,10 +722,13 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   p.H = (int)H; p.T = (int)T;
   p.scale = scale;
   p.scale_log2 = (float)((double)scale * 1.4426950408889634);
-  if (dtype == DEERS_ROCM_F16)
-    deers::launch_attn_bwd_f16(p, (int)B, (int)D, g_rt.stream);
-  else
+  if (dtype == DEERS_ROCM_F16) {
+    if (single_launch) g_rt.bwd_error_armed = true;
+    const int mode = !single_launch ? 0 : (g_rt.bwd_skip_producers ? 2 : 1);
+    deers::launch_attn_bwd_f16(p, (int)B, (int)D, mode, g_rt.stream);
+  } else {
     deers::launch_attn_bwd_f32(p, (int)B, (int)D, g_rt.stream);
+  }
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }
@@ -1325,7 +1425,9 @@ constexpr int kSkinnyCounters = 4096;  // column blocks a K-split launch of the 
 // of x's rows, 2 relu(x)^2.  The caller holds g_mu.
 static int skinny_locked(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t m,
                          int64_t n, int64_t k, bool accumulate, int prologue, float eps, bool packed) {
-  int splits = prologue == 1 ? 1 : deers::skinny_gemm_splits(n, k);  // row sums of squares need all of K
+  // row sums of squares need all of K; the split sum's hand-over needs the splits of a
+  // column block on one XCD
+  int splits = (prologue == 1 || !same_xcd_handover_now()) ? 1 : deers::skinny_gemm_splits(n, k);
   void* ws = nullptr;
   if (splits > 1 && (n + 31) / 32 > kSkinnyCounters) splits = 1;
   if (splits > 1) {

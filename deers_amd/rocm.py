@@ -60,6 +60,28 @@ def sync():
     _check(load().deers_rocm_sync())
 
 
+HANDOVER_STREAM_ORDER, HANDOVER_SAME_XCD = 0, 1
+
+
+def handover_policy(cu_count: int, cu_mask_set: bool) -> int:
+    """deers_rocm_handover_policy: the rule alone, no device needed."""
+    return int(load().deers_rocm_handover_policy(ctypes.c_int(cu_count), ctypes.c_int(int(cu_mask_set))))
+
+
+def handover_mode() -> int:
+    """Mode in force: HANDOVER_SAME_XCD / HANDOVER_STREAM_ORDER, -1 before init."""
+    return int(load().deers_rocm_handover_mode())
+
+
+def set_handover_mode(mode: int):
+    _check(load().deers_rocm_set_handover_mode(ctypes.c_int(mode)))
+
+
+def debug_bwd_wait(spin_limit: int = 1 << 20, skip_producers: bool = False):
+    """Test hook of the single-launch backward's bounded wait (see the header)."""
+    _check(load().deers_rocm_debug_bwd_wait(ctypes.c_int(spin_limit), ctypes.c_int(int(skip_producers))))
+
+
 def dtype_code(dtype) -> int:
     dtype = np.dtype(dtype)
     if dtype == np.float16:

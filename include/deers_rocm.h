@@ -51,6 +51,10 @@ extern "C" {
 #define DEERS_ROCM_ERR_NOT_INIT 4    /* deers_rocm_init has not succeeded */
 #define DEERS_ROCM_ERR_INDEX 5       /* an index tensor held a value out of range; reported by
                                         the next deers_rocm_sync / _dtoh (Error::IndexOutOfBounds) */
+#define DEERS_ROCM_ERR_HANDOVER 6    /* a workgroup of the backward gave up waiting for another
+                                        workgroup's results; reported by the next deers_rocm_sync /
+                                        _dtoh, the way a backend failure becomes Error::Cuda(String)
+                                        (src/error.rs:40-41) */
 
 /* ---- runtime ------------------------------------------------------------ */
 
@@ -75,6 +79,33 @@ const char* deers_rocm_last_error(void);
 /* The HIP stream all work is enqueued on (a hipStream_t), for callers that
  * want to order their own work after it. */
 void* deers_rocm_stream(void);
+
+/* ---- hand-overs between workgroups ----------------------------------------
+ * Two kernels pass data between workgroups inside one launch: the f16 attention backward
+ * (row statistics published by one half of the grid, read by the other) and the few-rows
+ * GEMM (K splits summed by the last workgroup to arrive).  Both publish with a drained
+ * store plus a relaxed flag / counter, which is sufficient only while producer and
+ * consumer run on the same XCD (one L2); the kernels arrange that by workgroup id % 8.
+ * deers_rocm_init checks what that mapping assumes, in the spirit of the capability
+ * checks of the reference's runtime construction (src/storage/cuda.rs:492-528), and
+ * otherwise selects forms without such a hand-over: the backward as two launches in
+ * stream order, the few-rows GEMM unsplit.  Same results either way (the backward bit for
+ * bit). */
+#define DEERS_ROCM_HANDOVER_STREAM_ORDER 0
+#define DEERS_ROCM_HANDOVER_SAME_XCD 1
+/* The rule itself, callable without a device: SAME_XCD only for an unpartitioned MI355X
+ * (256 compute units) with no CU mask in the environment. */
+int deers_rocm_handover_policy(int cu_count, int cu_mask_set);
+/* The mode in force (after deers_rocm_init; -1 before), and an override: mode -1 returns
+ * to the policy's choice for this device. */
+int deers_rocm_handover_mode(void);
+int deers_rocm_set_handover_mode(int mode);
+/* Test hook for the bounded wait of the single-launch backward: `spin_limit` polls (the
+ * default is 2^20) and, when `skip_producers` is non-zero, backward calls launch only the
+ * waiting half of the grid, so that every wait runs out, every kernel still exits, and the
+ * next deers_rocm_sync returns DEERS_ROCM_ERR_HANDOVER.  (spin_limit 2^20,
+ * skip_producers 0) restores normal operation. */
+int deers_rocm_debug_bwd_wait(int spin_limit, int skip_producers);
 
 /* ---- device memory (the storage backend's alloc / to-device / to_vec) ---- */
 
