@@ -161,6 +161,7 @@ int main(int argc, char** argv) {
 
     AdamW opt = AdamWConfig(3e-4).betas(0.9, 0.95).weight_decay(0.1).build(params);
     float last_loss = 0.f, last_norm = 0.f;
+    std::vector<float> losses, norms;  // every step of the run, in order (warm-up first)
     auto step = [&]() {
       Tensor loss = cross_entropy(model.forward(ids).reshape({B * T, cfg.vocab_size}), targets);
       GradientStore grads = loss.backward();
@@ -168,6 +169,8 @@ int main(int argc, char** argv) {
       last_norm = clip_grad_scale(params, grads, 1.0, &scale);  // reads 4 bytes back: one sync per step
       opt.step_with_grads(grads, scale);
       loss.to_host(&last_loss);
+      losses.push_back(last_loss);
+      norms.push_back(last_norm);
     };
     for (int i = 0; i < warmup; ++i) step();
     const float first_loss = last_loss;
@@ -197,11 +200,20 @@ int main(int argc, char** argv) {
     kernels += "}";
     check(deers_rocm_profile_enable(0));
 
+    auto join = [](const std::vector<float>& v) {
+      std::string out = "[";
+      char buf[32];
+      for (size_t i = 0; i < v.size(); ++i) {
+        std::snprintf(buf, sizeof(buf), "%s%.5f", i ? ", " : "", v[i]);
+        out += buf;
+      }
+      return out + "]";
+    };
     std::printf(
         "{\"gemm_tuning\": %s, \"ms_per_step\": %.3f, \"tokens_per_s\": %.1f, \"parameters\": %lld, \"batch\": %lld, \"seq_len\": %lld, "
-        "\"loss_first\": %.4f, \"loss_last\": %.4f, \"grad_norm\": %.4f, \"kernels\": %s}\n",
+        "\"loss_first\": %.4f, \"loss_last\": %.4f, \"grad_norm\": %.4f, \"losses\": %s, \"grad_norms\": %s, \"kernels\": %s}\n",
         tune ? "true" : "false", ms, 1e3 * (double)(B * T) / ms, (long long)n_params, (long long)B, (long long)T, first_loss, last_loss,
-        last_norm, kernels.c_str());
+        last_norm, join(losses).c_str(), join(norms).c_str(), kernels.c_str());
     return 0;
   } catch (const std::exception& e) {
     std::fprintf(stderr, "gpt_step: %s\n", e.what());
