@@ -63,3 +63,15 @@ def attention_inputs(config: str, B: int, H: int, T: int, D: int, dtype, base_se
         x = normal((B, H, t, D), tensor_seed(base_seed, config, name), sigma)
         out[name] = x.astype(dtype)
     return out
+
+
+def rotary_tables(seq_len: int, head_dim: int, base: float = 10000.0, dtype=np.float32):
+    """cos, sin [seq_len, head_dim/2] of the rotary embedding, the host-side table a model
+    uploads once (the reference builds it on the CPU in f32 and moves it to the device,
+    src/models/gpt.rs:12-47): inv_freq_i = base^(-2i/D), angle = t * inv_freq."""
+    half = head_dim // 2
+    inv_freq = (np.float32(1.0) / np.power(np.float32(base),
+                                           (2 * np.arange(half)).astype(np.float32) / np.float32(head_dim))
+                ).astype(np.float32)
+    ang = (np.arange(seq_len, dtype=np.float32)[:, None] * inv_freq[None, :]).astype(np.float32)
+    return np.cos(ang).astype(dtype), np.sin(ang).astype(dtype)

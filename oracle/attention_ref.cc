@@ -34,7 +34,10 @@
 //                           torch autograd
 //
 // Template parameter R is the real type: float follows the reference's f32 path
-// bit-for-op; double exists only so finite-difference tests have head-room.
+// op for op (built with -ffp-contract=off, so a multiply and an add stay two roundings
+// as in the element-wise Rust code; the GEMM inner loops of crate `gemm` may fuse them,
+// which is the unpinned ulp-level order named above); double exists only so
+// finite-difference tests have head-room.
 
 #include <algorithm>
 #include <cmath>

@@ -531,3 +531,14 @@ def test_cross_entropy_reference_cases_and_library():
     p /= p.sum(axis=1, keepdims=True)
     p[np.arange(7), t] -= 1
     assert np.abs(oracle.cross_entropy_bwd(x, t) - p / 7).max() < 1e-7
+
+
+def test_synthetic_rotary_tables_equal_the_oracle_tables():
+    """deers_amd.synth.rotary_tables feeds the benchmark; it must be the table the oracle
+    (src/models/gpt.rs:12-47) pins, bit for bit, in both storage types."""
+    from deers_amd import synth
+    for T, D in ((1, 2), (7, 32), (1024, 64), (300, 128)):
+        for dt in (np.float32, np.float16):
+            c, s = synth.rotary_tables(T, D, dtype=dt)
+            oc, os_ = oracle.rope_tables(T, D, dtype=dt)
+            assert c.dtype == dt and np.array_equal(c, oc) and np.array_equal(s, os_)
