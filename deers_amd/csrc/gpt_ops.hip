@@ -76,8 +76,12 @@ __global__ __launch_bounds__(256) void index_select_kernel(const T* table, const
 // is the same bits and the same from run to run: workgroup i owns the destination row
 // idx[i] if no earlier position names it, finds every later position that does (a
 // bitmap in LDS, built from the index vector, which stays in L2), and adds their source
-// rows in order.  Other workgroups leave at once.
-constexpr int kIndexAddMaxIdx = 1 << 18;  // bitmap of 32 KB of dynamic LDS
+// rows in order.  Other workgroups leave at once.  A launch covers at most
+// kIndexAddChunk positions (every workgroup scans its launch's whole index slice, so the
+// cost of a launch grows with the square of its length); longer index vectors take one
+// launch per slice, in order, which keeps the order of additions: a later slice adds to
+// what the earlier ones left.
+constexpr int kIndexAddChunk = 1 << 14;  // bitmap of 2 KB of dynamic LDS
 
 template <typename T>
 __global__ __launch_bounds__(256) void index_add_kernel(const T* src, const int64_t* idx, T* dst,
@@ -488,8 +492,6 @@ unsigned stream_grid(int64_t work_items) {
 
 }  // namespace
 
-int index_add_max_indices() { return kIndexAddMaxIdx; }
-
 template <typename T>
 static void index_select_t(const T* table, const int64_t* idx, T* out, int64_t n_rows, int64_t n_idx,
                            int width, int* flag, hipStream_t stream) {
@@ -513,15 +515,20 @@ void launch_index_select(int dtype_f16, const void* table, const int64_t* idx, v
 }
 
 void launch_index_add(int dtype_f16, const void* src, const int64_t* idx, void* dst, int64_t n_rows,
-                      int n_idx, int width, int* flag, hipStream_t stream) {
+                      int64_t n_idx, int width, int* flag, hipStream_t stream) {
   LaunchScope scope("index_add", stream);
-  const size_t lds = (size_t)((n_idx + 63) / 64) * 2 * sizeof(unsigned int);
-  if (dtype_f16)
-    hipLaunchKernelGGL(index_add_kernel<half_t>, dim3((unsigned)n_idx), dim3(256), lds, stream,
-                       (const half_t*)src, idx, (half_t*)dst, n_rows, n_idx, width, flag);
-  else
-    hipLaunchKernelGGL(index_add_kernel<float>, dim3((unsigned)n_idx), dim3(256), lds, stream,
-                       (const float*)src, idx, (float*)dst, n_rows, n_idx, width, flag);
+  for (int64_t first = 0; first < n_idx; first += kIndexAddChunk) {
+    const int n = (int)(n_idx - first < kIndexAddChunk ? n_idx - first : kIndexAddChunk);
+    const size_t lds = (size_t)((n + 63) / 64) * 2 * sizeof(unsigned int);
+    if (dtype_f16)
+      hipLaunchKernelGGL(index_add_kernel<half_t>, dim3((unsigned)n), dim3(256), lds, stream,
+                         (const half_t*)src + first * width, idx + first, (half_t*)dst, n_rows, n, width,
+                         flag);
+    else
+      hipLaunchKernelGGL(index_add_kernel<float>, dim3((unsigned)n), dim3(256), lds, stream,
+                         (const float*)src + first * width, idx + first, (float*)dst, n_rows, n, width,
+                         flag);
+  }
 }
 
 template <typename T>

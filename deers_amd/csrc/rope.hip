@@ -66,6 +66,31 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   }
 }
 
+// The same rotation one (x1, x2) pair per thread, for head widths whose half row is not a
+// whole number of 16-byte chunks (the reference's own GPT test runs head_dim 2,
+// tests/gpt.rs:38-49) or rows that are not 16-byte aligned.  Same arithmetic and rounding.
+template <typename T, bool INVERSE>
+__global__ __launch_bounds__(256) void rope_pair_kernel(RopeParams p) {
+  const int half = p.D / 2;
+  const int64_t total = (int64_t)p.B * p.T * p.H * half;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    const int c = (int)(i % half);
+    int64_t r = i / half;
+    const int h = (int)(r % p.H); r /= p.H;
+    const int t = (int)(r % p.T);
+    const int b = (int)(r / p.T);
+    const T* s = (const T*)p.src + b * p.s_b + t * p.s_t + h * p.s_h + c;
+    T* d = (T*)p.dst + b * p.d_b + t * p.d_t + h * p.d_h + c;
+    const float x1 = (float)s[0], x2 = (float)s[half];
+    const float co = (float)((const T*)p.cos)[(int64_t)t * half + c];
+    const float sn = (float)((const T*)p.sin)[(int64_t)t * half + c];
+    const float si = INVERSE ? -sn : sn;
+    d[0] = (T)(x1 * co + x2 * si);
+    d[half] = (T)(x2 * co - x1 * si);
+  }
+}
+
 // One generation step's handling of the new token's projections, in one launch: q and k
 // rotated at the step's position, q to a compact [B,H,D] tensor, k and the unrotated v to
 // row `pos` of their caches.  Inputs are [B,H,D] views by strides {b,h} (thirds of a fused
@@ -138,9 +163,11 @@ void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* 
 // x: logical [B,T,H,D] with element strides xs = {b,t,h} (D stride 1); y: [B,H,T,D],
 // compact or with element strides {b,h,t} (a row range of a KV cache).
 // inverse: dy [B,H,T,D] with strides {b,h,t} -> dx compact [B,T,H,D].
-void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
-                 const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
-                 int T, int H, int D, hipStream_t stream) {
+// vectorised: every row and half row on both sides is a whole number of aligned 16-byte
+// chunks; otherwise one pair per thread.
+void launch_rope(int dtype_f16, bool inverse, bool vectorised, const void* src,
+                 const int64_t* src_strides, const void* cos, const void* sin, void* dst,
+                 const int64_t* dst_strides, int B, int T, int H, int D, hipStream_t stream) {
   RopeParams p{};
   p.src = src; p.dst = dst; p.cos = cos; p.sin = sin;
   p.B = B; p.T = T; p.H = H; p.D = D;
@@ -153,10 +180,20 @@ void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* sr
     p.d_b = (int64_t)T * H * D; p.d_t = (int64_t)H * D; p.d_h = D;
   }
   const int n16 = dtype_f16 ? 8 : 4;
-  const int64_t total = (int64_t)B * T * H * (D / 2 / n16);
+  const int64_t total = vectorised ? (int64_t)B * T * H * (D / 2 / n16) : (int64_t)B * T * H * (D / 2);
   const int64_t blocks = (total + 255) / 256;
   const unsigned grid = (unsigned)(blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks));
   LaunchScope scope(inverse ? "rope_bwd" : "rope_fwd", stream);
+  if (!vectorised) {
+    if (dtype_f16) {
+      if (inverse) hipLaunchKernelGGL((rope_pair_kernel<half_t, true>), dim3(grid), dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((rope_pair_kernel<half_t, false>), dim3(grid), dim3(256), 0, stream, p);
+    } else {
+      if (inverse) hipLaunchKernelGGL((rope_pair_kernel<float, true>), dim3(grid), dim3(256), 0, stream, p);
+      else hipLaunchKernelGGL((rope_pair_kernel<float, false>), dim3(grid), dim3(256), 0, stream, p);
+    }
+    return;
+  }
   if (dtype_f16) {
     if (inverse) hipLaunchKernelGGL((rope_kernel<half_t, true>), dim3(grid), dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((rope_kernel<half_t, false>), dim3(grid), dim3(256), 0, stream, p);

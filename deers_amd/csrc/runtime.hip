@@ -47,18 +47,17 @@ void launch_decode_qkv(int dtype_f16, const void* q, const void* k, const void* 
                        const int64_t* in_strides, const void* cos_row, const void* sin_row, void* q_out,
                        void* k_cache, void* v_cache, const int64_t* cache_strides, int64_t pos, int B,
                        int H, int D, hipStream_t stream);
-void launch_rope(int dtype_f16, bool inverse, const void* src, const int64_t* src_strides,
-                 const void* cos, const void* sin, void* dst, const int64_t* dst_strides, int B,
-                 int T, int H, int D, hipStream_t stream);
+void launch_rope(int dtype_f16, bool inverse, bool vectorised, const void* src,
+                 const int64_t* src_strides, const void* cos, const void* sin, void* dst,
+                 const int64_t* dst_strides, int B, int T, int H, int D, hipStream_t stream);
 void launch_log_softmax_fwd(int dtype_f16, const void* x, void* out, int64_t outer, int64_t inner,
                             hipStream_t stream);
 void launch_log_softmax_bwd(int dtype_f16, const void* grad, const void* lsm, void* out,
                             int64_t outer, int64_t inner, hipStream_t stream);
-int index_add_max_indices();
 void launch_index_select(int dtype_f16, const void* table, const int64_t* idx, void* out,
                          int64_t n_rows, int64_t n_idx, int width, int* flag, hipStream_t stream);
 void launch_index_add(int dtype_f16, const void* src, const int64_t* idx, void* dst, int64_t n_rows,
-                      int n_idx, int width, int* flag, hipStream_t stream);
+                      int64_t n_idx, int width, int* flag, hipStream_t stream);
 void launch_rms_norm(int dtype_f16, const void* x, const void* dy, void* out, int64_t outer, int width,
                      float eps, int bwd, hipStream_t stream);
 void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int64_t n, int bwd,
@@ -984,14 +983,11 @@ int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, voi
   NEED_INIT();
   if (int rc = rows_check("index_add", dtype, n_indices, width)) return rc;
   if (n_rows < 0) return fail(DEERS_ROCM_ERR_ARG, "index_add: negative destination size");
-  if (n_indices > deers::index_add_max_indices())
-    return fail(DEERS_ROCM_ERR_ARG, "index_add: at most %d indices per call (got %lld)",
-                deers::index_add_max_indices(), (long long)n_indices);
   if (n_indices == 0) return DEERS_ROCM_OK;
   if (!src || !indices || !dst) return fail(DEERS_ROCM_ERR_ARG, "index_add: null pointer");
   int* flag = nullptr;
   if (int rc = index_flag(&flag)) return rc;
-  deers::launch_index_add(dtype == DEERS_ROCM_F16, src, indices, dst, n_rows, (int)n_indices,
+  deers::launch_index_add(dtype == DEERS_ROCM_F16, src, indices, dst, n_rows, n_indices,
                           (int)width, flag, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
@@ -1619,17 +1615,18 @@ int deers_rocm_decode_linear_hint(const void* next_w_packed, int64_t n, int64_t 
 
 // ---- rotary embedding fused with the head split / merge ----
 
+// Checks shared by rope_fwd / rope_bwd.  *vectorised: every row of the strided side is a
+// whole number of aligned 16-byte chunks (the fast kernel); any other even D, stride or
+// alignment takes the kernel that moves one pair per thread.
 static int rope_common(const char* what, int dtype, const void* src, const int64_t* strides,
                        const void* cos, const void* sin, void* dst, int64_t B, int64_t T,
-                       int64_t H, int64_t D, int64_t* resolved, bool inverse) {
+                       int64_t H, int64_t D, int64_t* resolved, bool inverse, bool* vectorised) {
   if (int rc = check_dtype(dtype)) return rc;
   if (!src || !cos || !sin || !dst) return fail(DEERS_ROCM_ERR_ARG, "%s: null pointer", what);
   const int64_t per16 = dtype == DEERS_ROCM_F16 ? 8 : 4;
-  if (B < 1 || T < 1 || H < 1 || D < 2 || (D / 2) % per16 || D % 2 ||
+  if (B < 1 || T < 1 || H < 1 || D < 2 || D % 2 ||
       B * T * H * D >= (int64_t(1) << 40) || B > INT32_MAX || T > INT32_MAX || H > INT32_MAX)
-    return fail(DEERS_ROCM_ERR_ARG,
-                "%s: need B,T,H >= 1 and D/2 a multiple of %lld elements (16 bytes)", what,
-                (long long)per16);
+    return fail(DEERS_ROCM_ERR_ARG, "%s: need B,T,H >= 1 and an even D >= 2", what);
   // compact defaults: forward input [B,T,H,D], backward input [B,H,T,D]
   resolved[0] = T * H * D;
   resolved[1] = inverse ? T * D : H * D;
@@ -1641,12 +1638,15 @@ static int rope_common(const char* what, int dtype, const void* src, const int64
   }
   if (last != 1)
     return fail(DEERS_ROCM_ERR_LAYOUT, "%s: innermost stride is %lld, need 1", what, (long long)last);
-  for (int d = 0; d < 3; ++d)
-    if (resolved[d] < 0 || resolved[d] % per16)
-      return fail(DEERS_ROCM_ERR_LAYOUT, "%s: strides must be non-negative multiples of 16 bytes", what);
+  *vectorised = (D / 2) % per16 == 0;
+  for (int d = 0; d < 3; ++d) {
+    if (resolved[d] < 0)
+      return fail(DEERS_ROCM_ERR_LAYOUT, "%s: strides must be non-negative", what);
+    if (resolved[d] % per16) *vectorised = false;
+  }
   if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) |
        reinterpret_cast<uintptr_t>(cos) | reinterpret_cast<uintptr_t>(sin)) & 15)
-    return fail(DEERS_ROCM_ERR_LAYOUT, "%s: pointers must be 16-byte aligned", what);
+    *vectorised = false;
   return DEERS_ROCM_OK;
 }
 
@@ -1656,19 +1656,22 @@ int deers_rocm_rope_fwd(int dtype, const void* x, const int64_t* x_strides, cons
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   int64_t st[3];
-  if (int rc = rope_common("rope_fwd", dtype, x, x_strides, cos, sin, y, B, T, H, D, st, false))
+  bool vectorised = false;
+  if (int rc = rope_common("rope_fwd", dtype, x, x_strides, cos, sin, y, B, T, H, D, st, false,
+                           &vectorised))
     return rc;
   if (y_strides) {
     const int64_t per16 = dtype == DEERS_ROCM_F16 ? 8 : 4;
     if (y_strides[3] != 1)
       return fail(DEERS_ROCM_ERR_LAYOUT, "rope_fwd: innermost output stride must be 1");
-    for (int d = 0; d < 3; ++d)
-      if (y_strides[d] < 0 || y_strides[d] % per16)
-        return fail(DEERS_ROCM_ERR_LAYOUT,
-                    "rope_fwd: output strides must be non-negative multiples of 16 bytes");
+    for (int d = 0; d < 3; ++d) {
+      if (y_strides[d] < 0)
+        return fail(DEERS_ROCM_ERR_LAYOUT, "rope_fwd: output strides must be non-negative");
+      if (y_strides[d] % per16) vectorised = false;
+    }
   }
-  deers::launch_rope(dtype == DEERS_ROCM_F16, false, x, st, cos, sin, y, y_strides, (int)B, (int)T,
-                     (int)H, (int)D, g_rt.stream);
+  deers::launch_rope(dtype == DEERS_ROCM_F16, false, vectorised, x, st, cos, sin, y, y_strides,
+                     (int)B, (int)T, (int)H, (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }
@@ -1707,10 +1710,12 @@ int deers_rocm_rope_bwd(int dtype, const void* dy, const int64_t* dy_strides, co
   std::lock_guard<std::mutex> lock(g_mu);
   NEED_INIT();
   int64_t st[3];
-  if (int rc = rope_common("rope_bwd", dtype, dy, dy_strides, cos, sin, dx, B, T, H, D, st, true))
+  bool vectorised = false;
+  if (int rc = rope_common("rope_bwd", dtype, dy, dy_strides, cos, sin, dx, B, T, H, D, st, true,
+                           &vectorised))
     return rc;
-  deers::launch_rope(dtype == DEERS_ROCM_F16, true, dy, st, cos, sin, dx, nullptr, (int)B, (int)T,
-                     (int)H, (int)D, g_rt.stream);
+  deers::launch_rope(dtype == DEERS_ROCM_F16, true, vectorised, dy, st, cos, sin, dx, nullptr,
+                     (int)B, (int)T, (int)H, (int)D, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

@@ -237,8 +237,12 @@ static int run_gpu(const std::string& dir) {
   {
     bool threw = false;
     try {
-      Tensor bad = Tensor::zeros({1, 1, 8, 48}, dtype);  // head_dim 48 is not supported
-      (void)causal_self_attention(bad, bad, bad);
+      // the fused kernels take head widths 32, 64, 128 only (the op routes other widths
+      // through the unfused chain; the entry point itself refuses them)
+      Tensor bad = Tensor::zeros({1, 1, 8, 48}, dtype);
+      Tensor lse = Tensor::zeros({1, 1, 8}, DType::F32);
+      check(deers_rocm_attn_fwd((int)dtype, bad.data(), nullptr, bad.data(), nullptr, bad.data(), nullptr,
+                                bad.data(), nullptr, (float*)lse.data(), 1, 1, 8, 48, 0.125f));
     } catch (const RocmError& e) {
       threw = std::strlen(e.what()) > 0;
     }

@@ -374,6 +374,7 @@ FusedCausalAttention::FusedCausalAttention(Tensor q, Tensor k, Tensor v, double 
 }
 
 Tensor FusedCausalAttention::forward(std::unique_ptr<FusedCausalAttention> self) {
+  if (!fused_kernels_take(self->q_.shape()[3])) return forward_composed(std::move(self));
   const Tensor q = kernel_ready(self->q_), k = kernel_ready(self->k_), v = kernel_ready(self->v_);
   const auto& s = q.shape();
   const int64_t B = s[0], H = s[1], T = s[2], D = s[3];
@@ -387,7 +388,95 @@ Tensor FusedCausalAttention::forward(std::unique_ptr<FusedCausalAttention> self)
   return Tensor(o.storage(), o.layout(), false, std::move(self));
 }
 
+namespace {
+
+// Additive causal mask [T,T] in the tensor's dtype: -inf where the key lies after the
+// query, else 0 (causal_mask with seqlen_offset 0, src/nn/functional.rs:12-55; the
+// reference builds [B,1,T,T] on the host per call, here one [T,T] block is broadcast over
+// batch and heads by stride 0).
+Tensor causal_mask_tt(int64_t T, DType dtype) {
+  if (dtype == DType::F32) {
+    std::vector<float> m((size_t)(T * T), 0.f);
+    for (int64_t i = 0; i < T; ++i)
+      for (int64_t j = i + 1; j < T; ++j) m[(size_t)(i * T + j)] = -INFINITY;
+    return Tensor::from_host(m.data(), {T, T}, dtype);
+  }
+  std::vector<uint16_t> m((size_t)(T * T), 0);
+  for (int64_t i = 0; i < T; ++i)
+    for (int64_t j = i + 1; j < T; ++j) m[(size_t)(i * T + j)] = 0xFC00;  // -inf
+  return Tensor::from_host(m.data(), {T, T}, dtype);
+}
+
+// c[batch,m,n] = a @ b with explicit (row, col, batch) element strides per operand
+void gemm(DType dt, const Tensor& a, int64_t ars, int64_t acs, int64_t abs_, const Tensor& b,
+          int64_t brs, int64_t bcs, int64_t bbs, Tensor& c, int64_t batch, int64_t m, int64_t n,
+          int64_t k) {
+  check(deers_rocm_matmul((int)dt, a.data(), ars, acs, abs_, b.data(), brs, bcs, bbs, c.data(), batch,
+                          m, n, k));
+}
+
+}  // namespace
+
+Tensor FusedCausalAttention::forward_composed(std::unique_ptr<FusedCausalAttention> self) {
+  const Tensor q = self->q_.compact(), k = self->k_.compact(), v = self->v_.compact();
+  const auto& s = q.shape();
+  const int64_t B = s[0], H = s[1], T = s[2], D = s[3], BH = B * H;
+  const DType dt = q.dtype();
+  if (BH * T * T >= ((int64_t)1 << 31))
+    throw std::logic_error("attention: head width " + std::to_string(D) +
+                           " takes the unfused path, whose [B,H,T,T] tensors would be too large here");
+  const std::vector<int64_t> sc_shape{B, H, T, T};
+  Tensor scores = empty(sc_shape, dt, true), scaled = empty(sc_shape, dt, true);
+  // q @ k^T: k read as [D,T] through its strides (MatMul on a transposed view)
+  gemm(dt, q, D, 1, T * D, k, 1, D, T * D, scores, BH, T, T, D);
+  check(deers_rocm_unary((int)dt, DEERS_ROCM_UNARY_SCALAR_MUL, scores.data(), 4, sc_shape.data(), nullptr,
+                         self->scale_, scaled.data()));
+  const Tensor mask = causal_mask_tt(T, dt);
+  const int64_t mask_strides[4] = {0, 0, T, 1};
+  check(deers_rocm_binary((int)dt, DEERS_ROCM_BINARY_ADD, scaled.data(), nullptr, mask.data(), mask_strides,
+                          4, sc_shape.data(), scores.data()));
+  // softmax = exp(log_softmax) (src/tensor.rs:456-458), log_softmax as the fused row kernel
+  Tensor lsm = empty(sc_shape, dt, true), p = empty(sc_shape, dt, true);
+  check(deers_rocm_log_softmax_fwd((int)dt, scores.data(), lsm.data(), BH * T, T));
+  check(deers_rocm_unary((int)dt, DEERS_ROCM_UNARY_EXP, lsm.data(), 4, sc_shape.data(), nullptr, 0.0,
+                         p.data()));
+  Tensor o = empty(s, dt, true);
+  gemm(dt, p, T, 1, T * T, v, D, 1, T * D, o, BH, T, D, T);
+  self->saved_p_ = p;
+  self->saved_lsm_ = lsm;
+  return Tensor(o.storage(), o.layout(), false, std::move(self));
+}
+
+void FusedCausalAttention::backward_composed(GradientStore& grads, const Tensor& out_grad) const {
+  const Tensor q = q_.compact(), k = k_.compact(), v = v_.compact(), g = out_grad.compact();
+  const auto& s = q.shape();
+  const int64_t B = s[0], H = s[1], T = s[2], D = s[3], BH = B * H;
+  const DType dt = q.dtype();
+  const std::vector<int64_t> sc_shape{B, H, T, T};
+  // MatMul::backward of attn @ v: dAttn = dY @ v^T, dV = attn^T @ dY (src/ops.rs:1089-1101)
+  Tensor dv = empty(s, dt, true), dp = empty(sc_shape, dt, true);
+  gemm(dt, saved_p_, 1, T, T * T, g, D, 1, T * D, dv, BH, T, D, T);
+  gemm(dt, g, D, 1, T * D, v, 1, D, T * D, dp, BH, T, T, D);
+  // EWiseExp::backward: dLsm = dAttn * exp(lsm) (src/ops.rs:422-425)
+  Tensor dlsm = empty(sc_shape, dt, true), dx = empty(sc_shape, dt, true);
+  check(deers_rocm_binary((int)dt, DEERS_ROCM_BINARY_MUL, dp.data(), nullptr, saved_p_.data(), nullptr, 4,
+                          sc_shape.data(), dlsm.data()));
+  // FusedLogSoftmax::backward: dX = dLsm - exp(lsm) * rowsum(dLsm) (src/ops.rs:1223-1246)
+  check(deers_rocm_log_softmax_bwd((int)dt, dlsm.data(), saved_lsm_.data(), dx.data(), BH * T, T));
+  // the mask has no gradient; ScalarMul::backward: dS = dX * scale (src/ops.rs:638-643)
+  check(deers_rocm_unary((int)dt, DEERS_ROCM_UNARY_SCALAR_MUL, dx.data(), 4, sc_shape.data(), nullptr, scale_,
+                         dlsm.data()));
+  // MatMul::backward of q @ k^T: dQ = dS @ k, d(k^T) = q^T @ dS, i.e. dK = dS^T @ q
+  Tensor dq = empty(s, dt, true), dk = empty(s, dt, true);
+  gemm(dt, dlsm, T, 1, T * T, k, D, 1, T * D, dq, BH, T, D, T);
+  gemm(dt, dlsm, 1, T, T * T, q, D, 1, T * D, dk, BH, T, D, T);
+  grads.accumulate(q_, dq);
+  grads.accumulate(k_, dk);
+  grads.accumulate(v_, dv);
+}
+
 void FusedCausalAttention::backward(GradientStore& grads, const Tensor& out_grad) const {
+  if (saved_p_.defined()) return backward_composed(grads, out_grad);
   if (!saved_o_.defined()) throw std::logic_error("forward must run before backward");
   // out_grad usually arrives as the inverse-permuted view of the reshape gradient:
   // logical [B,H,T,D] over [B,T,H,D] memory, which the kernels read directly.
@@ -502,6 +591,14 @@ Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Te
 }
 
 KvCache KvCache::create(int64_t B, int64_t H, int64_t capacity, int64_t D, DType dtype) {
+  // said here, once, rather than by the first decode_step deep inside a generation loop
+  if (dtype != DType::F16)
+    throw std::logic_error("KvCache: the decode kernels read f16 caches only; an f32 model "
+                           "generates through GPT::forward on the whole window, as the reference "
+                           "does (examples/tinystories_train.rs:250-276)");
+  if (D != 32 && D != 64 && D != 128)
+    throw std::logic_error("KvCache: the decode kernels take head widths 32, 64 and 128 (got " +
+                           std::to_string(D) + ")");
   KvCache c;
   c.k = Tensor::zeros({B, H, capacity, D}, dtype);
   c.v = Tensor::zeros({B, H, capacity, D}, dtype);

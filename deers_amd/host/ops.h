@@ -101,6 +101,11 @@ class MatMul : public TensorOp {
 // src/ops.rs:1205).  Returns a compact [B,H,T,D] tensor and keeps (O, LSE) for the
 // backward, which overwrites fresh dq/dk/dv buffers and hands them to
 // GradientStore::accumulate.
+// Head widths the fused kernels do not take (they take 32, 64, 128; the reference's own GPT
+// test runs head_dim 2, tests/gpt.rs:38-49) go through the reference's op chain on the
+// device instead, kernel by kernel (src/models/gpt.rs:139-144 forward; the backward bodies of
+// src/ops.rs:1089-1101, 422-425, 1186-1251, 638-643), materialising [B,H,T,T] tensors the
+// way the reference does; same op, same contract, only slower.
 class FusedCausalAttention : public TensorOp {
  public:
   FusedCausalAttention(Tensor q, Tensor k, Tensor v, double scale);
@@ -113,6 +118,11 @@ class FusedCausalAttention : public TensorOp {
   Tensor q_, k_, v_;
   double scale_;
   Tensor saved_o_, saved_lse_;  // set by forward, created with no op
+  Tensor saved_p_, saved_lsm_;  // composed path: softmax [B,H,T,T] and its logarithm
+
+  static bool fused_kernels_take(int64_t D) { return D == 32 || D == 64 || D == 128; }
+  static Tensor forward_composed(std::unique_ptr<FusedCausalAttention> self);
+  void backward_composed(GradientStore& grads, const Tensor& out_grad) const;
 };
 
 // src/ops.rs:1186-1251: log-softmax over the last axis in one kernel, its output saved

@@ -291,7 +291,8 @@ int deers_rocm_index_select(int dtype, const void* table, const int64_t* indices
  * (src/storage.rs:272-280; CPU src/storage/cpu.rs:612-660, 954-975), the backward of
  * index_select (src/ops.rs:1429-1447).  dst [n_rows, width] is accumulated into (zero
  * it first for the reference's semantics); additions happen in the reference's order,
- * so the result is the same bits and reproducible.  At most 2^18 indices per call. */
+ * so the result is the same bits and reproducible (any number of indices: the library
+ * walks long index vectors in slices, in order). */
 int deers_rocm_index_add(int dtype, const void* src, const int64_t* indices, void* dst,
                          int64_t n_rows, int64_t n_indices, int64_t width);
 /* index_select / index_add along a dimension other than the first
@@ -530,7 +531,9 @@ int deers_rocm_matmul_tune(int on);
  * (src/models/gpt.rs:49-73: narrow, 4 multiplies, 2 adds, cat) followed by
  * permute([0,2,1,3]).  cos and sin are the [1,T,1,D/2] tables of
  * precompute_rotary_embeddings (src/models/gpt.rs:12-47), compact, in the tensor's
- * dtype.  D/2 must be a multiple of 16 bytes; arithmetic is f32 with one rounding. */
+ * dtype.  Any even D: rows that are whole aligned 16-byte chunks on both sides take the
+ * vectorised kernel, everything else (the reference's GPT test runs head_dim 2,
+ * tests/gpt.rs:38-49) one pair per thread; arithmetic is f32 with one rounding. */
 
 /* y [B,H,T,D] = permute(apply_rotary_emb(x)), x logical [B,T,H,D] with element
  * strides x_strides = {b,t,h,d} (NULL = compact, d must be 1).  y is compact, or has

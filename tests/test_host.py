@@ -226,25 +226,37 @@ def test_host_adamw_and_clip_grad_norm_match_oracle(tmp_path, dtype, max_norm):
         assert np.array_equal(out(name), want, equal_nan=True), name
 
 
+REFERENCE_TEST_CFG = dict(vocab_size=8, sequence_len=4, n_layer=1, n_head=2, n_embd=4, mlp_hidden_dim=8,
+                          rms_norm_eps=1e-5, rope_base=10000.0)  # tests/gpt.rs:38-49: head_dim 2
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("cfg,B,T", [
     (dict(vocab_size=37, sequence_len=16, n_layer=2, n_head=2, n_embd=64, mlp_hidden_dim=96,
           rms_norm_eps=1e-5, rope_base=10000.0), 3, 11),
     (dict(vocab_size=300, sequence_len=160, n_layer=3, n_head=3, n_embd=192, mlp_hidden_dim=256,
           rms_norm_eps=1e-5, rope_base=10000.0), 2, 130),
-])
+    (REFERENCE_TEST_CFG, 2, 3),
+    (dict(vocab_size=50, sequence_len=40, n_layer=2, n_head=2, n_embd=12, mlp_hidden_dim=20,
+          rms_norm_eps=1e-5, rope_base=10000.0), 3, 37),  # head_dim 6
+], ids=["d32", "d64", "reference-test-geometry-d2", "d6"])
 def test_host_gpt_training_step_matches_oracle(tmp_path, cfg, B, T):
     """GPT forward, cross-entropy, backward and AdamW steps of the C++ host (f32) against
     the composed numpy oracle, the way tests/gpt.rs compares the reference with a library
-    model.  (The reference's own test geometry has head_dim 2; the device kernels take
-    head widths 32, 64 and 128.)"""
+    model.  Head widths 32 and 64 run the fused attention kernels; the reference's own test
+    geometry (head_dim 2, its token ids and targets, tests/gpt.rs:38-65) and a head_dim 6
+    model run the same op through the unfused device chain and the per-pair RoPE kernel."""
     import oracle
     from oracle import gpt as ogpt
     from test_oracle_gpt import make_weights
     rng = np.random.default_rng(17)
-    ids = rng.integers(0, cfg["vocab_size"], (B, T)).astype(np.int64)
-    ids[1, 2:6] = ids[0, 0]
-    targets = rng.integers(0, cfg["vocab_size"], B * T).astype(np.int64)
+    if cfg is REFERENCE_TEST_CFG:
+        ids = np.array([[1, 2, 3], [4, 3, 2]], np.int64)
+        targets = np.array([2, 3, 4, 3, 2, 1], np.int64)
+    else:
+        ids = rng.integers(0, cfg["vocab_size"], (B, T)).astype(np.int64)
+        ids[1, 2:6] = ids[0, 0]
+        targets = rng.integers(0, cfg["vocab_size"], B * T).astype(np.int64)
     w = make_weights(cfg, 19, dtype=np.float32)
     for i, a in enumerate(w):
         a.tofile(tmp_path / f"w{i}.bin")

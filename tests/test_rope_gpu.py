@@ -8,7 +8,8 @@ from deers_amd import rocm, synth
 
 TOL = {np.dtype(np.float16): 5e-3, np.dtype(np.float32): 1e-4}
 
-SHAPES = [(1, 1, 1, 32), (2, 5, 3, 32), (2, 33, 3, 64), (1, 130, 2, 128), (8, 1024, 12, 64)]
+SHAPES = [(1, 1, 1, 32), (2, 5, 3, 32), (2, 33, 3, 64), (1, 130, 2, 128), (8, 1024, 12, 64),
+          (2, 3, 2, 2), (1, 7, 3, 6), (2, 9, 2, 24), (1, 4, 2, 40)]  # the last four: one pair per thread
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -94,8 +95,8 @@ def test_rope_strided_views_and_errors():
     rocm.rope_bwd_raw(np.float16, ddy_bthd.ptr, dc.ptr, ds.ptr, g2.ptr, B, T, H, D,
                       dy_strides=(T * H * D, D, H * D, 1))
     assert np.array_equal(g1.numpy(), g2.numpy())
-    with pytest.raises(rocm.RocmError):  # D/2 not a multiple of 16 bytes
-        rocm.rope_fwd_raw(np.float16, dq.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, 24)
+    with pytest.raises(rocm.RocmError):  # odd head width
+        rocm.rope_fwd_raw(np.float16, dq.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, 23)
     with pytest.raises(rocm.RocmError):  # innermost stride must be 1
         rocm.rope_fwd_raw(np.float16, dq.ptr, dc.ptr, ds.ptr, y.ptr, B, T, H, D,
                           x_strides=(T * H * D, H * D, D, 2))
