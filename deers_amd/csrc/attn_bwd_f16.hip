@@ -200,29 +200,42 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
   }
   const float c = p.scale_log2;
 
-  // One 32-query block of the tile in `slot`: MASKED applies the causal element mask.
-  auto block = [&](auto masked, const char* slot, int mb, int qb0) {
+  // Per-iteration LDS read addresses: slot base + per-lane offset, one add each; everything
+  // else (second 32-row block, dO tile, contraction step) is an instruction offset.
+  uint32_t a_at[KS], t_lo_at[DB], t_hi_at[DB], vec_at;
+  auto set_slot = [&](uint32_t slot) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a_at[ks] = opaque(slot + aoff[ks]);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      t_lo_at[db] = opaque(slot + toff_lo[db]);
+      t_hi_at[db] = opaque(slot + toff_hi[db]);
+    }
+    vec_at = opaque(slot + 2 * TILE_B + 16 * g);
+  };
+
+  // One 32-query block of the current slot: MASKED applies the causal element mask.
+  auto block = [&](auto masked, auto mb_c, int qb0) {
     constexpr bool MASKED = decltype(masked)::value;
-    const char* Qt = slot + 32 * mb * RB;
-    const char* dOt = slot + TILE_B + 32 * mb * RB;
-    const float* l2v = (const float*)(slot + 2 * TILE_B) + 32 * mb + 4 * g;
-    const float* ndv = (const float*)(slot + 2 * TILE_B + VEC_B) + 32 * mb + 4 * g;
+    constexpr int MB = decltype(mb_c)::value;
+    constexpr uint32_t QT = 32 * MB * RB;            // Q rows of this block
+    constexpr uint32_t DOT = TILE_B + 32 * MB * RB;  // dO rows of this block
     // dP starts from -delta[q] (row value of every accumulator register)
     floatx16 s = ZERO16, dp;
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
-      const floatx4 nd = *(const floatx4*)(ndv + 8 * rq);
+      const floatx4 nd = lds_read_float4_at(vec_at + VEC_B + 128 * MB + 32 * rq);
 #pragma unroll
       for (int e = 0; e < 4; ++e) dp[4 * rq + e] = nd[e];
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      s = mfma_f16(*(const half8*)(Qt + aoff[ks]), kf[ks], s);
-      dp = mfma_f16(*(const half8*)(dOt + aoff[ks]), vf[ks], dp);
+      s = mfma_f16(lds_read_half8_at(a_at[ks] + QT), kf[ks], s);
+      dp = mfma_f16(lds_read_half8_at(a_at[ks] + DOT), vf[ks], dp);
     }
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
-      const floatx4 l4 = *(const floatx4*)(l2v + 8 * rq);
+      const floatx4 l4 = lds_read_float4_at(vec_at + 128 * MB + 32 * rq);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int r = 4 * rq + e;
@@ -243,14 +256,12 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
                      dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const char* tb = dOt + 16 * st * RB;
-        const half4 lo = lds_read_tr16((const half_t*)(tb + toff_lo[db]));
-        const half4 hi = lds_read_tr16((const half_t*)(tb + toff_hi[db]));
+        const half4 lo = lds_read_tr16_at(t_lo_at[db] + DOT + 16 * st * RB);
+        const half4 hi = lds_read_tr16_at(t_hi_at[db] + DOT + 16 * st * RB);
         dvacc[db] = mfma_f16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), pf,
                              dvacc[db]);
-        const char* tq = Qt + 16 * st * RB;
-        const half4 qlo = lds_read_tr16((const half_t*)(tq + toff_lo[db]));
-        const half4 qhi = lds_read_tr16((const half_t*)(tq + toff_hi[db]));
+        const half4 qlo = lds_read_tr16_at(t_lo_at[db] + QT + 16 * st * RB);
+        const half4 qhi = lds_read_tr16_at(t_hi_at[db] + QT + 16 * st * RB);
         dkacc[db] = mfma_f16(__builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7), dsf,
                              dkacc[db]);
       }
@@ -267,17 +278,18 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     wait_vmcnt<(P - 1) * LPI>();
     __syncthreads();
     request(j + P);
-    const char* slot = smem + (j % NS) * SLOT_B;
+    set_slot(lds0 + (j % NS) * SLOT_B);
     const int q0 = j * kBwdStep;
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      const int qb0 = q0 + 32 * mb;   // first query row of this 32-block
-      if (qb0 + 31 < kvw0) continue;  // every query here precedes the wave's keys
+    auto one = [&](auto mb_c) {
+      const int qb0 = q0 + 32 * decltype(mb_c)::value;  // first query row of this 32-block
+      if (qb0 + 31 < kvw0) return;                       // every query here precedes the wave's keys
       if (qb0 < kvw0 + 31)
-        block(yes, slot, mb, qb0);
+        block(yes, mb_c, qb0);
       else
-        block(no, slot, mb, qb0);
-    }
+        block(no, mb_c, qb0);
+    };
+    one(std::integral_constant<int, 0>{});
+    one(std::integral_constant<int, 1>{});
   }
 
   if (kvrow < T) {
@@ -423,15 +435,27 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
   for (int i = 0; i < DB; ++i) dqacc[i] = ZERO16;
   const float c = p.scale_log2;
 
-  auto block = [&](auto masked, const char* slot, int mb, int kvb0) {
+  uint32_t a_at[KS], t_lo_at[DB], t_hi_at[DB];  // per-iteration LDS read addresses (see dK/dV)
+  auto set_slot = [&](uint32_t slot) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a_at[ks] = opaque(slot + aoff[ks]);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      t_lo_at[db] = opaque(slot + toff_lo[db]);
+      t_hi_at[db] = opaque(slot + toff_hi[db]);
+    }
+  };
+
+  auto block = [&](auto masked, auto mb_c, int kvb0) {
     constexpr bool MASKED = decltype(masked)::value;
-    const char* Kt = slot + 32 * mb * RB;
-    const char* Vt = slot + TILE_B + 32 * mb * RB;
+    constexpr int MB = decltype(mb_c)::value;
+    constexpr uint32_t KT = 32 * MB * RB;           // K rows of this block
+    constexpr uint32_t VT = TILE_B + 32 * MB * RB;  // V rows of this block
     floatx16 s = ZERO16, dp = nd16;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      s = mfma_f16(*(const half8*)(Kt + aoff[ks]), qf[ks], s);
-      dp = mfma_f16(*(const half8*)(Vt + aoff[ks]), dof[ks], dp);
+      s = mfma_f16(lds_read_half8_at(a_at[ks] + KT), qf[ks], s);
+      dp = mfma_f16(lds_read_half8_at(a_at[ks] + VT), dof[ks], dp);
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -448,9 +472,8 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
                      dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const char* tb = Kt + 16 * st * RB;
-        const half4 lo = lds_read_tr16((const half_t*)(tb + toff_lo[db]));
-        const half4 hi = lds_read_tr16((const half_t*)(tb + toff_hi[db]));
+        const half4 lo = lds_read_tr16_at(t_lo_at[db] + KT + 16 * st * RB);
+        const half4 hi = lds_read_tr16_at(t_hi_at[db] + KT + 16 * st * RB);
         dqacc[db] = mfma_f16(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7), dsf,
                              dqacc[db]);
       }
@@ -470,17 +493,18 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
                          __HIP_MEMORY_SCOPE_AGENT);
     }
     request(j + P);
-    const char* slot = smem + (j % NS) * 2 * TILE_B;
+    set_slot(lds0 + (j % NS) * 2 * TILE_B);
     const int kv0 = j * kBwdStep;
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      const int kvb0 = kv0 + 32 * mb;
-      if (kvb0 > qw0 + 31) continue;  // block lies entirely in this wave's future
+    auto one = [&](auto mb_c) {
+      const int kvb0 = kv0 + 32 * decltype(mb_c)::value;
+      if (kvb0 > qw0 + 31) return;  // block lies entirely in this wave's future
       if (kvb0 + 31 > qw0)
-        block(yes, slot, mb, kvb0);
+        block(yes, mb_c, kvb0);
       else
-        block(no, slot, mb, kvb0);
-    }
+        block(no, mb_c, kvb0);
+    };
+    one(std::integral_constant<int, 0>{});
+    one(std::integral_constant<int, 1>{});
   }
 
   if (qrow < T) {

@@ -1,11 +1,30 @@
 // Fused causal attention backward, f32 storage and arithmetic, gfx950.
 //
-// Same three launches and orientations as the f16 backward (delta, dK/dV with
-// one key column per lane, dQ with one query column per lane) on
-// v_mfma_f32_32x32x2_f32.  One contraction element per lane per MFMA means the
-// accumulator registers of P / dS are B operands as they are, and the
-// "transposed" A fragments are ordinary 4-byte reads of the row-major LDS tiles.
-// Contraction over D gives lane group g the contiguous half [g*D/2, (g+1)*D/2).
+// v_mfma_f32_32x32x2_f32 runs at 1/16 of the f16 matrix rate, so these kernels are bound
+// by the matrix pipe alone (a 32x32 score block costs 160 MFMAs = ~10 k cycles with 5 tile
+// GEMMs; its softmax a few hundred).  Head widths 32 and 64 therefore take the ONE-PASS
+// form, 5 tile GEMMs per block instead of the 7 of a dQ pass plus a dK/dV pass:
+//   1. prep : delta = rowsum(dO o O) per query row, and dQ cleared.
+//   2. main : a workgroup owns 128 keys (32 per wave, K and V rows in registers as B
+//             operands) and walks the 32-row query tiles at or below the diagonal:
+//             S = Q K^T, dP = dO V^T, P = exp2(S*scale*log2e - lse2), dS = P o (dP - delta),
+//             dV^T += dO^T P, dK^T += Q^T dS; scale*dS goes to LDS as [128 keys][32
+//             queries], and after a barrier the waves share out
+//             dQ[q,d] += (scale dS)[q, 128 keys] K[128 keys, d]
+//             (K block resident in LDS) and add their blocks to dQ with no-return f32
+//             atomics: 2 k adds per 10 k cycles of MFMA work, far below what the L2
+//             atomic units sustain.  (For the f16 kernels, 16x faster per block, the same
+//             scheme lost to the atomics.)
+//           dQ sums the contributions of up to T/128 key blocks in arrival order: it is
+//           reproducible to f32 rounding (~1e-7 relative), not bit for bit; dK and dV are
+//           bit-reproducible.
+// One contraction element per lane per MFMA means the accumulator registers of P / dS are B
+// operands as they are, and the "transposed" A fragments are ordinary 4-byte reads of the
+// row-major LDS tiles.  Contraction over D gives lane group g the contiguous half
+// [g*D/2, (g+1)*D/2).
+// Head width 128 keeps the earlier three launches (delta, dK/dV with one key column per
+// lane, dQ with one query column per lane): its K block and exchange tile do not fit LDS
+// beside the streamed tiles.
 #include "common.h"
 #include "bwd_delta.h"
 
@@ -351,6 +370,291 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(BwdParams p, int B
   }
 }
 
+// ---------------------------------------------------------------------------
+// one-pass form (D = 32, 64)
+// ---------------------------------------------------------------------------
+// delta[b,h,t] = sum_d dO*O, and the dQ row cleared for the main kernel's atomic adds.
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_prep_f32_kernel(BwdParams p, int B) {
+  constexpr int LPR = D / 4;  // lanes per row, 16 bytes each
+  const int64_t rows = (int64_t)B * p.H * p.T;
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+  const int part = threadIdx.x % LPR;
+  float acc = 0.f;
+  if (row < rows) {
+    const int t = row % p.T;
+    const int bh = row / p.T;
+    const int b = bh / p.H, h = bh % p.H;
+    const float* o = (const float*)p.o + b * p.so.b + h * p.so.h + (int64_t)t * p.so.t + 4 * part;
+    const float* d = (const float*)p.d_o + b * p.sdo.b + h * p.sdo.h + (int64_t)t * p.sdo.t + 4 * part;
+    const floatx4 ov = *(const floatx4*)o, dv = *(const floatx4*)d;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc += ov[e] * dv[e];
+    *(floatx4*)((float*)p.dq + b * p.sdq.b + h * p.sdq.h + (int64_t)t * p.sdq.t + 4 * part) = ZEROF4;
+  }
+#pragma unroll
+  for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (row < rows && part == 0) p.delta[row] = acc;
+}
+
+template <int D>
+struct Fused32Cfg {
+  static constexpr int STEP = 32;        // query rows per iteration
+  static constexpr int LD = D + 4;       // row pitch of the Q, dO, K tiles (floats)
+  static constexpr int LDS_DS = STEP + 4;  // row pitch of the dS^T exchange tile
+  static constexpr int kFloats = 2 * STEP * LD + 2 * STEP + kBwd32Blk * LD + kBwd32Blk * LDS_DS;
+  static constexpr size_t kLds = kFloats * sizeof(float);
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_fused_f32_kernel(BwdParams p, int BH, int n_blocks,
+                                                                 int heads_per_xcd) {
+  using Cfg = Fused32Cfg<D>;
+  constexpr int STEP = Cfg::STEP, LD = Cfg::LD, LDS_DS = Cfg::LDS_DS;
+  constexpr int KH = D / 2;
+  constexpr int DB = D / 32;
+  constexpr int CH = D / 4;
+  constexpr int NLOAD = STEP * CH / 256;       // 16-byte loads per thread per streamed tile
+  constexpr int NKLOAD = kBwd32Blk * CH / 256;  // ... for the resident K block
+  // dQ tile of an iteration: 32 queries x D = DB blocks of 32x32, shared out over the four
+  // waves: wave w takes block w % DB over the keys [KPW * (w / DB), + KPW)
+  constexpr int KV_SPLIT = 4 / DB;
+  constexpr int KPW = kBwd32Blk / KV_SPLIT;
+  static_assert(NLOAD >= 1 && DB >= 1 && DB <= 2, "head width 32 or 64");
+
+  extern __shared__ __attribute__((aligned(16))) float smem32[];
+  float* Qs = smem32;
+  float* dOs = Qs + STEP * LD;
+  float* lse2s = dOs + STEP * LD;
+  float* deltas = lse2s + STEP;
+  float* Ks = deltas + STEP;           // the workgroup's 128 K rows, for dQ = dS K
+  float* dSs = Ks + kBwd32Blk * LD;    // scale * dS^T of the current tile: [128 keys][32 queries]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5;
+  const int T = p.T;
+  int bh, rank;
+  if (!map_block(blockIdx.x, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
+  const int kvblk = rank;  // key block 0 walks the most query tiles
+  const int b = bh / p.H, h = bh % p.H;
+
+  const float* Q = (const float*)p.q + b * p.sq.b + h * p.sq.h;
+  const float* K = (const float*)p.k + b * p.sk.b + h * p.sk.h;
+  const float* V = (const float*)p.v + b * p.sv.b + h * p.sv.h;
+  const float* dO = (const float*)p.d_o + b * p.sdo.b + h * p.sdo.h;
+  float* dQ = (float*)p.dq + b * p.sdq.b + h * p.sdq.h;
+  float* dK = (float*)p.dk + b * p.sdk.b + h * p.sdk.h;
+  float* dV = (float*)p.dv + b * p.sdv.b + h * p.sdv.h;
+  const float* lse = p.lse + (int64_t)bh * T;
+  const float* delta = p.delta + (int64_t)bh * T;
+
+  const int kv0 = kvblk * kBwd32Blk;
+  const int kvw0 = kv0 + 32 * wave;
+  const int kvrow = kvw0 + (lane & 31);
+
+  // K block -> LDS (rows past T-1 as zeros: their dS is zero anyway)
+#pragma unroll
+  for (int i = 0; i < NKLOAD; ++i) {
+    const int idx = tid + 256 * i;
+    const int row = idx / CH, ch = idx % CH;
+    floatx4 t = ZEROF4;
+    if (kv0 + row < T) t = *(const floatx4*)(K + (int64_t)(kv0 + row) * p.sk.t + 4 * ch);
+    *(floatx4*)(Ks + row * LD + 4 * ch) = t;
+  }
+
+  float kf[KH], vf[KH];
+#pragma unroll
+  for (int c = 0; c < KH / 4; ++c) {
+    floatx4 tk = ZEROF4, tv = ZEROF4;
+    if (kvrow < T) {
+      tk = *(const floatx4*)(K + (int64_t)kvrow * p.sk.t + g * KH + 4 * c);
+      tv = *(const floatx4*)(V + (int64_t)kvrow * p.sv.t + g * KH + 4 * c);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      kf[4 * c + e] = tk[e];
+      vf[4 * c + e] = tv[e];
+    }
+  }
+
+  floatx16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    dkacc[i] = ZERO16;
+    dvacc[i] = ZERO16;
+  }
+
+  const int first_tile = kv0 / STEP;
+  const int n_tiles = (T + STEP - 1) / STEP;
+
+  floatx4 qreg[NLOAD], doreg[NLOAD];
+  float lreg = 0.f, dreg = 0.f;
+  auto prefetch = [&](int tile) {
+    const int q0 = tile * STEP;
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+      const int idx = tid + 256 * i;
+      const int row = idx / CH, ch = idx % CH;
+      const int qr = q0 + row;
+      if (qr < T) {
+        qreg[i] = *(const floatx4*)(Q + (int64_t)qr * p.sq.t + 4 * ch);
+        doreg[i] = *(const floatx4*)(dO + (int64_t)qr * p.sdo.t + 4 * ch);
+      } else {
+        qreg[i] = ZEROF4;
+        doreg[i] = ZEROF4;
+      }
+    }
+    if (tid < STEP) {
+      const int qr = q0 + tid;
+      lreg = qr < T ? lse[qr] * kLog2e : 0.f;
+      dreg = qr < T ? delta[qr] : 0.f;
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+      const int idx = tid + 256 * i;
+      const int row = idx / CH, ch = idx % CH;
+      *(floatx4*)(Qs + row * LD + 4 * ch) = qreg[i];
+      *(floatx4*)(dOs + row * LD + 4 * ch) = doreg[i];
+    }
+    if (tid < STEP) {
+      lse2s[tid] = lreg;
+      deltas[tid] = dreg;
+    }
+  };
+
+  const int my_db = wave % DB;
+  const int my_kv = KPW * (wave / DB);  // first key (within the block) of this wave's dQ share
+
+  prefetch(first_tile);
+  for (int j = first_tile; j < n_tiles; ++j) {
+    __syncthreads();  // the previous tile's readers (Qs, dOs, dSs) are done
+    commit();
+    __syncthreads();
+    if (j + 1 < n_tiles) prefetch(j + 1);
+
+    const int qb0 = j * STEP;
+    if (qb0 + 31 >= kvw0) {  // else every query here precedes the wave's keys
+      floatx16 s = ZERO16, dp = ZERO16;
+      const float* qrow_p = Qs + (lane & 31) * LD + g * KH;
+      const float* dorow_p = dOs + (lane & 31) * LD + g * KH;
+#pragma unroll
+      for (int c = 0; c < KH / 4; ++c) {
+        const floatx4 a = *(const floatx4*)(qrow_p + 4 * c);
+        const floatx4 a2 = *(const floatx4*)(dorow_p + 4 * c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s = mfma_f32(a[e], kf[4 * c + e], s);
+          dp = mfma_f32(a2[e], vf[4 * c + e], dp);
+        }
+      }
+
+      const bool need_mask = (qb0 < kvw0 + 31);
+      float* ds_row = dSs + (32 * wave + (lane & 31)) * LDS_DS + 4 * g;
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const floatx4 l4 = *(const floatx4*)(lse2s + 8 * rq + 4 * g);
+        const floatx4 d4 = *(const floatx4*)(deltas + 8 * rq + 4 * g);
+        floatx4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * rq + e;
+          float pv = fast_exp2(s[r] * p.scale_log2 - l4[e]);
+          if (need_mask) {
+            const int qr = qb0 + 8 * rq + 4 * g + e;
+            if (kvrow > qr) pv = 0.f;
+          }
+          s[r] = pv;
+          dp[r] = pv * (dp[r] - d4[e]);
+          out[e] = dp[r] * p.scale;
+        }
+        *(floatx4*)(ds_row + 8 * rq) = out;
+      }
+
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * g + (r & 3);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const float ado = dOs[row * LD + 32 * db + (lane & 31)];
+          dvacc[db] = mfma_f32(ado, s[r], dvacc[db]);
+          const float aq = Qs[row * LD + 32 * db + (lane & 31)];
+          dkacc[db] = mfma_f32(aq, dp[r], dkacc[db]);
+        }
+      }
+    }
+    __syncthreads();  // scale * dS^T of this tile is complete
+
+    // dQ[q, d-block] += sum over this wave's keys of dS[q, kv] K[kv, d]; key sub-blocks
+    // whose wave skipped the tile hold no data: only the first live_kv keys do
+    {
+      const int live_kv = min(kBwd32Blk, qb0 + 32 - kv0);
+      const int n_pairs = max(0, min(KPW, live_kv - my_kv)) / 2;
+      floatx16 acc = ZERO16;
+      const float* a_p = dSs + (my_kv + g) * LDS_DS + (lane & 31);
+      const float* b_p = Ks + (my_kv + g) * LD + 32 * my_db + (lane & 31);
+#pragma unroll 8
+      for (int t = 0; t < n_pairs; ++t)
+        acc = mfma_f32(a_p[2 * t * LDS_DS], b_p[2 * t * LD], acc);
+      if (n_pairs > 0) {
+        float* dst = dQ + (int64_t)(qb0 + 4 * g) * p.sdq.t + 32 * my_db + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qo = 8 * (r >> 2) + (r & 3);
+          if (qb0 + 4 * g + qo < T) unsafeAtomicAdd(dst + (int64_t)qo * p.sdq.t, acc[r]);
+        }
+      }
+    }
+  }
+
+  if (kvrow < T) {
+    float* dkrow = dK + (int64_t)kvrow * p.sdk.t;
+    float* dvrow = dV + (int64_t)kvrow * p.sdv.t;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        floatx4 ok, ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ok[e] = dkacc[db][4 * rq + e] * p.scale;
+          ov[e] = dvacc[db][4 * rq + e];
+        }
+        *(floatx4*)(dkrow + 32 * db + 8 * rq + 4 * g) = ok;
+        *(floatx4*)(dvrow + 32 * db + 8 * rq + 4 * g) = ov;
+      }
+  }
+}
+
+template <int D>
+static void launch_bwd_fused_f32_d(const BwdParams& p, int B, hipStream_t stream) {
+  const int64_t rows = (int64_t)B * p.H * p.T;
+  constexpr int LPR = D / 4;
+  const int64_t threads = rows * LPR;
+  {
+    LaunchScope scope("attn_bwd_prep_f32", stream);
+    hipLaunchKernelGGL((attn_bwd_prep_f32_kernel<D>), dim3((threads + 255) / 256), dim3(256), 0, stream,
+                       p, B);
+  }
+  const int BH = B * p.H;
+  const int n_blocks = (p.T + kBwd32Blk - 1) / kBwd32Blk;
+  const int heads_per_xcd = (BH + 7) / 8;
+  constexpr size_t lds = Fused32Cfg<D>::kLds;
+  static bool attr_set = false;  // launches are serialised by the caller
+  if (!attr_set) {
+    if (lds > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_bwd_fused_f32_kernel<D>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    attr_set = true;
+  }
+  LaunchScope scope("attn_bwd_f32", stream);
+  hipLaunchKernelGGL((attn_bwd_fused_f32_kernel<D>), dim3(8 * n_blocks * heads_per_xcd), dim3(256), lds,
+                     stream, p, BH, n_blocks, heads_per_xcd);
+}
+
 template <int D, int STEP>
 static void launch_bwd_f32_d(const BwdParams& p, int B, hipStream_t stream) {
   const int64_t rows = (int64_t)B * p.H * p.T;
@@ -379,8 +683,8 @@ static void launch_bwd_f32_d(const BwdParams& p, int B, hipStream_t stream) {
 
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream) {
   switch (D) {
-    case 32: launch_bwd_f32_d<32, 64>(p, B, stream); break;
-    case 64: launch_bwd_f32_d<64, 64>(p, B, stream); break;
+    case 32: launch_bwd_fused_f32_d<32>(p, B, stream); break;
+    case 64: launch_bwd_fused_f32_d<64>(p, B, stream); break;
     case 128: launch_bwd_f32_d<128, 32>(p, B, stream); break;
   }
 }

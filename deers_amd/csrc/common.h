@@ -95,6 +95,15 @@ __device__ __forceinline__ uint32_t opaque(uint32_t x) {
   return x;
 }
 
+// 16-byte reads from a 32-bit LDS byte address (constant parts of the address written as
+// "+ constant" at the call site end up in the instruction's offset field).
+__device__ __forceinline__ half8 lds_read_half8_at(uint32_t lds_addr) {
+  return *(DEERS_LDS const half8*)(uintptr_t)lds_addr;
+}
+__device__ __forceinline__ floatx4 lds_read_float4_at(uint32_t lds_addr) {
+  return *(DEERS_LDS const floatx4*)(uintptr_t)lds_addr;
+}
+
 // Same read from a 32-bit LDS byte address.
 __device__ __forceinline__ half4 lds_read_tr16_at(uint32_t lds_addr) {
   fp16x4_raw r =

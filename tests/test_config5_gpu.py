@@ -49,8 +49,11 @@ def test_f32_attention_at_config5_size_matches_oracle_and_is_reproducible():
     np.testing.assert_array_equal(o[:, :, 0], v[:, :, 0])  # the first query sees only itself
     assert np.max(np.abs(dq[:, :, 0])) <= 1e-5             # ... so dS = P (dP - delta) cancels to rounding
     o2, lse2, dq2, dk2, dv2 = rocm.attn_fwd_bwd(q, k, v, do)
-    for a, b_ in ((o, o2), (lse, lse2), (dq, dq2), (dk, dk2), (dv, dv2)):
-        np.testing.assert_array_equal(a, b_)               # no atomics anywhere: bit-reproducible
+    for a, b_ in ((o, o2), (lse, lse2), (dk, dk2), (dv, dv2)):
+        np.testing.assert_array_equal(a, b_)               # bit-reproducible
+    # dQ adds the contributions of its (up to 8) key blocks with f32 atomics in arrival order:
+    # reproducible to f32 rounding of that sum
+    assert np.max(np.abs(dq - dq2)) <= 1e-6
 
 
 def test_gpt_training_step_at_baseline_geometry_learns():
