@@ -92,13 +92,13 @@ def test_host_fused_attention_matches_oracle(tmp_path, dtype, B, H, T, D, L, tol
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,B,T,C,H,tol", [
     (np.float32, 2, 70, 128, 4, 2e-4),
-    (np.float16, 2, 200, 256, 4, 2e-2),
+    (np.float16, 2, 200, 256, 4, 5e-3),
 ])
 def test_host_attention_module_matches_composed_oracle(tmp_path, dtype, B, T, C, H, tol):
     """x -> q/k/v projections -> RoPE -> causal attention -> head merge -> out projection
-    (src/models/gpt.rs:101-147) and its backward, against the same chain on the CPU oracle.
-    f16 tolerance: four GEMMs with f16 outputs around the core (the reference's own f16
-    helper uses 1e-2, tests/utils.rs:14; gradients of the weights sum over B*T rows)."""
+    (src/models/gpt.rs:101-147) and its backward, against the same chain on the CPU oracle
+    (rounded to f16 where the device rounds).  Tolerance: the path's 5e-3 (f16) per unit of
+    the tensor's largest value (weight gradients sum over B*T rows and reach tens)."""
     import oracle
     rng = np.random.default_rng(41)
     D = C // H
@@ -134,11 +134,12 @@ def test_host_attention_module_matches_composed_oracle(tmp_path, dtype, B, T, C,
     want = {"dwq": mm(xf.T, dq), "dwk": mm(xf.T, dk), "dwv": mm(xf.T, dv), "dwo": want_dwo,
             "dx": mm(dq, wq.T) + mm(dk, wk.T) + mm(dv, wv.T)}
     got = lambda name, shape: np.fromfile(tmp_path / f"{name}.bin", dtype=dtype).reshape(shape).astype(np.float64)
-    assert np.max(np.abs(got("y", (B * T, C)) - want_y)) <= tol
+    ytol = tol * max(1.0, float(np.max(np.abs(want_y))))
+    assert np.max(np.abs(got("y", (B * T, C)) - want_y)) <= ytol
     if dtype == np.float16:
         # token-by-token generation through the KV cache reproduces the full forward's rows
-        assert np.max(np.abs(got("y_decode", (B * T, C)) - want_y)) <= tol
-        assert np.max(np.abs(got("y_decode", (B * T, C)) - got("y", (B * T, C)))) <= tol
+        assert np.max(np.abs(got("y_decode", (B * T, C)) - want_y)) <= ytol
+        assert np.max(np.abs(got("y_decode", (B * T, C)) - got("y", (B * T, C)))) <= ytol
     for name, ref in want.items():
         g = got(name, ref.shape)
         scale = max(1.0, float(np.max(np.abs(ref))))
