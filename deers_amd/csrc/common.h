@@ -225,6 +225,11 @@ struct FwdParams {
   float scale_log2;  // scale * log2(e)
 };
 
+// Whether the single-launch f16 backward runs its dQ groups shortest first: when a group
+// (one block length over all heads) is at least an eighth of the workgroups the device
+// holds at once (attn_bwd_f16.hip).
+inline bool bwd_dq_short_first(int group_wgs, int capacity) { return 8 * group_wgs >= capacity; }
+
 struct BwdParams {
   const void* q; const void* k; const void* v; const void* o; const void* d_o;
   const float* lse; float* delta;  // delta: [B,H,T] workspace, rowsum(dO o O)
