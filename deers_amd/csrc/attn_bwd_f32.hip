@@ -406,9 +406,13 @@ struct Fused32Cfg {
   static constexpr size_t kLds = kFloats * sizeof(float);
 };
 
+// Two workgroups per CU, so that one's barriers, softmax and atomics run under the other's
+// MFMAs (414 -> 354 us at 8x12x1024x64; three at D = 32 were slower than two, 234 against
+// 218 us).  The bound is needed at D = 64: left free, the compiler spreads into 80
+// accumulation registers it has no use for and a CU holds a single workgroup.
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_fused_f32_kernel(BwdParams p, int BH, int n_blocks,
-                                                                 int heads_per_xcd) {
+__global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
+    BwdParams p, int BH, int n_blocks, int heads_per_xcd) {
   using Cfg = Fused32Cfg<D>;
   constexpr int STEP = Cfg::STEP, LD = Cfg::LD, LDS_DS = Cfg::LDS_DS;
   constexpr int KH = D / 2;
