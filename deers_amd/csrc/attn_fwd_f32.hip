@@ -35,7 +35,7 @@ struct Fwd32Lists {
 };
 
 template <int D, int BN>
-__global__ __launch_bounds__(256, (D == 32 ? 3 : D == 64 ? 2 : 1)) void attn_fwd_f32_kernel(FwdParams p, int BH, int n_qtiles,
+__global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(FwdParams p, int BH, int n_qtiles,
                                                            int heads_per_xcd, const int* lists,
                                                            int max_len) {
   constexpr int LD = D + 4;   // LDS row stride in floats
