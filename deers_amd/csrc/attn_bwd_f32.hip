@@ -25,6 +25,11 @@
 // Head width 128 keeps the earlier three launches (delta, dK/dV with one key column per
 // lane, dQ with one query column per lane): its K block and exchange tile do not fit LDS
 // beside the streamed tiles.
+#include <algorithm>
+#include <map>
+#include <utility>
+#include <vector>
+
 #include "common.h"
 #include "bwd_delta.h"
 
@@ -373,9 +378,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(BwdParams p, int B
 // ---------------------------------------------------------------------------
 // one-pass form (D = 32, 64)
 // ---------------------------------------------------------------------------
-// delta[b,h,t] = sum_d dO*O, and the dQ row cleared for the main kernel's atomic adds.
+// delta[b,h,t] = sum_d dO*O, and what the main kernel adds to with atomics cleared: the dQ
+// row, and the dK and dV rows of the key blocks that two work items share (rows < split_rows).
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_prep_f32_kernel(BwdParams p, int B) {
+__global__ __launch_bounds__(256) void attn_bwd_prep_f32_kernel(BwdParams p, int B, int split_rows) {
   constexpr int LPR = D / 4;  // lanes per row, 16 bytes each
   const int64_t rows = (int64_t)B * p.H * p.T;
   const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
@@ -391,11 +397,21 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_f32_kernel(BwdParams p, int
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc += ov[e] * dv[e];
     *(floatx4*)((float*)p.dq + b * p.sdq.b + h * p.sdq.h + (int64_t)t * p.sdq.t + 4 * part) = ZEROF4;
+    if (t < split_rows) {
+      *(floatx4*)((float*)p.dk + b * p.sdk.b + h * p.sdk.h + (int64_t)t * p.sdk.t + 4 * part) = ZEROF4;
+      *(floatx4*)((float*)p.dv + b * p.sdv.b + h * p.sdv.h + (int64_t)t * p.sdv.t + 4 * part) = ZEROF4;
+    }
   }
 #pragma unroll
   for (int off = LPR / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
   if (row < rows && part == 0) p.delta[row] = acc;
 }
+
+// One workgroup's work in the one-pass kernel: the query tiles [tile_begin, tile_end) (32 rows
+// each) of key block kvblk.  `shared`: the block has a second item and both add to dK / dV.
+struct Bwd32Item {
+  int kvblk, tile_begin, tile_end, shared;
+};
 
 template <int D>
 struct Fused32Cfg {
@@ -412,7 +428,7 @@ struct Fused32Cfg {
 // accumulation registers it has no use for and a CU holds a single workgroup.
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
-    BwdParams p, int BH, int n_blocks, int heads_per_xcd) {
+    BwdParams p, int BH, int n_items, int heads_per_xcd, const Bwd32Item* items) {
   using Cfg = Fused32Cfg<D>;
   constexpr int STEP = Cfg::STEP, LD = Cfg::LD, LDS_DS = Cfg::LDS_DS;
   constexpr int KH = D / 2;
@@ -440,8 +456,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
   const int g = lane >> 5;
   const int T = p.T;
   int bh, rank;
-  if (!map_block(blockIdx.x, n_blocks, heads_per_xcd, BH, &bh, &rank)) return;
-  const int kvblk = rank;  // key block 0 walks the most query tiles
+  if (!map_block(blockIdx.x, n_items, heads_per_xcd, BH, &bh, &rank)) return;
+  const Bwd32Item it = items[rank];  // items are listed longest first
+  const int kvblk = it.kvblk;
   const int b = bh / p.H, h = bh % p.H;
 
   const float* Q = (const float*)p.q + b * p.sq.b + h * p.sq.h;
@@ -490,8 +507,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
     dvacc[i] = ZERO16;
   }
 
-  const int first_tile = kv0 / STEP;
-  const int n_tiles = (T + STEP - 1) / STEP;
+  const int first_tile = it.tile_begin;  // this item's share of the block's query tiles
+  const int n_tiles = it.tile_end;
 
   floatx4 qreg[NLOAD], doreg[NLOAD];
   float lreg = 0.f, dreg = 0.f;
@@ -614,7 +631,36 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
     }
   }
 
-  if (kvrow < T) {
+  if (it.shared) {
+    // The block's other item adds its half too (the prep kernel cleared the rows).  In the
+    // accumulator layout a lane owns a key row, so an atomic instruction would touch 64
+    // cache lines; staged through LDS (the K block's space) each one covers one row's
+    // contiguous floats instead.
+    constexpr int NOUT = kBwd32Blk * D / 256;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      __syncthreads();  // Ks free: dQ products of the last tile / the previous staging are done
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          floatx4 o4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o4[e] = which == 0 ? dkacc[db][4 * rq + e] * p.scale : dvacc[db][4 * rq + e];
+          *(floatx4*)(Ks + (32 * wave + (lane & 31)) * LD + 32 * db + 8 * rq + 4 * g) = o4;
+        }
+      __syncthreads();
+      float* dst = which == 0 ? dK : dV;
+      const int64_t pitch = which == 0 ? p.sdk.t : p.sdv.t;
+#pragma unroll 4
+      for (int i = 0; i < NOUT; ++i) {
+        const int idx = tid + 256 * i;
+        const int row = idx / D, col = idx % D;
+        if (kv0 + row < T) unsafeAtomicAdd(dst + (int64_t)(kv0 + row) * pitch + col, Ks[row * LD + col]);
+      }
+    }
+  } else if (kvrow < T) {
     float* dkrow = dK + (int64_t)kvrow * p.sdk.t;
     float* dvrow = dV + (int64_t)kvrow * p.sdv.t;
 #pragma unroll
@@ -633,30 +679,92 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
   }
 }
 
+// Work items of a launch at sequence length T, longest first, in device memory (built once
+// per (T, split) and kept for the life of the process).  A key block walks the query tiles
+// from its diagonal to the end, so block 0 has twice the mean number of iterations.  When
+// the launch has fewer workgroups than the device holds, blocks with more than half of block
+// 0's iterations are cut into two items of half the range, which add their dK / dV halves
+// with atomics onto cleared rows (a sum of exactly two terms, so dK and dV stay
+// bit-reproducible): 42 -> 29 us at 4x6x256x32, 145 -> 81 us at 3x5x640x64.  A launch that
+// fills the device is bound by CU throughput, not by its longest chain, and the extra
+// prologues and write-outs only cost (354 -> 386 us at 8x12x1024x64): it is not split.
+// split_rows: key rows [0, split_rows) of every head are shared.
+struct Bwd32Items {
+  const Bwd32Item* dev = nullptr;
+  int n_items = 0;
+  int split_rows = 0;
+};
+static Bwd32Items bwd32_items(int T, bool split) {
+  static std::map<std::pair<int, bool>, Bwd32Items> cache;  // launches are serialised by the caller
+  auto it = cache.find({T, split});
+  if (it != cache.end()) return it->second;
+  constexpr int kStep = 32, kTilesPerBlock = kBwd32Blk / kStep;
+  const int n_blocks = (T + kBwd32Blk - 1) / kBwd32Blk;
+  const int n_tiles = (T + kStep - 1) / kStep;
+  std::vector<Bwd32Item> items;
+  Bwd32Items out;
+  for (int kb = 0; kb < n_blocks; ++kb) {
+    const int first = kb * kTilesPerBlock;
+    const int n = n_tiles - first;
+    if (split && 2 * n > n_tiles && n >= 2) {
+      const int mid = first + (n + 1) / 2;
+      items.push_back({kb, first, mid, 1});
+      items.push_back({kb, mid, n_tiles, 1});
+      out.split_rows = std::min(T, (kb + 1) * kBwd32Blk);
+    } else {
+      items.push_back({kb, first, n_tiles, 0});
+    }
+  }
+  std::stable_sort(items.begin(), items.end(), [](const Bwd32Item& a, const Bwd32Item& b) {
+    return a.tile_end - a.tile_begin > b.tile_end - b.tile_begin;
+  });
+  Bwd32Item* dev = nullptr;
+  if (hipMalloc(&dev, items.size() * sizeof(Bwd32Item)) != hipSuccess) return Bwd32Items{};
+  if (hipMemcpy(dev, items.data(), items.size() * sizeof(Bwd32Item), hipMemcpyHostToDevice) !=
+      hipSuccess) {
+    (void)hipFree(dev);
+    return Bwd32Items{};
+  }
+  out.dev = dev;
+  out.n_items = (int)items.size();
+  cache.emplace(std::make_pair(T, split), out);
+  return out;
+}
+
 template <int D>
-static void launch_bwd_fused_f32_d(const BwdParams& p, int B, hipStream_t stream) {
+static bool launch_bwd_fused_f32_d(const BwdParams& p, int B, hipStream_t stream) {
+  constexpr size_t lds = Fused32Cfg<D>::kLds;
+  static bool attr_set = false;  // launches are serialised by the caller
+  static int capacity = 0;       // workgroups of the main kernel the device holds at once
+  if (!attr_set) {
+    if (lds > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_bwd_fused_f32_kernel<D>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    int dev = 0, per_cu = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_bwd_fused_f32_kernel<D>, 256, lds) ==
+            hipSuccess)
+      capacity = per_cu * prop.multiProcessorCount;
+    attr_set = true;
+  }
+  const int n_blocks = (p.T + kBwd32Blk - 1) / kBwd32Blk;
+  const Bwd32Items items = bwd32_items(p.T, (int64_t)n_blocks * B * p.H < capacity);
+  if (!items.dev) return false;
   const int64_t rows = (int64_t)B * p.H * p.T;
   constexpr int LPR = D / 4;
   const int64_t threads = rows * LPR;
   {
     LaunchScope scope("attn_bwd_prep_f32", stream);
     hipLaunchKernelGGL((attn_bwd_prep_f32_kernel<D>), dim3((threads + 255) / 256), dim3(256), 0, stream,
-                       p, B);
+                       p, B, items.split_rows);
   }
   const int BH = B * p.H;
-  const int n_blocks = (p.T + kBwd32Blk - 1) / kBwd32Blk;
   const int heads_per_xcd = (BH + 7) / 8;
-  constexpr size_t lds = Fused32Cfg<D>::kLds;
-  static bool attr_set = false;  // launches are serialised by the caller
-  if (!attr_set) {
-    if (lds > 64 * 1024)
-      (void)hipFuncSetAttribute((const void*)attn_bwd_fused_f32_kernel<D>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    attr_set = true;
-  }
   LaunchScope scope("attn_bwd_f32", stream);
-  hipLaunchKernelGGL((attn_bwd_fused_f32_kernel<D>), dim3(8 * n_blocks * heads_per_xcd), dim3(256), lds,
-                     stream, p, BH, n_blocks, heads_per_xcd);
+  hipLaunchKernelGGL((attn_bwd_fused_f32_kernel<D>), dim3(8 * items.n_items * heads_per_xcd), dim3(256),
+                     lds, stream, p, BH, items.n_items, heads_per_xcd, items.dev);
+  return true;
 }
 
 template <int D, int STEP>
@@ -687,8 +795,13 @@ static void launch_bwd_f32_d(const BwdParams& p, int B, hipStream_t stream) {
 
 void launch_attn_bwd_f32(const BwdParams& p, int B, int D, hipStream_t stream) {
   switch (D) {
-    case 32: launch_bwd_fused_f32_d<32>(p, B, stream); break;
-    case 64: launch_bwd_fused_f32_d<64>(p, B, stream); break;
+    // the two-pass form stands in if the one-pass kernel's item table cannot be allocated
+    case 32:
+      if (!launch_bwd_fused_f32_d<32>(p, B, stream)) launch_bwd_f32_d<32, 64>(p, B, stream);
+      break;
+    case 64:
+      if (!launch_bwd_fused_f32_d<64>(p, B, stream)) launch_bwd_f32_d<64, 64>(p, B, stream);
+      break;
     case 128: launch_bwd_f32_d<128, 32>(p, B, stream); break;
   }
 }
