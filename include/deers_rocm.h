@@ -97,7 +97,9 @@ void* deers_rocm_stream(void);
  * (256 compute units) with no CU mask in the environment. */
 int deers_rocm_handover_policy(int cu_count, int cu_mask_set);
 /* The mode in force (after deers_rocm_init; -1 before), and an override: mode -1 returns
- * to the policy's choice for this device. */
+ * to the policy's choice for this device.  A caller that captures backward calls into a HIP
+ * graph selects STREAM_ORDER first: the single launch's flag epoch is a kernel argument, so
+ * a replayed launch would find its flags already set. */
 int deers_rocm_handover_mode(void);
 int deers_rocm_set_handover_mode(int mode);
 /* Test hook for the bounded wait of the single-launch backward: `spin_limit` polls (the
