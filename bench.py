@@ -70,6 +70,24 @@ def bench_train(steps: int, warmup: int, only: str = "all"):
         if only in ("all", "bwd"):
             bwd()
 
+    # first pass: per-kernel device times over at least KERNEL_PASS_MIN_STEPS steps whatever
+    # `steps` is (`roofline` is computed from this pass), after as many untimed steps.  It
+    # runs before the timed region so that the K timed steps see the device in the state a
+    # long job keeps it in: from idle, the first few milliseconds of launches run 5-8 % slower
+    # while the clocks settle, and K = 20 steps are 2 ms in all.
+    ksteps = max(steps, KERNEL_PASS_MIN_STEPS)
+    for _ in range(ksteps):
+        step()
+    rocm.sync()
+    rocm.profile_enable(True)
+    for _ in range(ksteps):
+        step()
+    prof = rocm.profile_collect()
+    rocm.profile_enable(False)
+    kernels = {n: {"calls": c, "avg_us": 1e3 * ms / c} for n, (c, ms) in prof.items()}
+
+    # the timed region: `warmup` untimed steps, then exactly `steps` steps between two events
+    # (and two host clock reads), synchronised on both sides
     for _ in range(warmup):
         step()
     rocm.sync()
@@ -82,20 +100,6 @@ def bench_train(steps: int, warmup: int, only: str = "all"):
     rocm.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
     dev_ms = timer.elapsed_ms()
-
-    # second pass: per-kernel device times over at least KERNEL_PASS_MIN_STEPS steps whatever
-    # `steps` is (a kernel's first launches after a pause run slower than its settled time,
-    # and `roofline` is computed from this pass), after as many untimed steps again
-    ksteps = max(steps, KERNEL_PASS_MIN_STEPS)
-    for _ in range(max(0, ksteps - steps - warmup)):
-        step()
-    rocm.sync()
-    rocm.profile_enable(True)
-    for _ in range(ksteps):
-        step()
-    prof = rocm.profile_collect()
-    rocm.profile_enable(False)
-    kernels = {n: {"calls": c, "avg_us": 1e3 * ms / c} for n, (c, ms) in prof.items()}
 
     # third pass: every step between its own pair of events (median and minimum of a step)
     timers = [rocm.Timer() for _ in range(steps)]
@@ -553,6 +557,8 @@ def main():
                    "flops_per_step": fwd_f + bwd_f, "flop_convention": "7*B*H*T^2*D"},
         "frac_mfma_peak": tflops / PEAK_F16_TFLOPS,
         "peak_tflops_f16_dense": PEAK_F16_TFLOPS,
+        "timed_region": "`warmup` untimed + exactly `steps` timed fwd+bwd steps, run after the per-kernel pass "
+                        "(2 x %d steps) so that short runs see settled clocks" % max(args.steps, KERNEL_PASS_MIN_STEPS),
         "wall_ms_per_step": tr["wall_ms"] / args.steps,
         "step_us_event_pairs": tr["step_us"],
         "kernels": kern,
