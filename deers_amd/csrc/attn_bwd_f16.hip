@@ -156,13 +156,11 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     async_load4_to_lds(vec, lane * 4, slot + 2 * TILE_B + (wave & 1) * VEC_B);
   };
 
-#pragma unroll
-  for (int i = 0; i < P; ++i) request(first_tile + i);
-
   // K^T and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.
   // Rows past T-1 read row T-1 instead: their keys are masked for every valid query
   // and their dK/dV rows are not stored, and without a branch the loads issue as one
-  // batch with a single wait.
+  // batch with a single wait.  Issued before the first tile requests, whose flag poll is a
+  // round trip to L2 of its own: the two latencies overlap.
   half8 kf[KS], vf[KS];
   {
     const int krow = min(kvrow, T - 1);
@@ -174,6 +172,9 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
       vf[ks] = *(const half8*)(vp + 16 * ks);
     }
   }
+
+#pragma unroll
+  for (int i = 0; i < P; ++i) request(first_tile + i);
 
   // ---- per-lane swizzled read offsets (bytes within a tile) ----
   int aoff[KS];  // row-major A operand: row lane%32 (+32 for the second block), chunk 2ks+g
