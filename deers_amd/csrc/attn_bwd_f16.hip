@@ -119,29 +119,33 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     ld_do_tail[i] = (uint32_t)(row_tail * sdot * 2 + col);
   }
   // The row statistics of query block qb come from the dQ workgroup that owns it, which
-  // runs in the same launch on the same XCD (see the launch kernel below).
-  int ready_upto = -1;  // query blocks [0, ready_upto] are known to be published
-  auto wait_published = [&](int qb) {
-    if (qb <= ready_upto) return;
-    const int* flag = p.ready + (int64_t)bh * n_blocks + qb;
-    // Bounded: a producer cannot be held up by this workgroup (it was dispatched
-    // earlier and waits for nothing), so the bound is not reached in practice; it
-    // guarantees that every wave leaves the loop.  A wait that does run out raises the
-    // error word in front of the flags (the statistics it then reads are not valid and
-    // this call's dK / dV are wrong): the host reports it at the next synchronisation.
-    int spins = 0;
-    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
-      if (++spins >= p.spin_limit) {
-        __hip_atomic_store(p.ready - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
+  // runs in the same launch on the same XCD (see the launch kernel below).  This block needs
+  // those of query blocks kvblk .. n_blocks-1: before its first request it polls all their
+  // flags at once, one per lane, so the loop itself never waits for a flag (a poll there
+  // drains the wave's whole ring of tile loads, every other iteration).
+  // Bounded: a producer cannot be held up by this workgroup (it was dispatched earlier and
+  // waits for nothing), so the bound is not reached in practice; it guarantees that every
+  // wave leaves the loop.  A wait that does run out raises the error word in front of the
+  // flags (the statistics it then reads are not valid and this call's dK / dV are wrong):
+  // the host reports it at the next synchronisation.
+  auto wait_published = [&]() {
+    for (int base = kvblk; base < n_blocks; base += 64) {
+      const int qb = base + lane;
+      const int* flag = p.ready + (int64_t)bh * n_blocks + min(qb, n_blocks - 1);
+      int spins = 0;
+      for (;;) {
+        const int seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__all(seen == p.epoch)) break;
+        if (++spins >= p.spin_limit) {
+          __hip_atomic_store(p.ready - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
       }
-      __builtin_amdgcn_s_sleep(8);
     }
-    ready_upto = qb;
   };
   auto request = [&](int t) {
     const int tc = min(t, n_tiles - 1);  // clamped repeats are never consumed
-    wait_published(tc * kBwdStep / kBwdBlk);
     const uint32_t slot = lds0 + (t % NS) * SLOT_B;
     const half_t* qbase = Q + (uint32_t)(tc * kBwdStep * sqt);
     const half_t* dobase = dO + (uint32_t)(tc * kBwdStep * sdot);
@@ -159,8 +163,8 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
   // K^T and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.
   // Rows past T-1 read row T-1 instead: their keys are masked for every valid query
   // and their dK/dV rows are not stored, and without a branch the loads issue as one
-  // batch with a single wait.  Issued before the first tile requests, whose flag poll is a
-  // round trip to L2 of its own: the two latencies overlap.
+  // batch with a single wait.  Issued before the flag poll, which is a round trip to L2 of
+  // its own: the two latencies overlap.
   half8 kf[KS], vf[KS];
   {
     const int krow = min(kvrow, T - 1);
@@ -173,6 +177,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
     }
   }
 
+  wait_published();
 #pragma unroll
   for (int i = 0; i < P; ++i) request(first_tile + i);
 
