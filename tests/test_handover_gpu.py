@@ -62,6 +62,28 @@ def test_two_launch_backward_equals_single_launch_bit_for_bit(gpu, B, H, T, D):
 
 
 @pytest.mark.gpu
+def test_more_than_64_query_blocks_per_head(gpu):
+    """A dK/dV workgroup polls its flags one per lane: 66 query blocks take a second round of
+    the 64-lane poll.  Single launch against two launches bit for bit, and one whole head
+    against the oracle."""
+    B, H, T, D = 1, 2, 8400, 64
+    x = synth.attention_inputs("handover-long", B, H, T, D, np.float16, base_seed=13)
+    print(f"case handover-long f16 B={B} H={H} T={T} D={D}", flush=True)
+    rocm.set_handover_mode(rocm.HANDOVER_SAME_XCD)
+    one = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])
+    rocm.set_handover_mode(rocm.HANDOVER_STREAM_ORDER)
+    two = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])
+    rocm.sync()
+    for a, b in zip(one, two):
+        np.testing.assert_array_equal(a, b)
+    sl = (slice(0, 1), slice(1, 2))
+    rdq, rdk, rdv = oracle.attn_bwd(x["q"][sl], x["k"][sl], x["v"][sl], x["do"][sl])
+    for name, got, want in zip(("dq", "dk", "dv"), one[2:], (rdq, rdk, rdv)):
+        err = np.max(np.abs(got[sl].astype(np.float64) - want))
+        assert err <= 5e-3, f"{name}: max abs err {err:.3e}"
+
+
+@pytest.mark.gpu
 def test_unsplit_few_rows_gemm_matches_split_within_rounding(gpu):
     m, n, k = 32, 768, 3072  # the shape whose K is split over workgroups
     rng = np.random.default_rng(5)
