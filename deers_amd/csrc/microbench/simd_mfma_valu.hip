@@ -1,0 +1,396 @@
+// Micro-benchmarks behind the attention kernels' roofline argument: what one gfx950 SIMD does
+// with the instruction mix of the f16 attention loops, with no memory system in the way.
+//
+//   0  a bare MFMA stream on every SIMD: sustained matrix rate and shader clock
+//   A  vector issue rate of 1..4 waves per SIMD (independent v_fma_f32 chains, a dependent
+//      chain, v_exp_f32, three-operand v_max3_f32)
+//   B  one wave streaming v_mfma_f32_32x32x16_f16 beside one wave streaming vector ops on
+//      the same SIMD: each alone, then together
+//   C  one instruction stream with NV vector ops between consecutive MFMAs, 1 and 2 waves
+//   D  the forward's wave-iteration (S = K Q^T on 64 keys, online softmax on the results,
+//      O += V^T P) with its memory features switched on one at a time: LDS fragment reads,
+//      the per-iteration barrier, asynchronous global->LDS tile loads; 1, 2, 3 waves per SIMD
+//
+// Every launch covers all CUs (256 workgroups x waves); times are clock64() deltas from the
+// common start of a CU's waves to the end of its slowest wave, averaged over the CUs, so
+// figures are shader clocks.  A first section times a bare MFMA stream on all CUs with events:
+// the matrix rate and the shader clock the device actually sustains.  Build: make -C deers_amd/csrc
+// microbench; run: deers_amd/csrc/microbench/simd_mfma_valu.
+#include <cstdio>
+#include <cstdlib>
+
+#include "../common.h"
+
+using namespace deers;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#define CK(x)                                                              \
+  do {                                                                     \
+    hipError_t e_ = (x);                                                   \
+    if (e_ != hipSuccess) {                                                \
+      printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); \
+      exit(1);                                                             \
+    }                                                                      \
+  } while (0)
+#define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
+#define MF(acc) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b))
+#define FM(v) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v) : "v"(c1), "v"(c2))
+#define EX(v) asm volatile("v_exp_f32 %0, %0" : "+v"(v))
+#define MX(v, w) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(v) : "v"(w), "v"(c2))
+#define REP8(X) X X X X X X X X
+
+static long long* g_clk = nullptr;  // per-wave elapsed clocks of the last launch
+static float* g_out = nullptr;
+// Clocks from the common start of a workgroup's waves to the end of the slowest of waves
+// [first_wave, first_wave + n_waves) of each workgroup, averaged over the workgroups.  (The
+// SIMD serves its waves oldest first, so their end times differ; the last one bounds the
+// SIMD's time.)
+static double slowest_wave_clocks(int n_blocks, int first_wave, int n_waves) {
+  static long long h[256 * 16];
+  CK(hipMemcpy(h, g_clk, sizeof(h), hipMemcpyDeviceToHost));
+  double s = 0;
+  for (int blk = 0; blk < n_blocks; ++blk) {
+    long long mx = 0;
+    for (int w = first_wave; w < first_wave + n_waves; ++w) mx = h[blk * 16 + w] > mx ? h[blk * 16 + w] : mx;
+    s += (double)mx;
+  }
+  return s / n_blocks;
+}
+
+// ---- 0: bare MFMA stream on all CUs, by events and by the 100 MHz wall clock ---------------
+__global__ __launch_bounds__(1024) void mfma_stream_kernel(float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (half_t)(0.001f * (lane + i));
+    b[i] = (half_t)(0.002f * (lane - i));
+  }
+  floatx16 acc0 = ZERO16, acc1 = ZERO16, acc2 = ZERO16, acc3 = ZERO16;
+  __syncthreads();
+  const long long w0 = wall_clock64(), t0 = clock64();
+  for (int it = 0; it < iters; ++it) { REP8(MF(acc0); MF(acc1);) REP8(MF(acc2); MF(acc3);) }
+  const long long t1 = clock64(), w1 = wall_clock64();
+  float s = 0;
+  for (int i = 0; i < 16; ++i) s += acc0[i] + acc1[i] + acc2[i] + acc3[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = wave == 0 ? ((t1 - t0) << 32 | (w1 - w0)) : 0;
+}
+static void run_mfma_stream() {
+  const int iters = 10000;
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  for (int rep = 0; rep < 3; ++rep)
+    for (int waves = 4; waves <= 16; waves += 4) {
+      mfma_stream_kernel<<<256, 64 * waves>>>(g_out, g_clk, 100);
+      CK(hipEventRecord(e0));
+      mfma_stream_kernel<<<256, 64 * waves>>>(g_out, g_clk, iters);
+      CK(hipEventRecord(e1));
+      CK(hipEventSynchronize(e1));
+      float ms;
+      CK(hipEventElapsedTime(&ms, e0, e1));
+      static long long h[256 * 16];
+      CK(hipMemcpy(h, g_clk, sizeof(h), hipMemcpyDeviceToHost));
+      double ghz = 0;
+      for (int blk = 0; blk < 256; ++blk) ghz += (double)(h[blk * 16] >> 32) / ((double)(h[blk * 16] & 0xffffffff) * 10.0);
+      ghz /= 256;
+      const double mfmas_per_simd = (double)iters * 32.0 * (waves / 4);
+      const double ns = ms * 1e6 / mfmas_per_simd;
+      if (rep == 2)
+        printf("0 bare MFMA stream, %d wave(s)/SIMD: %5.2f ns per MFMA per SIMD = %4.0f TFLOP/s on 1024 SIMDs, shader clock %4.2f "
+               "GHz (%4.1f clocks per MFMA)\n",
+               waves / 4, ns, 32768.0 * 1024 / ns / 1e3, ghz, ns * ghz);
+    }
+}
+
+// ---- A: vector issue rate --------------------------------------------------------------
+template <int KIND>
+__global__ __launch_bounds__(1024) void valu_rate_kernel(float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3, v4 = lane + 4, v5 = lane + 5, v6 = lane + 6,
+        v7 = lane + 7;
+  float c1 = 0.999f, c2 = 0.001f;
+  __syncthreads();
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {  // 32 ops per pass
+    if (KIND == 0) { REP8(FM(v0); FM(v1); FM(v2); FM(v3);) }
+    if (KIND == 1) { REP8(FM(v0); FM(v0); FM(v0); FM(v0);) }
+    if (KIND == 2) { REP8(EX(v0); EX(v1); EX(v2); EX(v3);) }
+    if (KIND == 3) { REP8(MX(v0, v4); MX(v1, v5); MX(v2, v6); MX(v3, v7);) }
+  }
+  const long long t1 = clock64();
+  out[blockIdx.x * blockDim.x + threadIdx.x] = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+template <int KIND>
+static void run_valu_rate(const char* name) {
+  const int iters = 4000;
+  for (int waves = 4; waves <= 16; waves += 4) {
+    valu_rate_kernel<KIND><<<256, 64 * waves>>>(g_out, g_clk, 50);
+    valu_rate_kernel<KIND><<<256, 64 * waves>>>(g_out, g_clk, iters);
+    CK(hipDeviceSynchronize());
+    const double per_op = slowest_wave_clocks(256, 0, waves) / (iters * 32.0);
+    printf("A %-22s %d wave(s)/SIMD: %5.2f clocks per op per wave = one op per %4.2f clocks per SIMD\n", name,
+           waves / 4, per_op, per_op / (waves / 4));
+  }
+}
+
+// ---- B: an MFMA wave beside a vector wave ------------------------------------------------
+__global__ __launch_bounds__(512) void side_by_side_kernel(float* out, long long* clk, int iters, int mfma_on,
+                                                           int valu_kind) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (half_t)(0.001f * (lane + i));
+    b[i] = (half_t)(0.002f * (lane - i));
+  }
+  floatx16 acc0 = ZERO16, acc1 = ZERO16;
+  float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3;
+  float c1 = 0.999f, c2 = 0.001f;
+  __syncthreads();
+  const long long t0 = clock64();
+  if (wave < 4) {  // two dependent chains, as the S and dP accumulators of a block
+    if (mfma_on)
+      for (int it = 0; it < iters; ++it) { REP8(MF(acc0); MF(acc1);) }
+  } else {
+    if (valu_kind == 1)
+      for (int it = 0; it < 4 * iters; ++it) { REP8(FM(v0); FM(v1); FM(v2); FM(v3);) }
+    if (valu_kind == 2)
+      for (int it = 0; it < 4 * iters; ++it) { REP8(EX(v0); EX(v1); EX(v2); EX(v3);) }
+  }
+  const long long t1 = clock64();
+  float s = v0 + v1 + v2 + v3;
+  for (int i = 0; i < 16; ++i) s += acc0[i] + acc1[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+static void run_side_by_side() {
+  const int iters = 2000;
+  const int cfg[][2] = {{1, 0}, {0, 1}, {0, 2}, {1, 1}, {1, 2}};
+  for (const auto& c : cfg) {
+    side_by_side_kernel<<<256, 512>>>(g_out, g_clk, 50, c[0], c[1]);
+    side_by_side_kernel<<<256, 512>>>(g_out, g_clk, iters, c[0], c[1]);
+    CK(hipDeviceSynchronize());
+    const double m = slowest_wave_clocks(256, 0, 4) / (iters * 16.0);
+    const double v = slowest_wave_clocks(256, 4, 4) / (iters * 128.0);
+    printf("B MFMA wave %s, vector wave %-4s: %5.1f clocks per MFMA, %5.2f clocks per vector op\n",
+           c[0] ? "on " : "off", c[1] == 0 ? "off" : c[1] == 1 ? "fma" : "exp", c[0] ? m : 0.0, c[1] ? v : 0.0);
+  }
+}
+
+// ---- C: NV vector ops between consecutive MFMAs of one wave -------------------------------
+template <int NV>
+__global__ __launch_bounds__(512) void interleaved_kernel(float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (half_t)(0.001f * (lane + i));
+    b[i] = (half_t)(0.002f * (lane - i));
+  }
+  floatx16 acc0 = ZERO16, acc1 = ZERO16, acc2 = ZERO16, acc3 = ZERO16;
+  float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3, v4 = lane + 4, v5 = lane + 5, v6 = lane + 6,
+        v7 = lane + 7;
+  float c1 = 0.999f, c2 = 0.001f;
+#define VGRP()                                                                                      \
+  do {                                                                                              \
+    if (NV >= 1) FM(v0); if (NV >= 2) FM(v1); if (NV >= 3) FM(v2); if (NV >= 4) FM(v3);             \
+    if (NV >= 5) FM(v4); if (NV >= 6) FM(v5); if (NV >= 7) FM(v6); if (NV >= 8) FM(v7);             \
+    if (NV >= 9) FM(v0); if (NV >= 10) FM(v1); if (NV >= 11) FM(v2); if (NV >= 12) FM(v3);          \
+    if (NV >= 13) FM(v4); if (NV >= 14) FM(v5); if (NV >= 15) FM(v6); if (NV >= 16) FM(v7);         \
+  } while (0)
+  __syncthreads();
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      MF(acc0); VGRP(); MF(acc1); VGRP(); MF(acc2); VGRP(); MF(acc3); VGRP();
+    }
+  }
+  const long long t1 = clock64();
+  float s = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7;
+  for (int i = 0; i < 16; ++i) s += acc0[i] + acc1[i] + acc2[i] + acc3[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+template <int NV>
+static void run_interleaved() {
+  const int iters = 3000;
+  for (int waves = 4; waves <= 8; waves += 4) {
+    interleaved_kernel<NV><<<256, 64 * waves>>>(g_out, g_clk, 50);
+    interleaved_kernel<NV><<<256, 64 * waves>>>(g_out, g_clk, iters);
+    CK(hipDeviceSynchronize());
+    const double per_mfma = slowest_wave_clocks(256, 0, waves) / (iters * 16.0) / (waves / 4);
+    printf("C %2d vector ops per MFMA, %d wave(s)/SIMD: %5.1f clocks of SIMD time per MFMA (32 = matrix pipe full)\n",
+           NV, waves / 4, per_mfma);
+  }
+}
+
+// ---- D: the forward's wave-iteration --------------------------------------------------------
+constexpr int D = 64, KS = 4, DB = 2, CH = 8, RB = 128, TILE_B = 64 * RB, P = 2, NS = 3, NWLW = 2, LPI = 4,
+              RPW = 8;
+template <bool F_LDS, bool F_BAR, bool F_REQ>
+__global__ __launch_bounds__(256, 3) void fwd_iteration_kernel(const half_t* Kg, const half_t* Vg, float* out,
+                                                               long long* clk, int iters, float c) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lds0 = lds_address(smem);
+  const half_t* K = Kg + (size_t)(blockIdx.x % 96) * 1024 * D;
+  const half_t* V = Vg + (size_t)(blockIdx.x % 96) * 1024 * D;
+  uint32_t ld_k[NWLW];
+  for (int i = 0; i < NWLW; ++i) {
+    const int row = (wave * NWLW + i) * RPW + lane / CH;
+    ld_k[i] = (uint32_t)(row * D * 2 + 16 * ((lane % CH) ^ lds_swizzle<CH>(row)));
+  }
+  auto request = [&](int t) {  // K and V tile t % 16 of this head into ring slot t % NS
+    const int tc = t & 15;
+    const uint32_t kdst = lds0 + (t % NS) * TILE_B + wave * (NWLW * 1024);
+    const uint32_t vdst = kdst + NS * TILE_B;
+#pragma unroll
+    for (int i = 0; i < NWLW; ++i) {
+      async_load16_to_lds(K + (uint32_t)(tc * 64 * D), ld_k[i], kdst + i * 1024);
+      async_load16_to_lds(V + (uint32_t)(tc * 64 * D), ld_k[i], vdst + i * 1024);
+    }
+  };
+  for (int t = 0; t < NS; ++t) request(t);
+  half8 qf[KS], kreg[8], vreg[8];
+  for (int ks = 0; ks < KS; ++ks)
+    for (int i = 0; i < 8; ++i) qf[ks][i] = (half_t)(0.02f * ((lane - i - ks) % 11));
+  for (int j = 0; j < 8; ++j)
+    for (int i = 0; i < 8; ++i) {
+      kreg[j][i] = (half_t)(0.01f * ((lane + i + j) % 13) - 0.05f);
+      vreg[j][i] = (half_t)(0.01f * ((lane ^ (i + j)) % 7));
+    }
+  int koff[KS], voff_lo[DB], voff_hi[DB];
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = (lane & 31) * RB + (((2 * ks + g) ^ lds_swizzle<CH>(lane & 31)) << 4);
+  {
+    const int lrow = 4 * g + ((lane & 15) >> 2), c4 = lane & 3;
+    for (int db = 0; db < DB; ++db) {
+      const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + (c4 >> 1);
+      voff_lo[db] = lrow * RB + ((chunk ^ lds_swizzle<CH>(lrow)) << 4) + (c4 & 1) * 8;
+      voff_hi[db] = (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
+    }
+  }
+  floatx16 oacc[DB] = {ZERO16, ZERO16};
+  float m = -1e30f, lsum = 0.f;
+  wait_all_vmem();
+  __syncthreads();
+  const long long t0 = clock64();
+  for (int j = 0; j < iters; ++j) {
+    if (F_REQ) wait_vmcnt<(P - 1) * LPI>();
+    if (F_BAR) __syncthreads();
+    if (F_REQ) request(j + P);
+    const uint32_t kb = lds0 + (j % NS) * TILE_B, vb = kb + NS * TILE_B;
+    floatx16 cb[2] = {ZERO16, ZERO16};
+    if (!F_LDS)
+      for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(kreg[i]), "+v"(vreg[i]));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint32_t addr = opaque(kb + koff[ks]);
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+        cb[nb] = mfma_f16(F_LDS ? *(DEERS_LDS const half8*)(uintptr_t)(addr + nb * 32 * RB) : kreg[2 * ks + nb],
+                          qf[ks], cb[nb]);
+    }
+    half8 vfr[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      if (F_LDS) {
+        const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]));
+        const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]));
+        vfr[db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      } else {
+        vfr[db] = vreg[db];
+      }
+    }
+    float mx4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mx4[i] = fmaxf(cb[0][i], cb[1][i]);
+#pragma unroll
+    for (int r = 4; r < 16; ++r) mx4[r & 3] = fmaxf(fmaxf(mx4[r & 3], cb[0][r]), cb[1][r]);
+    const float mx = pair_max(fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3])));
+    if (__any((mx - m) * c > 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = fast_exp2((m - m_new) * c);
+      m = m_new;
+      lsum *= alpha;
+      oacc[0] *= alpha;
+      oacc[1] *= alpha;
+    }
+    const float mc = m * c;
+    uint32_t pw[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const floatx16& cc = cb[i >> 3];
+      const int r = 2 * (i & 7);
+      const float e0 = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
+      const float e1 = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
+      pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)e0, (half_t)e1});
+      lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
+    }
+#pragma unroll
+    for (int ms = 0; ms < 4; ++ms) {
+      const half8 pb = __builtin_bit_cast(half8, u32x4{pw[4 * ms], pw[4 * ms + 1], pw[4 * ms + 2], pw[4 * ms + 3]});
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        half8 av;
+        if (ms == 0) {
+          av = vfr[db];
+        } else if (F_LDS) {
+          const uint32_t ro = 16 * ms * RB;
+          const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
+          const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
+          av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+          av = vreg[2 * ms + db];
+        }
+        oacc[db] = mfma_f16(av, pb, oacc[db]);
+      }
+    }
+  }
+  const long long t1 = clock64();
+  wait_all_vmem();
+  float sum = lsum + m;
+  for (int i = 0; i < 16; ++i) sum += oacc[0][i] + oacc[1][i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+  if (lane == 0) clk[(blockIdx.x % 256) * 16 + (blockIdx.x / 256) * 4 + wave] = t1 - t0;
+}
+template <bool F_LDS, bool F_BAR, bool F_REQ>
+static void run_fwd_iteration(const half_t* Kg, const half_t* Vg) {
+  const int iters = 3000;
+  const size_t lds = 2 * NS * TILE_B;
+  for (int wgs = 1; wgs <= 3; ++wgs) {
+    fwd_iteration_kernel<F_LDS, F_BAR, F_REQ><<<256 * wgs, 256, lds>>>(Kg, Vg, g_out, g_clk, 50, 0.18f);
+    fwd_iteration_kernel<F_LDS, F_BAR, F_REQ><<<256 * wgs, 256, lds>>>(Kg, Vg, g_out, g_clk, iters, 0.18f);
+    CK(hipDeviceSynchronize());
+    const double per_iter = slowest_wave_clocks(256, 0, 4 * wgs) / iters;
+    printf("D lds reads %d, barrier %d, tile loads %d, %d wave(s)/SIMD: %5.0f clocks per wave-iteration = %4.0f of "
+           "SIMD time (its 16 MFMAs alone: 512)\n",
+           (int)F_LDS, (int)F_BAR, (int)F_REQ, wgs, per_iter, per_iter / wgs);
+  }
+}
+
+int main() {
+  CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
+  CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
+  run_mfma_stream();
+  run_valu_rate<0>("v_fma_f32 independent");
+  run_valu_rate<1>("v_fma_f32 dependent");
+  run_valu_rate<2>("v_exp_f32");
+  run_valu_rate<3>("v_max3_f32");
+  run_side_by_side();
+  run_interleaved<0>();
+  run_interleaved<4>();
+  run_interleaved<8>();
+  run_interleaved<12>();
+  run_interleaved<16>();
+  half_t *Kg, *Vg;
+  CK(hipMalloc(&Kg, 96 * 1024 * D * 2));
+  CK(hipMalloc(&Vg, 96 * 1024 * D * 2));
+  CK(hipMemset(Kg, 0, 96 * 1024 * D * 2));
+  CK(hipMemset(Vg, 0, 96 * 1024 * D * 2));
+  run_fwd_iteration<false, false, false>(Kg, Vg);
+  run_fwd_iteration<true, false, false>(Kg, Vg);
+  run_fwd_iteration<true, true, false>(Kg, Vg);
+  run_fwd_iteration<true, true, true>(Kg, Vg);
+  return 0;
+}
