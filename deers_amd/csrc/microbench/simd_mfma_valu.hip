@@ -3,7 +3,8 @@
 //
 //   0  a bare MFMA stream on every SIMD: sustained matrix rate and shader clock
 //   A  vector issue rate of 1..4 waves per SIMD (independent v_fma_f32 chains, a dependent
-//      chain, v_exp_f32, three-operand v_max3_f32)
+//      chain, v_exp_f32, v_max3_f32, v_fma_f32 with a scalar-register operand,
+//      v_cvt_pk_f16_f32, v_dot2c_f32_f16, v_exp_f16)
 //   B  one wave streaming v_mfma_f32_32x32x16_f16 beside one wave streaming vector ops on
 //      the same SIMD: each alone, then together
 //   C  one instruction stream with NV vector ops between consecutive MFMAs, 1 and 2 waves
@@ -36,6 +37,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define FM(v) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v) : "v"(c1), "v"(c2))
 #define EX(v) asm volatile("v_exp_f32 %0, %0" : "+v"(v))
 #define MX(v, w) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(v) : "v"(w), "v"(c2))
+#define FMS(v) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v) : "s"(sc), "v"(c2))
+#define CVT(d, x, y) asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y))
+#define DOT(acc, x) asm volatile("v_dot2c_f32_f16 %0, %1, %2" : "+v"(acc) : "v"(x), "v"(ones))
+#define EXH(v) asm volatile("v_exp_f16 %0, %0" : "+v"(v))
 #define REP8(X) X X X X X X X X
 
 static long long* g_clk = nullptr;  // per-wave elapsed clocks of the last launch
@@ -109,6 +114,9 @@ __global__ __launch_bounds__(1024) void valu_rate_kernel(float* out, long long* 
   float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3, v4 = lane + 4, v5 = lane + 5, v6 = lane + 6,
         v7 = lane + 7;
   float c1 = 0.999f, c2 = 0.001f;
+  const float sc = 0.18f;                   // stays in a scalar register
+  unsigned h0 = 0xb800b400u + lane, h1 = 0xb900b500u + lane, h2 = 0xba00b600u + lane, h3 = 0xbb00b700u + lane;
+  const unsigned ones = 0x3c003c00u;        // (1, 1) as packed halfs
   __syncthreads();
   const long long t0 = clock64();
   for (int it = 0; it < iters; ++it) {  // 32 ops per pass
@@ -116,9 +124,13 @@ __global__ __launch_bounds__(1024) void valu_rate_kernel(float* out, long long* 
     if (KIND == 1) { REP8(FM(v0); FM(v0); FM(v0); FM(v0);) }
     if (KIND == 2) { REP8(EX(v0); EX(v1); EX(v2); EX(v3);) }
     if (KIND == 3) { REP8(MX(v0, v4); MX(v1, v5); MX(v2, v6); MX(v3, v7);) }
+    if (KIND == 4) { REP8(FMS(v0); FMS(v1); FMS(v2); FMS(v3);) }
+    if (KIND == 5) { REP8(CVT(h0, v0, v1); CVT(h1, v1, v2); CVT(h2, v2, v3); CVT(h3, v3, v0);) }
+    if (KIND == 6) { REP8(DOT(v0, h0); DOT(v1, h1); DOT(v2, h2); DOT(v3, h3);) }
+    if (KIND == 7) { REP8(EXH(h0); EXH(h1); EXH(h2); EXH(h3);) }
   }
   const long long t1 = clock64();
-  out[blockIdx.x * blockDim.x + threadIdx.x] = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7;
+  out[blockIdx.x * blockDim.x + threadIdx.x] = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7 + (float)(h0 + h1 + h2 + h3);
   if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
 }
 template <int KIND>
@@ -377,6 +389,10 @@ int main() {
   run_valu_rate<1>("v_fma_f32 dependent");
   run_valu_rate<2>("v_exp_f32");
   run_valu_rate<3>("v_max3_f32");
+  run_valu_rate<4>("v_fma_f32 v, s, v");
+  run_valu_rate<5>("v_cvt_pk_f16_f32");
+  run_valu_rate<6>("v_dot2c_f32_f16");
+  run_valu_rate<7>("v_exp_f16");
   run_side_by_side();
   run_interleaved<0>();
   run_interleaved<4>();
