@@ -4,10 +4,10 @@
 // causal_mask + add, log_sum_exp, sub, exp, matmul) with one kernel that never
 // materialises the [T,T] score tensor.
 //
-// Two kernels share this decomposition: the software-pipelined one described below
-// (two workgroups per CU) and, for D <= 64 launches with more than two tiles per CU, a
-// plain one at three or four workgroups per CU (attn_fwd_f16_resident_kernel, further
-// down), whose workgroups are all resident from the start when they fit.
+// Two kernels share this decomposition: the tile-pipelined one described below (two
+// workgroups per CU; head width 128 and small launches) and, for D <= 64 launches with
+// more than two tiles per CU, the block-pipelined one of attn_fwd_f16_bp.h at three
+// workgroups per CU, whose workgroups are all resident from the start when they fit.
 //
 // Work decomposition
 //   grid  = one workgroup per (head, 128-row query tile), dealt to the XCDs so a
@@ -35,35 +35,24 @@
 // of their use so HBM/L2 latency is off the critical path; tiles are unpadded and
 // XOR-swizzled by 16-byte chunk.  One barrier per iteration.
 #include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <tuple>
 #include <type_traits>
 #include <vector>
 
+#include "attn_fwd_f16_bp.h"
 #include "common.h"
 
 namespace deers {
 
-constexpr int kFwdBM = 128;  // query rows per workgroup
-constexpr int kFwdBN = 64;   // key/value rows per iteration
 // The running row maximum is only advanced when some row's new maximum exceeds
 // the one in use by more than this many powers of two; until then probabilities
 // are formed against the stale maximum (values up to 2^8, exact in f16/f32).
 constexpr float kLazyRescale = 8.0f;
 
-#define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
 
-template <int D>
-struct FwdCfg {
-  // prefetch distance in iterations; D = 128 keeps one tile less in flight so that two
-  // workgroups' rings (2 x 64 KB) share a CU
-  static constexpr int P = D == 128 ? 1 : 2;
-  static constexpr int NS = P + 1;              // ring slots per tensor
-  static constexpr int RB = D * 2;              // row bytes
-  static constexpr int TILE_B = kFwdBN * RB;    // tile bytes
-  static constexpr size_t kLds = 2 * NS * TILE_B;
-};
 
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int BH, int n_qtiles,
@@ -440,211 +429,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_f16_kernel(FwdParams p, int B
   }
 }
 
-// Position -> tile table of a launch whose workgroups are all resident at once, passed in
-// the kernel arguments: entry p = (head index within the XCD) << 16 | query tile for the
-// workgroup at position p = blockIdx.x / 8 of its XCD.
-constexpr int kMaxResidentTiles = 128;  // per XCD: 32 CUs x at most 4 workgroups
-struct TileOrder {
-  int32_t code[kMaxResidentTiles];
-};
-
-// ---- variant: three workgroups per CU, no software pipeline inside the wave ----
-// Each iteration is S = K Q^T, softmax, O += V^T P in program order on ONE S
-// accumulator; the overlap of matrix and vector work comes from three waves per SIMD
-// instead of from interleaving inside one (<= 168 registers).  K(j) and V(j) travel
-// together, P iterations ahead.
-template <int D>
-__global__ __launch_bounds__(256, 3) void attn_fwd_f16_resident_kernel(FwdParams p, int BH, int n_qtiles,
-                                                                   int heads_per_xcd, TileOrder order) {
-  using Cfg = FwdCfg<D>;
-  constexpr int P = Cfg::P, NS = Cfg::NS, RB = Cfg::RB, TILE_B = Cfg::TILE_B;
-  constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
-  constexpr int RPW = 1024 / RB, NWLW = TILE_B / 4096, LPI = 2 * NWLW;
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g = lane >> 5;
-  const int T = p.T;
-  int bh, qtile;
-  if (order.code[0] >= 0) {
-    // every workgroup is resident at once: position -> tile chosen for even CU totals
-    const int code = order.code[blockIdx.x >> 3];
-    bh = (code >> 16) * 8 + (blockIdx.x & 7);
-    qtile = code & 0xffff;
-    if (bh >= BH) return;
-  } else {  // no table: each XCD's list longest first, handed out by the dispatcher
-    int rank;
-    if (!map_block(blockIdx.x, n_qtiles, heads_per_xcd, BH, &bh, &rank)) return;
-    qtile = n_qtiles - 1 - rank;
-  }
-  [[maybe_unused]] const int trace_row = blockIdx.x;
-  const int b = bh / p.H, h = bh % p.H;
-  const half_t* Q = (const half_t*)p.q + b * p.sq.b + h * p.sq.h;
-  const half_t* K = (const half_t*)p.k + b * p.sk.b + h * p.sk.h;
-  const half_t* V = (const half_t*)p.v + b * p.sv.b + h * p.sv.h;
-  half_t* O = (half_t*)p.o + b * p.so.b + h * p.so.h;
-  const int q0 = qtile * kFwdBM, qw0 = q0 + 32 * wave, qrow = qw0 + (lane & 31);
-  const int n_tiles = min(q0 + kFwdBM - 1, T - 1) / kFwdBN + 1;
-  const uint32_t lds0 = lds_address(smem);
-  const int tail_tile = (T - 1) / kFwdBN;
-  const int skt = (int)p.sk.t, svt = (int)p.sv.t;
-  uint32_t ld_k[NWLW], ld_v[NWLW], ld_k_tail[NWLW], ld_v_tail[NWLW];
-#pragma unroll
-  for (int i = 0; i < NWLW; ++i) {
-    const int row = (wave * NWLW + i) * RPW + lane / CH;
-    const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-    const int row_tail = min(row, T - 1 - tail_tile * kFwdBN);
-    ld_k[i] = (uint32_t)(row * skt * 2 + col);
-    ld_v[i] = (uint32_t)(row * svt * 2 + col);
-    ld_k_tail[i] = (uint32_t)(row_tail * skt * 2 + col);
-    ld_v_tail[i] = (uint32_t)(row_tail * svt * 2 + col);
-  }
-  auto request = [&](int t) {  // K(t) and V(t) into slot t % NS; past the end: clamped, never consumed
-    const int tc = min(t, n_tiles - 1);
-    const uint32_t kdst = lds0 + (t % NS) * TILE_B + wave * (NWLW * 1024);
-    const uint32_t vdst = kdst + NS * TILE_B;
-    const half_t* kbase = K + (uint32_t)(tc * kFwdBN * skt);
-    const half_t* vbase = V + (uint32_t)(tc * kFwdBN * svt);
-#pragma unroll
-    for (int i = 0; i < NWLW; ++i) {
-      async_load16_to_lds(kbase, tc == tail_tile ? ld_k_tail[i] : ld_k[i], kdst + i * 1024);
-      async_load16_to_lds(vbase, tc == tail_tile ? ld_v_tail[i] : ld_v[i], vdst + i * 1024);
-    }
-  };
-#pragma unroll
-  for (int t = 0; t < P; ++t) request(t);
-  half8 qf[KS];
-  {
-    const half_t* qp = Q + (int64_t)min(qrow, T - 1) * p.sq.t + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const half8*)(qp + 16 * ks);
-  }
-  int koff[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    koff[ks] = (lane & 31) * RB + (((2 * ks + g) ^ lds_swizzle<CH>(lane & 31)) << 4);
-  int voff_lo[DB], voff_hi[DB];
-  {
-    const int lrow = 4 * g + ((lane & 15) >> 2);
-    const int c4 = lane & 3;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + (c4 >> 1);
-      voff_lo[db] = lrow * RB + ((chunk ^ lds_swizzle<CH>(lrow)) << 4) + (c4 & 1) * 8;
-      voff_hi[db] = (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
-    }
-  }
-  floatx16 oacc[DB];
-#pragma unroll
-  for (int i = 0; i < DB; ++i) oacc[i] = ZERO16;
-  float m = -INFINITY, lsum = 0.f;
-  // kept in a vector register: v_fma_f32 with a scalar-register operand issues at 4.4 clocks
-  // per SIMD against 2.6 with three vector registers, and every score passes through one
-  float c = p.scale_log2;
-  asm volatile("" : "+v"(c));
-  wait_all_vmem();  // Q fragments (and with them every request so far)
-
-  for (int j = 0; j < n_tiles; ++j) {
-    const int kv0 = j * kFwdBN;
-    wait_vmcnt<(P - 1) * LPI>();
-    __syncthreads();
-    request(j + P);
-    const uint32_t kb = lds0 + (j % NS) * TILE_B;
-    const uint32_t vb = kb + NS * TILE_B;
-    // A wave skips what lies entirely in its rows' future: the whole tile, or its second
-    // 32-key block (both happen only in a query tile's last two iterations).
-    if (kv0 > qw0 + 31) continue;
-    auto tile_step = [&](auto n_blocks) {
-      constexpr int NB = decltype(n_blocks)::value;  // 32-key blocks of this tile the wave needs
-      // ---- S^T = K Q^T ----
-      floatx16 cb[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) cb[nb] = ZERO16;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const uint32_t addr = opaque(kb + koff[ks]);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          cb[nb] = mfma_f16(*(DEERS_LDS const half8*)(uintptr_t)(addr + nb * 32 * RB), qf[ks], cb[nb]);
-      }
-      // V fragments of the first 16 keys, fetched while the vector pipe works
-      half8 vfr[DB];
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]));
-        const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]));
-        vfr[db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
-      if (kv0 + 32 * NB - 1 > qw0) {
-        const int dist = qrow - 4 * g - kv0;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int kr = 8 * (r >> 2) + (r & 3);
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-            if (kr + 32 * nb > dist) cb[nb][r] = -INFINITY;
-        }
-      }
-      float mx4[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx4[i] = NB == 2 ? fmaxf(cb[0][i], cb[NB - 1][i]) : cb[0][i];
-#pragma unroll
-      for (int r = 4; r < 16; ++r)
-        mx4[r & 3] = NB == 2 ? fmaxf(fmaxf(mx4[r & 3], cb[0][r]), cb[NB - 1][r]) : fmaxf(mx4[r & 3], cb[0][r]);
-      const float mx = pair_max(fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3])));
-      if (__any((mx - m) * c > kLazyRescale)) {
-        const float m_new = fmaxf(m, mx);
-        const float alpha = fast_exp2((m - m_new) * c);
-        m = m_new;
-        lsum *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-      }
-      const float mc = m * c;
-      uint32_t pw[8 * NB];
-#pragma unroll
-      for (int i = 0; i < 8 * NB; ++i) {
-        const floatx16& cc = cb[i >> 3];
-        const int r = 2 * (i & 7);
-        const float e0 = fast_exp2(__builtin_fmaf(cc[r], c, -mc));
-        const float e1 = fast_exp2(__builtin_fmaf(cc[r + 1], c, -mc));
-        pw[i] = __builtin_bit_cast(uint32_t, half2v{(half_t)e0, (half_t)e1});
-        lsum = add_half2(__builtin_bit_cast(half2v, pw[i]), lsum);
-      }
-      // ---- O^T += V^T P^T ----
-#pragma unroll
-      for (int ms = 0; ms < 2 * NB; ++ms) {
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const half8 pb = __builtin_bit_cast(half8, u32x4{pw[4 * ms], pw[4 * ms + 1], pw[4 * ms + 2], pw[4 * ms + 3]});
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          half8 a;
-          if (ms == 0) {
-            a = vfr[db];
-          } else {
-            const uint32_t ro = 16 * ms * RB;
-            const half4 lo = lds_read_tr16_at(opaque(vb + voff_lo[db]) + ro);
-            const half4 hi = lds_read_tr16_at(opaque(vb + voff_hi[db]) + ro);
-            a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          }
-          oacc[db] = mfma_f16(a, pb, oacc[db]);
-        }
-      }
-    };
-    if (kv0 + 32 > qw0 + 31)
-      tile_step(std::integral_constant<int, 1>{});
-    else
-      tile_step(std::integral_constant<int, 2>{});
-  }
-  lsum = pair_sum(lsum);
-  if (qrow < T) {
-    const float inv = 1.f / lsum;
-    half_t* orow = O + (int64_t)qrow * p.so.t;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) store_block_f16(orow + 32 * db, oacc[db], inv, g);
-    if (g == 0) p.lse[(int64_t)bh * T + qrow] = (m * c + fast_log2(lsum)) * kLn2;
-  }
-}
 
 // Builds the TileOrder of a launch whose workgroups are all resident at once (their
 // number does not exceed what the chip holds).  Workgroup position p of an XCD (id / 8)
@@ -679,8 +463,8 @@ static const TileOrder* resident_order(int heads_per_xcd, int T, bool* use_resid
   *use_resident_kernel = false;
   int cus = 0, per_cu = 0;
   (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_fwd_f16_resident_kernel<D>, 256,
-                                                     FwdCfg<D>::kLds);
+  (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_fwd_f16_bp_kernel<D>, 256,
+                                                     BpCfg<D>::kLds);
   const int n_cu = std::max(cus / 8, 1);
   const int n_qtiles = (T + kFwdBM - 1) / kFwdBM;
   const int n_items = heads_per_xcd * n_qtiles;
@@ -725,13 +509,12 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
   }
   LaunchScope scope("attn_fwd_f16", stream);
   if constexpr (D <= 64) {
-    // More tiles than the pipelined kernel holds at once (two workgroups per CU): the plain
-    // kernel at three or four workgroups per CU.  While they all fit, every workgroup is
-    // resident from the start, placed for even CU totals, and nothing is left to a tail of
-    // late, short workgroups (8x12x1024x64: 32.2 -> 27.4 us; 8x12x1024x32: 22.9 -> 20.8 us);
-    // beyond that the dispatcher hands out each XCD's list longest first (32x12x1024x64:
-    // 114.4 -> 95.1 us; 4x12x4096x64: 171 -> 159 us).  Smaller launches are faster on the
-    // pipelined kernel (2x12x1024x64: 20.1 against 21.3 us).
+    // More tiles than the tile-pipelined kernel holds at once (two workgroups per CU): the
+    // block-pipelined kernel at three workgroups per CU.  While they all fit, every workgroup
+    // is resident from the start, placed for even CU totals, and nothing is left to a tail of
+    // late, short workgroups; beyond that the dispatcher hands out each XCD's list longest
+    // first.  Smaller launches are faster on the tile-pipelined kernel (2x12x2048x64: 33.6
+    // against 34.6 us).
     bool use_resident = false;
     const TileOrder* table = resident_order<D>(heads_per_xcd, p.T, &use_resident);
     static const TileOrder kNoTable = [] {
@@ -740,7 +523,7 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
       return t;
     }();
     if (const TileOrder* order = use_resident ? (table ? table : &kNoTable) : nullptr) {
-      hipLaunchKernelGGL(attn_fwd_f16_resident_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), lds,
+      hipLaunchKernelGGL(attn_fwd_f16_bp_kernel<D>, dim3(8 * n_qtiles * heads_per_xcd), dim3(256), BpCfg<D>::kLds,
                          stream, p, BH, n_qtiles, heads_per_xcd, *order);
       return;
     }

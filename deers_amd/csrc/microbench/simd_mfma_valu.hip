@@ -20,6 +20,7 @@
 #include <cstdio>
 #include <cstdlib>
 
+#include "../attn_fwd_f16_bp.h"
 #include "../common.h"
 
 using namespace deers;
@@ -381,9 +382,51 @@ static void run_fwd_iteration(const half_t* Kg, const half_t* Vg) {
   }
 }
 
+
+// ---- F: the block-pipelined forward's own loop (attn_fwd_f16_bp.h compiled in its bench mode) ----
+template <int OCC>
+__global__ __launch_bounds__(256, OCC) void fwd_bp_bench_kernel(FwdParams p, int BH, int n_qtiles, int heads_per_xcd,
+                                                                TileOrder order, int stages, long long* clk) {
+  attn_fwd_f16_bp_body<64, true>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
+}
+template <int OCC>
+static void run_fwd_bp(int wgs) {
+  const int stages = 4000, T = 1024, n_qtiles = 8, heads_per_xcd = 4 * wgs, BH = 8 * heads_per_xcd;
+  const size_t elems = (size_t)BH * T * 64;
+  half_t *q, *k, *v, *o;
+  float* lse;
+  long long* clk;
+  CK(hipMalloc(&q, elems * 2)); CK(hipMalloc(&k, elems * 2)); CK(hipMalloc(&v, elems * 2)); CK(hipMalloc(&o, elems * 2));
+  CK(hipMalloc(&lse, (size_t)BH * T * 4));
+  CK(hipMalloc(&clk, 256 * 4 * 4 * sizeof(long long)));
+  CK(hipMemset(q, 0, elems * 2)); CK(hipMemset(k, 0, elems * 2)); CK(hipMemset(v, 0, elems * 2));
+  FwdParams p{};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
+  p.sq = p.sk = p.sv = p.so = Strides3{(int64_t)T * 64, (int64_t)T * 64, 64};  // B = BH "batches" of one head
+  p.H = 1; p.T = T; p.scale_log2 = 0.18f;
+  TileOrder order{};
+  order.code[0] = -1;
+  const size_t lds = BpCfg<64>::kLds;
+  fwd_bp_bench_kernel<OCC><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, 100, clk);
+  fwd_bp_bench_kernel<OCC><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
+  CK(hipDeviceSynchronize());
+  static long long h[256 * 4 * 4];
+  CK(hipMemcpy(h, clk, sizeof(long long) * 256 * wgs * 4, hipMemcpyDeviceToHost));
+  double s = 0;
+  for (int i = 0; i < 256 * wgs * 4; ++i) s += (double)h[i];
+  const double per_stage = s / (256.0 * wgs * 4) / stages;
+  printf("F block-pipelined forward (launch bound %d), %d workgroup(s) = wave(s)/SIMD per CU: %5.0f clocks per wave-stage (32 keys) = %4.0f of SIMD time (its 8 MFMAs alone: 256)\n",
+         OCC, wgs, per_stage, per_stage / wgs);
+  CK(hipFree(q)); CK(hipFree(k)); CK(hipFree(v)); CK(hipFree(o)); CK(hipFree(lse)); CK(hipFree(clk));
+}
+
 int main() {
   CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
   CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
+  if (getenv("MICROBENCH_ONLY_F")) {
+    run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3); run_fwd_bp<2>(1); run_fwd_bp<2>(2);
+    return 0;
+  }
   run_mfma_stream();
   run_valu_rate<0>("v_fma_f32 independent");
   run_valu_rate<1>("v_fma_f32 dependent");

@@ -117,6 +117,33 @@ def test_forward_on_the_plain_kernel(B, H, T, D):
     np.testing.assert_array_equal(lse, lse2)
 
 
+@pytest.mark.parametrize("beta", [0.3, 1.5, 14.0])
+def test_forward_when_the_row_maximum_grows_late(beta):
+    """The block-pipelined forward keeps the maximum of a row's first 32 keys as its reference
+    and only moves it when a block's probabilities would leave the f16 range.  Here some keys
+    beyond the first block are aligned with every query of their head, so their scores stand
+    about 8 * beta above everything before them (11.5 * beta in the base-2 exponent: within the
+    f16 head-room, beyond it, and beyond what f32 can exponentiate), in the middle of a tile, on
+    a diagonal block and in the last block; every row must still match the oracle (forward only;
+    LSE gets a relative term: the scale is folded into the f16 queries, one rounding of 2^-12
+    per product, the precision the reference's own f16 scores have)."""
+    B, H, T, D = 8, 12, 1024, 64
+    x = synth.attention_inputs(f"late-max-{beta}", B, H, T, D, np.float16, base_seed=11)
+    q, k, v = x["q"].copy(), x["k"].copy(), x["v"].copy()
+    base = q[:, :, :1, :].astype(np.float32)                       # one direction per head
+    q = (base + 0.5 * q.astype(np.float32)).astype(np.float16)     # every query has a component along it
+    for t in (40, 333, 736, 1023):
+        k[:, :, t, :] = (beta * base[:, :, 0, :]).astype(np.float16)
+    o, lse = rocm.attn_fwd(q, k, v)
+    assert np.isfinite(o.astype(np.float32)).all() and np.isfinite(lse).all()
+    for b in (0, B - 1):
+        ro, rlse = oracle.attn_fwd(q[b:b + 1], k[b:b + 1], v[b:b + 1], return_lse=True, heads_per_call=1)
+        eo = max_err(o[b:b + 1], ro)
+        el = float(np.max(np.abs(lse[b:b + 1] - rlse) / (5e-3 + 2e-4 * np.abs(rlse))))
+        say(f"late maximum beta {beta} batch {b}: o={eo:.2e} lse/bound={el:.2f} max lse {np.max(rlse):.1f}")
+        assert eo <= 5e-3 and el <= 1.0
+
+
 def test_config3_long_context_f16():
     """B=1 H=16 T=8192 D=128 f16, sigma 0.5: GPU on all heads, oracle on heads 0 and 15."""
     x = synth.attention_inputs("c3", 1, 16, 8192, 128, np.float16, base_seed=0, sigma=0.5)
