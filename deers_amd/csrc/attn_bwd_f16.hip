@@ -34,6 +34,9 @@
 // requested P iterations ahead; one barrier per iteration.
 #include <type_traits>
 
+#include <cstdlib>
+
+#include "attn_bwd_f16_bp.h"
 #include "common.h"
 
 namespace deers {
@@ -41,7 +44,6 @@ namespace deers {
 constexpr int kBwdBlk = 128;  // rows owned by a workgroup (keys in dK/dV, queries in dQ)
 constexpr int kBwdStep = 64;  // rows of the streamed operand per iteration
 
-#define ZERO16 floatx16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define ZEROH8 half8{0, 0, 0, 0, 0, 0, 0, 0}
 
 template <int D>
@@ -567,24 +569,52 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(B
   }
 }
 
+// The same launch with the block-pipelined role bodies (head widths 32 and 64).
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_bwd_f16_bp_kernel(BwdParams p, int BH, int n_blocks, int heads_per_xcd,
+                                                                  int first_id, int dq_short_first) {
+  const int group_wgs = 8 * heads_per_xcd;
+  const int per_role = n_blocks * group_wgs;
+  const int id = (int)blockIdx.x + first_id;
+  if (id < per_role) {
+    const int group = id / group_wgs;
+    const int rank = dq_short_first ? n_blocks - 1 - group : group;
+#ifndef BP_NO_DQ
+    bwd_dq_f16_bp_body<D>(p, BH, n_blocks, heads_per_xcd, rank * group_wgs + id % group_wgs);
+#endif
+  } else {
+#ifndef BP_NO_DKDV
+    bwd_dkdv_f16_bp_body<D>(p, BH, n_blocks, heads_per_xcd, id - per_role);
+#endif
+  }
+}
+
 template <int D>
 static void launch_bwd_f16_d(const BwdParams& p, int B, int mode, hipStream_t stream) {
   const int BH = B * p.H;
   const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
   const int heads_per_xcd = (BH + 7) / 8;
   const int per_role = 8 * n_blocks * heads_per_xcd;
-  constexpr size_t lds = BwdCfg<D>::kLdsDkdv > BwdCfg<D>::kLdsDq ? BwdCfg<D>::kLdsDkdv : BwdCfg<D>::kLdsDq;
+  // head widths 32 and 64 take the block-pipelined bodies, 128 the tile bodies of this file
+  typedef void (*Kernel)(BwdParams, int, int, int, int, int);
+  Kernel kernel = attn_bwd_f16_kernel<D>;
+  size_t lds = BwdCfg<D>::kLdsDkdv > BwdCfg<D>::kLdsDq ? BwdCfg<D>::kLdsDkdv : BwdCfg<D>::kLdsDq;
+  if constexpr (D <= 64) {
+    static const int use_bp = [] { const char* e = getenv("DEERS_BWD_BP"); return e ? atoi(e) : 1; }();
+    if (use_bp) {
+      kernel = attn_bwd_f16_bp_kernel<D>;
+      lds = BwdBpCfg<D>::kLds;
+    }
+  }
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
     if (lds > 64 * 1024)
-      (void)hipFuncSetAttribute((const void*)attn_bwd_f16_kernel<D>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     attr_set = true;
   }
   if (mode == 2) {  // test hook: consumers only, so that their bounded wait runs out
     LaunchScope scope("attn_bwd_f16_dkdv", stream);
-    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
-                       n_blocks, heads_per_xcd, per_role, 0);
+    hipLaunchKernelGGL(kernel, dim3(per_role), dim3(256), lds, stream, p, BH, n_blocks, heads_per_xcd, per_role, 0);
     return;
   }
   if (mode == 1) {
@@ -598,28 +628,24 @@ static void launch_bwd_f16_d(const BwdParams& p, int B, int mode, hipStream_t st
       int dev = 0, per_cu = 0;
       hipDeviceProp_t prop;
       if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_bwd_f16_kernel<D>, 256, lds) ==
-              hipSuccess &&
-          per_cu > 0)
+          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds) == hipSuccess && per_cu > 0)
         capacity = per_cu * prop.multiProcessorCount;
       else
         capacity = -1;
     }
     const int dq_short_first = capacity > 0 && bwd_dq_short_first(8 * heads_per_xcd, capacity);
     LaunchScope scope("attn_bwd_f16", stream);
-    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(2 * per_role), dim3(256), lds, stream, p, BH,
-                       n_blocks, heads_per_xcd, 0, dq_short_first);
+    hipLaunchKernelGGL(kernel, dim3(2 * per_role), dim3(256), lds, stream, p, BH, n_blocks, heads_per_xcd, 0,
+                       dq_short_first);
     return;
   }
   {
     LaunchScope scope("attn_bwd_f16_dq", stream);
-    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
-                       n_blocks, heads_per_xcd, 0, 0);
+    hipLaunchKernelGGL(kernel, dim3(per_role), dim3(256), lds, stream, p, BH, n_blocks, heads_per_xcd, 0, 0);
   }
   {
     LaunchScope scope("attn_bwd_f16_dkdv", stream);
-    hipLaunchKernelGGL(attn_bwd_f16_kernel<D>, dim3(per_role), dim3(256), lds, stream, p, BH,
-                       n_blocks, heads_per_xcd, per_role, 0);
+    hipLaunchKernelGGL(kernel, dim3(per_role), dim3(256), lds, stream, p, BH, n_blocks, heads_per_xcd, per_role, 0);
   }
 }
 

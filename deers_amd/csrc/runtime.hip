@@ -690,7 +690,8 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   if (int rc = resolve_strides("dv", dv, dv_strides, H, T, D, elem, &p.sdv)) return rc;
   // f32: delta[B,H,T].  f16: lse2 and negdelta, rows padded to a multiple of 64 per head.
   const int64_t t_pad = (T + 63) / 64 * 64;
-  const size_t ws_floats = dtype == DEERS_ROCM_F16 ? (size_t)(2 * B * H * t_pad) : (size_t)(B * H * T);
+  // f16: + 64 floats, the block-pipelined dK/dV role loads row vectors 64 floats at a time
+  const size_t ws_floats = dtype == DEERS_ROCM_F16 ? (size_t)(2 * B * H * t_pad + 64) : (size_t)(B * H * T);
   void* ws = nullptr;
   if (int rc = workspace(ws_floats * sizeof(float), &ws)) return rc;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
