@@ -34,7 +34,6 @@
 // requested P iterations ahead; one barrier per iteration.
 #include <type_traits>
 
-#include <cstdlib>
 
 #include "attn_bwd_f16_bp.h"
 #include "common.h"
@@ -131,6 +130,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
   // flags (the statistics it then reads are not valid and this call's dK / dV are wrong):
   // the host reports it at the next synchronisation.
   auto wait_published = [&]() {
+    if (p.epoch == 0) return;  // the statistics were published by an earlier launch
     for (int base = kvblk; base < n_blocks; base += 64) {
       const int qb = base + lane;
       const int* flag = p.ready + (int64_t)bh * n_blocks + min(qb, n_blocks - 1);
@@ -139,7 +139,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_body(const BwdParams& p, int BH, in
         const int seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__all(seen == p.epoch)) break;
         if (++spins >= p.spin_limit) {
-          __hip_atomic_store(p.ready - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(p.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
         __builtin_amdgcn_s_sleep(8);
@@ -552,11 +552,15 @@ __device__ __forceinline__ void bwd_dq_f16_body(const BwdParams& p, int BH, int 
 // the stores (vmcnt 0) and sets the flag with relaxed atomics and no cache write-back,
 // which is only enough when producer and consumer share one L2, i.e. one XCD: the host
 // takes the single launch only on a device where workgroup id % 8 is known to be the XCD.
+//
+// The flags hold epochs (one per backward call, passed by the host) and are never cleared.
+// Epoch 0 means that the flags are not used: the dK/dV role does not wait.  The host passes it
+// with the two-launch form while the stream is being captured into a graph, whose replays
+// could not be given a fresh epoch each.
 template <int D>
-__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(BwdParams p, int BH,
-                                                              int n_blocks,
-                                                              int heads_per_xcd,
-                                                              int first_id, int dq_short_first) {
+__global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(BwdParams p, int BH, int n_blocks,
+                                                                               int heads_per_xcd, int first_id,
+                                                                               int dq_short_first) {
   const int group_wgs = 8 * heads_per_xcd;
   const int per_role = n_blocks * group_wgs;
   const int id = (int)blockIdx.x + first_id;
@@ -569,23 +573,24 @@ __global__ __launch_bounds__(256, (D == 128 ? 1 : 2)) void attn_bwd_f16_kernel(B
   }
 }
 
-// The same launch with the block-pipelined role bodies (head widths 32 and 64).
+// The same grid with the block-pipelined role bodies (head widths 32 and 64).
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_bwd_f16_bp_kernel(BwdParams p, int BH, int n_blocks, int heads_per_xcd,
                                                                   int first_id, int dq_short_first) {
   const int group_wgs = 8 * heads_per_xcd;
   const int per_role = n_blocks * group_wgs;
   const int id = (int)blockIdx.x + first_id;
+  int bh, rank;
   if (id < per_role) {
     const int group = id / group_wgs;
-    const int rank = dq_short_first ? n_blocks - 1 - group : group;
-#ifndef BP_NO_DQ
-    bwd_dq_f16_bp_body<D>(p, BH, n_blocks, heads_per_xcd, rank * group_wgs + id % group_wgs);
-#endif
+    const int r = dq_short_first ? n_blocks - 1 - group : group;
+    if (map_block(r * group_wgs + id % group_wgs, n_blocks, heads_per_xcd, BH, &bh, &rank))
+      bwd_dq_f16_bp_body<D>(p, __builtin_amdgcn_readfirstlane(bh), n_blocks - 1 - __builtin_amdgcn_readfirstlane(rank),
+                            n_blocks, blockIdx.x);
   } else {
-#ifndef BP_NO_DKDV
-    bwd_dkdv_f16_bp_body<D>(p, BH, n_blocks, heads_per_xcd, id - per_role);
-#endif
+    if (map_block(id - per_role, n_blocks, heads_per_xcd, BH, &bh, &rank))
+      bwd_dkdv_f16_bp_body<D>(p, __builtin_amdgcn_readfirstlane(bh), __builtin_amdgcn_readfirstlane(rank), n_blocks,
+                              blockIdx.x);
   }
 }
 
@@ -595,16 +600,12 @@ static void launch_bwd_f16_d(const BwdParams& p, int B, int mode, hipStream_t st
   const int n_blocks = (p.T + kBwdBlk - 1) / kBwdBlk;
   const int heads_per_xcd = (BH + 7) / 8;
   const int per_role = 8 * n_blocks * heads_per_xcd;
-  // head widths 32 and 64 take the block-pipelined bodies, 128 the tile bodies of this file
   typedef void (*Kernel)(BwdParams, int, int, int, int, int);
   Kernel kernel = attn_bwd_f16_kernel<D>;
   size_t lds = BwdCfg<D>::kLdsDkdv > BwdCfg<D>::kLdsDq ? BwdCfg<D>::kLdsDkdv : BwdCfg<D>::kLdsDq;
-  if constexpr (D <= 64) {
-    static const int use_bp = [] { const char* e = getenv("DEERS_BWD_BP"); return e ? atoi(e) : 1; }();
-    if (use_bp) {
-      kernel = attn_bwd_f16_bp_kernel<D>;
-      lds = BwdBpCfg<D>::kLds;
-    }
+  if constexpr (D <= 64) {  // head widths 32 and 64 take the block-pipelined bodies
+    kernel = attn_bwd_f16_bp_kernel<D>;
+    lds = BwdBpCfg<D>::kLds;
   }
   static bool attr_set = false;  // launches are serialised by the caller
   if (!attr_set) {
@@ -620,9 +621,7 @@ static void launch_bwd_f16_d(const BwdParams& p, int B, int mode, hipStream_t st
   if (mode == 1) {
     // Device capacity in workgroups of this kernel, found once (launches are serialised by
     // the caller).  The shortest-first dQ order pays when the longest dQ groups would
-    // otherwise hold the device to themselves: measured on 8x12x1024 launches it is
-    // 2-3 % (D = 64, 128) to 10 % (D = 32) faster, and 2 % slower on launches of few heads
-    // and many block lengths (2x12x2048x64, 1x16x8192x128), whose groups are small.
+    // otherwise hold the device to themselves.
     static int capacity = 0;
     if (capacity == 0) {
       int dev = 0, per_cu = 0;

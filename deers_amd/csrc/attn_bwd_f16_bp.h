@@ -67,8 +67,8 @@ __device__ __forceinline__ uint32_t pack_pair_f16(float a, float b) {
 // dK / dV
 // ---------------------------------------------------------------------------
 template <int D>
-__device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH, int n_own, int heads_per_xcd,
-                                                     int block_id) {
+__device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh, int kvblk, int n_own,
+                                                     [[maybe_unused]] int trace_row) {
   using Cfg = BwdBpCfg<D>;
   constexpr int R = Cfg::R, F = Cfg::F, RB = Cfg::RB, TB = Cfg::TB, VEC_B = Cfg::VEC_B, SLOT_B = Cfg::SLOT_DKDV;
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -84,14 +84,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  int bh, rank;
-  if (!map_block(block_id, n_own, heads_per_xcd, BH, &bh, &rank)) return;
-  bh = __builtin_amdgcn_readfirstlane(bh);
-  const int kvblk = __builtin_amdgcn_readfirstlane(rank);  // key block 0 walks the most queries
-  [[maybe_unused]] const int trace_row = blockIdx.x;
-  [[maybe_unused]] const int trace_len = 0;
-  DEERS_TRACE_POINT(0);
-  set_block_priority(kvblk, n_own);
+  DEERS_TRACE_POINT(0);  // key block 0 walks the most queries
   const int b_ = bh / p.H, h_ = bh % p.H;
   const half_t* Q = (const half_t*)p.q + b_ * p.sq.b + h_ * p.sq.h;
   const half_t* K = (const half_t*)p.k + b_ * p.sk.b + h_ * p.sk.h;
@@ -110,40 +103,44 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
   const uint32_t lds0 = lds_address(smem);
   const int sqt = (int)p.sq.t, sdot = (int)p.sdo.t;
 
-  // ---- this wave's loads of a stage: NLT of the 2 * TB / 1024 tile loads (first half Q, second
-  // half dO; a load covers RPW rows) and its two row vectors ----
+  // ---- this wave's loads of a stage: NLT of the 2 * TB / 1024 tile loads (waves 0 and 1 fetch
+  // the Q block, waves 2 and 3 the dO block; a load covers RPW rows) and its two row vectors.
+  // Lane offsets are fixed; rows past T-1 of a last, partial block read row T-1 (their
+  // statistics give probability 0). ----
   constexpr int NLH = TB / 1024;
-  uint32_t ld_off[NLT], ld_dst[NLT];
+  const bool w_do = wave * NLT >= NLH;  // wave-uniform
+  const half_t* tbase = w_do ? dO : Q;
+  const int tstride = w_do ? sdot : sqt;
+  const bool partial = (T & (kBwdBpBlk - 1)) != 0;
+  uint32_t ld_off[NLT], ld_off_last[NLT], ld_dst[NLT];
 #pragma unroll
   for (int i = 0; i < NLT; ++i) {
-    const int n = wave * NLT + i;
-    const bool is_do = n >= NLH;
-    const int row = (is_do ? n - NLH : n) * RPW + lane / CH;
+    const int n = (wave * NLT + i) % NLH;
+    const int row = n * RPW + lane / CH;
     const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-    ld_off[i] = (uint32_t)(row * (is_do ? sdot : sqt) * 2 + col);
-    ld_dst[i] = lds0 + (is_do ? TB + (n - NLH) * 1024 : n * 1024);
+    ld_off[i] = (uint32_t)(row * tstride * 2 + col);
+    ld_off_last[i] = (uint32_t)(min(row, T - 1 - last_blk * kBwdBpBlk) * tstride * 2 + col);
+    ld_dst[i] = lds0 + (w_do ? TB : 0) + n * 1024;
   }
   const uint32_t vec_dst = lds0 + 2 * TB + wave * 2 * VEC_B;
-  auto request = [&](int nb, uint32_t slot) {  // relative block nb -> ring slot
+  // The loads of relative block nb into ring slot `slot`, one instruction per part (tile loads,
+  // then the two row vectors: the block's 32 floats, twice, since a wave load writes 64;
+  // nothing outside the block is read, so no line of rows that are not published yet enters
+  // this CU's L1).
+  auto request_part = [&](int part, int nb, uint32_t slot) {
     const int blk = min(blk0 + min(max(nb, 0), n_blk - 1), last_blk);
-    const half_t* qbase = Q + (uint32_t)(blk * kBwdBpBlk * sqt);
-    const half_t* dobase = dO + (uint32_t)(blk * kBwdBpBlk * sdot);
-#pragma unroll
-    for (int i = 0; i < NLT; ++i) {
-      const bool is_do = wave * NLT + i >= NLH;  // wave-uniform
-      uint32_t off = ld_off[i];
-      if (blk == last_blk) {  // rows past T-1 read row T-1 (their statistics give probability 0)
-        const int n = wave * NLT + i;
-        const int row = (is_do ? n - NLH : n) * RPW + lane / CH;
-        const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-        off = (uint32_t)(min(row, T - 1 - last_blk * kBwdBpBlk) * (is_do ? sdot : sqt) * 2 + col);
-      }
-      async_load16_to_lds(is_do ? dobase : qbase, off, ld_dst[i] + slot * SLOT_B);
+    if (part < NLT) {
+      const uint32_t off = partial && blk == last_blk ? ld_off_last[part] : ld_off[part];
+      async_load16_to_lds(tbase + (uint32_t)(blk * kBwdBpBlk * tstride), off, ld_dst[part] + slot * SLOT_B);
+    } else if (part == NLT) {
+      async_load4_to_lds(neglse2 + blk * kBwdBpBlk, (lane & 31) * 4, vec_dst + slot * SLOT_B);
+    } else {
+      async_load4_to_lds(negdelta + blk * kBwdBpBlk, (lane & 31) * 4, vec_dst + VEC_B + slot * SLOT_B);
     }
-    // row vectors: 64 floats from the block's first row (the workspace is padded; the upper 32
-    // are not read back)
-    async_load4_to_lds(neglse2 + blk * kBwdBpBlk, lane * 4, vec_dst + slot * SLOT_B);
-    async_load4_to_lds(negdelta + blk * kBwdBpBlk, lane * 4, vec_dst + VEC_B + slot * SLOT_B);
+  };
+  auto request = [&](int nb, uint32_t slot) {
+#pragma unroll
+    for (int part = 0; part < LPI; ++part) request_part(part, nb, slot);
   };
 
   // K^T (scaled) and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.  Rows past
@@ -162,7 +159,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
   // The row statistics of query block qb come from the dQ workgroup that owns it (same launch,
   // same XCD).  Poll the flags of all the 128-row query blocks this workgroup will walk, one
   // per lane, before the first request; bounded, and a wait that runs out raises the error word.
-  {
+  if (p.epoch != 0) {  // epoch 0: the statistics were published by an earlier launch
     for (int base = kvblk; base < n_own; base += 64) {
       const int qb = base + lane;
       const int* flag = p.ready + (int64_t)bh * n_own + min(qb, n_own - 1);
@@ -171,7 +168,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
         const int seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__all(seen == p.epoch)) break;
         if (++spins >= p.spin_limit) {
-          __hip_atomic_store(p.ready - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(p.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
         __builtin_amdgcn_s_sleep(8);
@@ -233,33 +230,48 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
     return lds_read_half8_at(aa[mi >> 1] + slot * SLOT_B + ((mi & 1) ? TB : 0));
   };
   // accumulator seeds of the block in `slot`: S from -lse2, dP from -delta (row values)
-  auto seed = [&](floatx16& s, floatx16& dp, uint32_t slot) {
+  // One eighth of the accumulator seeds of the block in `slot`: part 2 rq gives S rows from
+  // -lse2, part 2 rq + 1 gives dP rows from -delta (row values, the same for every lane of a half)
+  auto seed_part = [&](int part, floatx16& s, floatx16& dp, uint32_t slot) {
+    const int rq = part >> 1;
+    const floatx4 a = lds_read_float4_at(va + slot * SLOT_B + ((part & 1) ? VEC_B : 0) + 32 * rq);
 #pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      const floatx4 a = lds_read_float4_at(va + slot * SLOT_B + 32 * rq);
-      const floatx4 b = lds_read_float4_at(va + slot * SLOT_B + VEC_B + 32 * rq);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 4; ++e) {
+      if (part & 1)
+        dp[4 * rq + e] = a[e];
+      else
         s[4 * rq + e] = a[e];
-        dp[4 * rq + e] = b[e];
-      }
     }
   };
 
   // One stage (relative block n in ring slot SLOT = n % R), entered right after its barrier.
   // (s, dp) = S and dP of block n; (sn, dpn) = those of block n+1, produced here.  FIRST: n == 0,
-  // no block n-1.  Order of the MFMAs: the consumers of block n-1 (their first W fragments are
-  // in fr already), then the producers of block n+1.  Ends by fetching the first fragments of
-  // block n's consumers for the next stage.
+  // no block n-1.  A wave issues one instruction every four clocks at best, and only what
+  // follows an MFMA within its 32 clocks costs nothing: so everything a stage does is spread
+  // over its 16 chunks, one MFMA each: the consumers of block n-1 first (their first W fragments
+  // were fetched by the previous stage), then the producers of block n+1, each followed by the
+  // fetch of a fragment W MFMAs ahead (rolling into the next stage's consumers, which read
+  // block n), by one of the eight seed reads, by one of the loads that refill the slot of
+  // block n-2 with block n+1+F, and by the exponential, product and packing of block n.
   auto stage = [&](auto first_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s, floatx16& dp,
                    floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
     constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + NM1;
-    constexpr int NPRE = FIRST ? 0 : (NM2 < W ? NM2 : W);
+    constexpr int NPRE = NM2 < W ? NM2 : W;  // fragments a stage finds fetched
+    // whether the fetches can roll on into the next stage (a fragment must land in the register
+    // its MFMA names, which is the one just freed only if the counts are multiples of W)
+    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0;
+    const uint32_t RSLOT = (SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
+    if constexpr (FIRST) {
 #pragma unroll
-    for (int mi = NPRE; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
-    seed(sn, dpn, NSLOT);
+      for (int mi = 0; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
+#pragma unroll
+      for (int part = 0; part < 8; ++part) seed_part(part, sn, dpn, NSLOT);
+    } else {
+#pragma unroll
+      for (int mi = NPRE; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
+    }
     __builtin_amdgcn_sched_barrier(0);
     uint32_t pw[8], dw[8];
     auto finish_pair = [&](int i) {  // f16 packing of the pair finished in chunk 2i+1
@@ -284,17 +296,23 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
           else
             sn = mfma_f16(fr[mi % W], kf[ks], sn);
         }
-        if (mi + W < NMS) fr[mi % W] = fetch(mi + W);
+        if (mi + W < NMS)
+          fr[mi % W] = fetch(mi + W);
+        else if (ROLL && mi + W - NMS < NPRE)
+          fr[mi % W] = fetch2(mi + W - NMS, SLOT);
       }
+      if (!FIRST && i < 8) seed_part(i, sn, dpn, NSLOT);
+      if (i >= 1 && i <= LPI) request_part(i - 1, n + 1 + F, RSLOT);
       s[i] = fast_exp2(s[i]);
       if (i > 0) dp[i - 1] = s[i - 1] * dp[i - 1];
       if (i > 2 && (i & 1)) finish_pair((i - 3) >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     dp[15] = s[15] * dp[15];
-    // the next stage's first fragments (consumers of block n) leave LDS now
+    if constexpr (!ROLL) {
 #pragma unroll
-    for (int mi = 0; mi < W && mi < NM2; ++mi) fr[mi] = fetch2(mi, SLOT);
+      for (int mi = 0; mi < NPRE; ++mi) fr[mi] = fetch2(mi, SLOT);
+    }
     finish_pair(7);
     // Causal mask, on the packed pairs: query row 32 (blk0 + n) + 8 (r/4) + 4g + r%4 of register r
     // against this lane's key.  Only the wave's first blocks have masked entries.
@@ -320,7 +338,8 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
 
   // ---- S, dP of block 0 ----
   floatx16 sa, dpa, sb, dpb;
-  seed(sa, dpa, 0);
+#pragma unroll
+  for (int part = 0; part < 8; ++part) seed_part(part, sa, dpa, 0);
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     sa = mfma_f16(fetch1(2 * ks, 0), kf[ks], sa);
@@ -328,24 +347,23 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
   }
   // ---- stage n: barrier n retires the reads of block n-2, whose slot request(n) refills with
   // block n+1+F, and makes block n+1 (requested F stages ago) visible ----
-  auto open_stage = [&](uint32_t refill_slot, int n) {
+  auto open_stage = [&]() {
     wait_vmcnt<(F - 1) * LPI>();
     // bare barrier: the LDS reads in flight (next stage's first fragments) touch slots that are
     // not refilled for two more stages
     __builtin_amdgcn_s_barrier();
-    request(n + 1 + F, refill_slot);
   };
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
   DEERS_TRACE_POINT(2);
-  open_stage((1 + F) % R, 0);
+  open_stage();
   stage(yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
     const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
-    open_stage((slot + 1 + F) % R, n);
+    open_stage();
     stage(no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
-    open_stage((s1 + 1 + F) % R, n + 1);
+    open_stage();
     stage(no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
   // Stages 1 .. n_blk, rounded up to an even count (the closing stages only consume: their own
@@ -376,11 +394,11 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int BH,
 }
 
 // ---------------------------------------------------------------------------
-// dQ (and the row statistics)
+// dQ
 // ---------------------------------------------------------------------------
 template <int D>
-__device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, int n_own, int heads_per_xcd,
-                                                   int block_id) {
+__device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, int qtile, int n_own,
+                                                   [[maybe_unused]] int trace_row) {
   using Cfg = BwdBpCfg<D>;
   constexpr int R = Cfg::R, F = Cfg::F, RB = Cfg::RB, TB = Cfg::TB, SLOT_B = Cfg::SLOT_DQ;
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -394,20 +412,12 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
-  int bh, rank;
-  if (!map_block(block_id, n_own, heads_per_xcd, BH, &bh, &rank)) return;
-  bh = __builtin_amdgcn_readfirstlane(bh);
-  rank = __builtin_amdgcn_readfirstlane(rank);
-  const int qtile = n_own - 1 - rank;  // the last query block walks the most keys
-  [[maybe_unused]] const int trace_row = blockIdx.x;
-  DEERS_TRACE_POINT(0);
-  set_block_priority(rank, n_own);
+  DEERS_TRACE_POINT(0);  // the last query block walks the most keys
   const int b_ = bh / p.H, h_ = bh % p.H;
   const half_t* Q = (const half_t*)p.q + b_ * p.sq.b + h_ * p.sq.h;
   const half_t* K = (const half_t*)p.k + b_ * p.sk.b + h_ * p.sk.h;
   const half_t* V = (const half_t*)p.v + b_ * p.sv.b + h_ * p.sv.h;
   const half_t* dO = (const half_t*)p.d_o + b_ * p.sdo.b + h_ * p.sdo.h;
-  const half_t* O = (const half_t*)p.o + b_ * p.so.b + h_ * p.so.h;
   half_t* dQ = (half_t*)p.dq + b_ * p.sdq.b + h_ * p.sdq.h;
   const int q0 = qtile * kBwdBpOwn, qw0 = q0 + 32 * wave, qrow = qw0 + (lane & 31);
   const int n_blk = (min(q0 + kBwdBpOwn - 1, T - 1) >> 5) + 1;  // key blocks 0 .. n_blk-1
@@ -415,67 +425,70 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
   const int last_blk = (T - 1) >> 5;
   const uint32_t lds0 = lds_address(smem);
   const int skt = (int)p.sk.t, svt = (int)p.sv.t;
+  // This wave's LPI tile loads of a stage (waves 0 and 1 fetch the K block, waves 2 and 3 the
+  // V block); rows past T-1 of a last, partial block read row T-1 (masked for every query).
   constexpr int NLH = TB / 1024;
-  uint32_t ld_off[LPI], ld_dst[LPI];
+  const bool w_v = wave * LPI >= NLH;  // wave-uniform
+  const half_t* tbase = w_v ? V : K;
+  const int tstride = w_v ? svt : skt;
+  const bool partial = (T & (kBwdBpBlk - 1)) != 0;
+  uint32_t ld_off[LPI], ld_off_last[LPI], ld_dst[LPI];
 #pragma unroll
   for (int i = 0; i < LPI; ++i) {
-    const int n = wave * LPI + i;
-    const bool is_v = n >= NLH;
-    const int row = (is_v ? n - NLH : n) * RPW + lane / CH;
+    const int n = (wave * LPI + i) % NLH;
+    const int row = n * RPW + lane / CH;
     const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-    ld_off[i] = (uint32_t)(row * (is_v ? svt : skt) * 2 + col);
-    ld_dst[i] = lds0 + (is_v ? TB + (n - NLH) * 1024 : n * 1024);
+    ld_off[i] = (uint32_t)(row * tstride * 2 + col);
+    ld_off_last[i] = (uint32_t)(min(row, T - 1 - last_blk * kBwdBpBlk) * tstride * 2 + col);
+    ld_dst[i] = lds0 + (w_v ? TB : 0) + n * 1024;
   }
-  auto request = [&](int nb, uint32_t slot) {
+  auto request_part = [&](int part, int nb, uint32_t slot) {
     const int blk = min(max(nb, 0), n_blk - 1);
-    const half_t* kbase = K + (uint32_t)(blk * kBwdBpBlk * skt);
-    const half_t* vbase = V + (uint32_t)(blk * kBwdBpBlk * svt);
+    const uint32_t off = partial && blk == last_blk ? ld_off_last[part] : ld_off[part];
+    async_load16_to_lds(tbase + (uint32_t)(blk * kBwdBpBlk * tstride), off, ld_dst[part] + slot * SLOT_B);
+  };
+  auto request = [&](int nb, uint32_t slot) {
 #pragma unroll
-    for (int i = 0; i < LPI; ++i) {
-      const bool is_v = wave * LPI + i >= NLH;
-      uint32_t off = ld_off[i];
-      if (blk == last_blk) {
-        const int n = wave * LPI + i;
-        const int row = (is_v ? n - NLH : n) * RPW + lane / CH;
-        const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-        off = (uint32_t)(min(row, T - 1 - last_blk * kBwdBpBlk) * (is_v ? svt : skt) * 2 + col);
-      }
-      async_load16_to_lds(is_v ? vbase : kbase, off, ld_dst[i] + slot * SLOT_B);
-    }
+    for (int part = 0; part < LPI; ++part) request_part(part, nb, slot);
   };
 
-  // Q (scaled), dO as B operands and this row's statistics.  Rows past T-1 read row T-1: their
-  // dQ rows are not stored and a query owns its accumulator column.
+  // Q (scaled) and dO as B operands.  Rows past T-1 read row T-1: their dQ rows are not stored
+  // and a query owns its accumulator column.
   half8 qf[KS], dof[KS];
-  float dsum = 0.f, lse_row;
   {
     const int lrow = min(qrow, T - 1);
     const half_t* qp = Q + (int64_t)lrow * p.sq.t + 8 * g;
     const half_t* dop = dO + (int64_t)lrow * p.sdo.t + 8 * g;
-    const half_t* op = O + (int64_t)lrow * p.so.t + 8 * g;
-    half8 of[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       qf[ks] = *(const half8*)(qp + 16 * ks);
       dof[ks] = *(const half8*)(dop + 16 * ks);
-      of[ks] = *(const half8*)(op + 16 * ks);
     }
-    lse_row = p.lse[(int64_t)bh * T + lrow];
+  }
+#pragma unroll
+  for (int nb = 0; nb <= F; ++nb) request(nb, nb % R);
+  // This row's statistics, published for the dK/dV role: rows in the padding [T, t_pad) get
+  // -lse2 = -inf and -delta = 0, i.e. probability 0.
+  float nl2, nd;
+  {
+    const int lrow = min(qrow, T - 1);
+    const half_t* op = (const half_t*)p.o + b_ * p.so.b + h_ * p.so.h + (int64_t)lrow * p.so.t + 8 * g;
+    half8 of[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) of[ks] = *(const half8*)(op + 16 * ks);
+    const float lse_row = p.lse[(int64_t)bh * T + lrow];
+    float dsum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int e = 0; e < 8; ++e) dsum += (float)dof[ks][e] * (float)of[ks][e];
     if (qrow >= T) dsum = 0.f;
-  }
-#pragma unroll
-  for (int nb = 0; nb <= F; ++nb) request(nb, nb % R);
-  // Published for the dK/dV role: rows in the padding [T, t_pad) get -lse2 = -inf and -delta = 0,
-  // i.e. probability 0.
-  const float nd = -pair_sum(dsum);
-  const float nl2 = qrow < T ? -lse_row * kLog2e : -INFINITY;
-  if (g == 0 && qrow < p.t_pad) {
-    p.lse2[(int64_t)bh * p.t_pad + qrow] = nl2;
-    p.negdelta[(int64_t)bh * p.t_pad + qrow] = nd;
+    nd = -pair_sum(dsum);
+    nl2 = qrow < T ? -lse_row * kLog2e : -INFINITY;
+    if (g == 0 && qrow < p.t_pad) {
+      p.lse2[(int64_t)bh * p.t_pad + qrow] = nl2;
+      p.negdelta[(int64_t)bh * p.t_pad + qrow] = nd;
+    }
   }
   floatx16 nl16, nd16;  // initial values of the S^T and dP^T accumulators (this lane's query)
 #pragma unroll
@@ -503,7 +516,7 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   half8 dsf[2];
   half8 fr[W];
-  wait_all_vmem();  // fragments loaded, statistics stored
+  wait_all_vmem();
   {
     const float c = p.scale_log2;
 #pragma unroll
@@ -512,11 +525,10 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
       for (int e = 0; e < 8; ++e) qf[ks][e] = (half_t)((float)qf[ks][e] * c);
   }
   __syncthreads();
-  if (tid == 0) {
-    // every wave drained its stores of the statistics before this barrier: the rows are in the
-    // XCD's L2, tell the dK/dV workgroups
+  // every wave drained its stores of the statistics before this barrier: the rows are in the
+  // XCD's L2, tell the dK/dV workgroups
+  if (tid == 0)
     __hip_atomic_store(p.ready + (int64_t)bh * n_own + qtile, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
 
   auto fetch2 = [&](int mi, uint32_t slot) -> half8 {  // dQ: (step, output block) = (mi / DB, mi % DB), K^T
     const int st = mi / DB, db = mi % DB;
@@ -529,14 +541,19 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
     return lds_read_half8_at(aa[mi >> 1] + slot * SLOT_B + ((mi & 1) ? TB : 0));
   };
 
+  // One stage, spread over 16 chunks as in the dK/dV role: the consumers of block n-1 (dQ), the
+  // producers of block n+1 (S^T, dP^T), the rolling fragment fetches, the loads that refill the
+  // slot of block n-2, and the vector ops of block n.
   auto stage = [&](auto first_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s, floatx16& dp,
                    floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
     constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + NM1;
-    constexpr int NPRE = FIRST ? 0 : (NM2 < W ? NM2 : W);
+    constexpr int NPRE = NM2 < W ? NM2 : W;
+    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0;
+    const uint32_t RSLOT = (SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
 #pragma unroll
-    for (int mi = NPRE; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
+    for (int mi = FIRST ? 0 : NPRE; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
     __builtin_amdgcn_sched_barrier(0);
     uint32_t dw[8];
     auto finish_pair = [&](int i) {
@@ -557,16 +574,22 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
           else
             sn = mfma_f16(fr[mi % W], qf[ks], ks == 0 ? nl16 : sn);
         }
-        if (mi + W < NMS) fr[mi % W] = fetch(mi + W);
+        if (mi + W < NMS)
+          fr[mi % W] = fetch(mi + W);
+        else if (ROLL && mi + W - NMS < NPRE)
+          fr[mi % W] = fetch2(mi + W - NMS, SLOT);
       }
+      if (i >= 1 && i <= LPI) request_part(i - 1, n + 1 + F, RSLOT);
       s[i] = fast_exp2(s[i]);
       if (i > 0) dp[i - 1] = s[i - 1] * dp[i - 1];
       if (i > 2 && (i & 1)) finish_pair((i - 3) >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     dp[15] = s[15] * dp[15];
+    if constexpr (!ROLL) {
 #pragma unroll
-    for (int mi = 0; mi < W && mi < NM2; ++mi) fr[mi] = fetch2(mi, SLOT);
+      for (int mi = 0; mi < NPRE; ++mi) fr[mi] = fetch2(mi, SLOT);
+    }
     finish_pair(7);
     // Causal mask on the packed pairs: key 32 n + 8 (r/4) + 4g + r%4 of register r against this
     // lane's query; from the wave's diagonal block on (blocks beyond it are masked entirely).
@@ -591,22 +614,21 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int BH, i
     sa = mfma_f16(fetch1(2 * ks, 0), qf[ks], ks == 0 ? nl16 : sa);
     dpa = mfma_f16(fetch1(2 * ks + 1, 0), dof[ks], ks == 0 ? nd16 : dpa);
   }
-  auto open_stage = [&](uint32_t refill_slot, int n) {
+  auto open_stage = [&]() {
     wait_vmcnt<(F - 1) * LPI>();
     __builtin_amdgcn_s_barrier();
-    request(n + 1 + F, refill_slot);
   };
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
   DEERS_TRACE_POINT(2);
-  open_stage((1 + F) % R, 0);
+  open_stage();
   stage(yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
     const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
-    open_stage((slot + 1 + F) % R, n);
+    open_stage();
     stage(no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
-    open_stage((s1 + 1 + F) % R, n + 1);
+    open_stage();
     stage(no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
   // Stages 1 .. n_blk, rounded up to an even count (the closing stages only consume: their own

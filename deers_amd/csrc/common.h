@@ -236,11 +236,11 @@ struct BwdParams {
   // f16 path workspace, rows padded to a multiple of 64 per head (t_pad):
   // lse2 = LSE*log2(e) (+inf in the padding), negdelta = -rowsum(dO o O) (0 in the padding)
   float* lse2; float* negdelta; int t_pad;
-  // ready[bh * n_blocks + q_block] == epoch once the dQ workgroup of that 128-row query
-  // block has published its lse2 / negdelta rows (f16 path, single-launch backward)
-  // ready[-1] is the hand-over error word: set to 1 by a dK/dV workgroup whose bounded
-  // wait for a flag ran out (spin_limit polls), read by the host after the next sync
-  int* ready; int epoch; int spin_limit;
+  // ready[bh * n_blocks + q_block] == epoch once the lse2 / negdelta rows of that 128-row
+  // query block are published (f16 path, hand-over inside one launch); epoch 0: the flags
+  // are not used (two launches in stream order).  *error is set to 1 by a workgroup whose
+  // bounded wait for a flag ran out (spin_limit polls) and read by the host after the next sync.
+  int* ready; int* error; int epoch; int spin_limit;
   void* dq; void* dk; void* dv;
   Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
   int H, T;

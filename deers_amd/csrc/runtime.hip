@@ -696,11 +696,25 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   if (int rc = workspace(ws_floats * sizeof(float), &ws)) return rc;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
   p.delta = static_cast<float*>(ws);
+  // A launch that is being captured into a graph gets no fresh epoch on replay: it takes the
+  // two-launch form with the flags switched off (epoch 0).  The workspace and the flags must
+  // have been grown by an earlier, eager call of the same geometry: capture allows neither
+  // the synchronisation nor the allocation.
+  bool capturing = false;
   if (dtype == DEERS_ROCM_F16) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(g_rt.stream, &cs));
+    capturing = cs != hipStreamCaptureStatusNone;
     const size_t n_flags = (size_t)(B * H) * (size_t)((T + 127) / 128);
     if (n_flags > g_rt.bwd_ready_len || g_rt.bwd_epoch == INT32_MAX) {
+      if (capturing)
+        return fail(DEERS_ROCM_ERR_ARG,
+                    "attn_bwd: call once outside stream capture with this geometry first (the "
+                    "hand-over flags have to grow)");
       if (g_rt.bwd_ready) {
         HIP_TRY(hipStreamSynchronize(g_rt.stream));
+        // an error raised by a launch before this point is reported by this call
+        if (int rc = check_handover_error()) return rc;
         HIP_TRY(hipFree(g_rt.bwd_ready));
         g_rt.bwd_ready = nullptr;
       }
@@ -710,11 +724,12 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
       g_rt.bwd_ready_len = want;
       g_rt.bwd_epoch = 0;
     }
+    p.error = g_rt.bwd_ready;
     p.ready = g_rt.bwd_ready + 1;
-    p.epoch = ++g_rt.bwd_epoch;
+    p.epoch = capturing ? 0 : ++g_rt.bwd_epoch;
     p.spin_limit = g_rt.bwd_spin_limit;
   }
-  const bool single_launch = same_xcd_handover_now();
+  const bool single_launch = !capturing && same_xcd_handover_now();
   p.lse2 = static_cast<float*>(ws);
   p.negdelta = static_cast<float*>(ws) + B * H * t_pad;
   p.t_pad = (int)t_pad;

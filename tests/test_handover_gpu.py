@@ -127,3 +127,48 @@ def test_a_wait_that_runs_out_is_reported_and_then_cleared(gpu):
     rocm.sync()
     for a, b in zip(good, again):
         np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.gpu
+def test_captured_backward_replays_correctly(gpu):
+    """A replayed graph cannot be given a fresh hand-over epoch, so a backward that is being
+    captured takes the two-launch form without the flags.  The captured backward is replayed
+    three times, with eager backwards of another geometry and synchronisations between the
+    replays, and every replay must give the eager result bit for bit."""
+    import ctypes
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    B, H, T, D = 2, 3, 300, 64
+    x = synth.attention_inputs("handover-graph", B, H, T, D, np.float16, base_seed=14)
+    y = synth.attention_inputs("handover-graph-other", 1, 2, 129, 32, np.float16, base_seed=15)
+    rocm.set_handover_mode(rocm.HANDOVER_SAME_XCD)
+    want = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])  # also grows the workspace and the flags
+    rocm.sync()
+    bufs = [rocm.DeviceBuffer.from_numpy(x[n]) for n in ("q", "k", "v", "do")]
+    o, lse = rocm.DeviceBuffer.from_numpy(want[0]), rocm.DeviceBuffer.from_numpy(want[1])
+    grads = [rocm.DeviceBuffer((B, H, T, D), np.float16) for _ in range(3)]
+    stream = ctypes.c_void_p(rocm.load().deers_rocm_stream())
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 2) == 0  # hipStreamCaptureModeRelaxed
+    try:
+        rocm.attn_bwd_raw(np.float16, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, o.ptr, lse.ptr, bufs[3].ptr,
+                          grads[0].ptr, grads[1].ptr, grads[2].ptr, B, H, T, D, rocm.default_scale(D))
+    finally:
+        assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+    nan = np.full((B, H, T, D), np.nan, np.float16)
+    try:
+        for replay in range(3):
+            for gbuf in grads:  # poison the outputs
+                rocm.load().deers_rocm_htod(gbuf.ptr, nan.ctypes.data_as(ctypes.c_void_p),
+                                            ctypes.c_size_t(gbuf.nbytes))
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            rocm.sync()
+            for name, gbuf, ref in zip(("dq", "dk", "dv"), grads, want[2:]):
+                np.testing.assert_array_equal(gbuf.numpy(), ref, err_msg=f"replay {replay}: {name}")
+            # eager work between the replays: other geometry, other flags, epochs move on
+            rocm.attn_fwd_bwd(y["q"], y["k"], y["v"], y["do"])
+            rocm.sync()
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
