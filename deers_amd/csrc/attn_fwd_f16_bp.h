@@ -125,38 +125,35 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
   const uint32_t lds0 = lds_address(smem);
   const int last_blk = (T - 1) >> 5;  // the block that holds row T-1: its rows are clamped
   const int skt = (int)p.sk.t, svt = (int)p.sv.t;
-  // This wave's loads of a stage: numbers wave * LPI + i of the stage's NL loads (first half K,
-  // second half V); a load covers RPW rows.  lane -> (row, 16-byte chunk), chunk swizzled.
+  // This wave's LPI loads of a stage (waves 0 and 1 fetch the K block, waves 2 and 3 the V
+  // block; a load covers RPW rows).  lane -> (row, 16-byte chunk), chunk swizzled; rows past T-1
+  // of a last, partial block read row T-1.
   constexpr int NLH = Cfg::NL / 2;
-  uint32_t ld_off[LPI], ld_dst[LPI];
+  const bool w_v = wave * LPI >= NLH;  // wave-uniform
+  const half_t* tbase = w_v ? V : K;
+  const int tstride = w_v ? svt : skt;
+  const bool partial = (T & (kBpBlk - 1)) != 0;
+  uint32_t ld_off[LPI], ld_off_last[LPI], ld_dst[LPI];
 #pragma unroll
   for (int i = 0; i < LPI; ++i) {
-    const int n = wave * LPI + i;
-    const bool is_v = n >= NLH;
-    const int row = (is_v ? n - NLH : n) * RPW + lane / CH;
+    const int n = (wave * LPI + i) % NLH;
+    const int row = n * RPW + lane / CH;
     const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-    ld_off[i] = (uint32_t)(row * (is_v ? svt : skt) * 2 + col);
-    ld_dst[i] = lds0 + (is_v ? R * TB + (n - NLH) * 1024 : n * 1024);
+    ld_off[i] = (uint32_t)(row * tstride * 2 + col);
+    ld_off_last[i] = (uint32_t)(min(row, T - 1 - last_blk * kBpBlk) * tstride * 2 + col);
+    ld_dst[i] = lds0 + (w_v ? R * TB : 0) + n * 1024;
   }
-  // Requests K block kb into ring slot kslot and V block vb into vslot.  Blocks outside
-  // [0, n_blk) are clamped: they are never consumed.
+  // Load `part` of the request of K block kb into ring slot kslot and V block vb into vslot.
+  // Blocks outside [0, n_blk) are clamped: they are never consumed.
+  auto request_part = [&](int part, int kb, int vb, uint32_t kslot, uint32_t vslot) {
+    const int want = w_v ? vb : kb;
+    const int blk = BENCH ? (want & 15) : min(max(want, 0), n_blk - 1);
+    const uint32_t off = partial && blk == last_blk ? ld_off_last[part] : ld_off[part];
+    async_load16_to_lds(tbase + (uint32_t)(blk * kBpBlk * tstride), off, ld_dst[part] + (w_v ? vslot : kslot) * TB);
+  };
   auto request = [&](int kb, int vb, uint32_t kslot, uint32_t vslot) {
-    const int kc = BENCH ? (kb & 15) : min(max(kb, 0), n_blk - 1), vc = BENCH ? (vb & 15) : min(max(vb, 0), n_blk - 1);
-    const half_t* kbase = K + (uint32_t)(kc * kBpBlk * skt);
-    const half_t* vbase = V + (uint32_t)(vc * kBpBlk * svt);
 #pragma unroll
-    for (int i = 0; i < LPI; ++i) {
-      const bool is_v = wave * LPI + i >= NLH;  // wave-uniform
-      const int blk = is_v ? vc : kc;
-      uint32_t off = ld_off[i];
-      if (blk == last_blk) {  // rows past T-1 read row T-1
-        const int n = wave * LPI + i;
-        const int row = (is_v ? n - NLH : n) * RPW + lane / CH;
-        const int col = 16 * ((lane % CH) ^ lds_swizzle<CH>(row));
-        off = (uint32_t)(min(row, T - 1 - last_blk * kBpBlk) * (is_v ? svt : skt) * 2 + col);
-      }
-      async_load16_to_lds(is_v ? vbase : kbase, off, ld_dst[i] + (is_v ? vslot : kslot) * TB);
-    }
+    for (int part = 0; part < LPI; ++part) request_part(part, kb, vb, kslot, vslot);
   };
   // Q fragments first (ordinary loads), then K(0) .. K(F), V(0) .. V(F-1)
   half8 qf[KS];
@@ -227,14 +224,11 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
   // -m of this lane's row, four copies: lane l of wave w owns 16 bytes at seed_at
   const uint32_t seed_at = lds0 + (uint32_t)Cfg::kRings + wave * 1024 + lane * 16;
   auto set_negm = [&]() { *(DEERS_LDS floatx4*)(uintptr_t)seed_at = floatx4{-m, -m, -m, -m}; };
-  auto seed = [&](floatx16& s) {  // s = -m in every register
+  auto seed_part = [&](int j, floatx16& s) {  // registers 4j .. 4j+3 of s = -m
+    // volatile: four separate reads (one read and twelve register moves otherwise)
+    const floatx4 x = *(volatile DEERS_LDS const floatx4*)(uintptr_t)seed_at;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // volatile: four separate reads (one read and twelve register moves otherwise)
-      const floatx4 x = *(volatile DEERS_LDS const floatx4*)(uintptr_t)seed_at;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) s[4 * j + e] = x[e];
-    }
+    for (int e = 0; e < 4; ++e) s[4 * j + e] = x[e];
   };
   // V fragment j of the block in ring slot `slot` (16-key step j / DB, output rows 32 (j % DB) ..)
   // and K fragment ks of the block in `slot`
@@ -250,15 +244,20 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
   // (already -m unless FIRST), nxt = S(b+1) to be produced (only while b is before the wave's
   // diagonal block; from there on the wave sees masked blocks).  FIRST: b == 0, cur is the raw
   // product and fixes m, and there is no block b-1; otherwise the first NPF V fragments of
-  // block b-1 are in fr.  MFMA order: PV, then S.  Ends by fetching the first V fragments of
-  // block b for the next stage.  One body serves every position of a wave: variants per
-  // position made the register allocator spill hundreds of values.
+  // block b-1 are in fr.  MFMA order: PV, then S.  A wave issues one instruction every four
+  // clocks at best and only what follows an MFMA within its 32 clocks costs nothing, so the
+  // stage's other work is spread over its eight chunks: the fetch of a fragment W MFMAs ahead
+  // (rolling into the next stage's first V fragments), the four seed reads, the loads that
+  // refill the slots of K(b) and V(b-2), and the exponentials, sums and packing of block b.
+  // One body serves every position of a wave: variants per position made the register
+  // allocator spill hundreds of values.
   auto stage = [&](auto first_c, auto slot_c, int b, floatx16& cur, floatx16& nxt) {
     constexpr bool FIRST = decltype(first_c)::value, HAS_PV = !FIRST;
     constexpr int SLOT = decltype(slot_c)::value;
     constexpr uint32_t KSLOT = (SLOT + 1) % R, VSLOT = (SLOT + R - 1) % R;
     constexpr int NPV = HAS_PV ? 2 * DB : 0, NMS = KS, NM = NPV + NMS;
     constexpr int NPRE = HAS_PV ? NPF : 0;  // fragments already in fr
+    constexpr bool ROLL = NM % W == 0;      // a fetched fragment lands in the register its MFMA names
     const bool has_s = b < bd;    // wave-uniform: the wave needs block b+1
     const bool masked = b >= bd;  // block b is the wave's diagonal block, or lies beyond it
     auto fetch = [&](int mi) -> half8 { return mi < NPV ? fetch_v(mi, VSLOT) : fetch_k(mi - NPV, KSLOT); };
@@ -269,7 +268,12 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
       m = row_max(cur);
       set_negm();
     }
-    if (has_s) seed(nxt);
+    if constexpr (FIRST) {
+      if (has_s) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) seed_part(j, nxt);
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
     uint32_t pw[8];
     float bs0, bs1;
@@ -295,8 +299,13 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
           const int ks = mi - NPV;
           if (has_s) nxt = mfma_f16(fr[mi % W], qf[ks], nxt);
         }
-        if (mi + W < NM) fr[mi % W] = fetch(mi + W);
+        if (mi + W < NM)
+          fr[mi % W] = fetch(mi + W);
+        else if (ROLL && mi + W - NM < NPF)
+          fr[mi % W] = fetch_v(mi + W - NM, SLOT);  // the next stage multiplies V(b) by P(b)
       }
+      if (!FIRST && i < 4 && has_s) seed_part(i, nxt);
+      if (i >= 1 && i <= LPI) request_part(i - 1, b + 1 + F, b + F, (SLOT + 1 + F) % R, (SLOT + F) % R);
       if constexpr (FIRST) {
         cur[2 * i] = fast_exp2(cur[2 * i] - m);
         cur[2 * i + 1] = fast_exp2(cur[2 * i + 1] - m);
@@ -307,9 +316,10 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
       if (i > 0) finish_pair(i - 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // the next stage multiplies V(b) by P(b): its first fragments leave LDS now
+    if constexpr (!ROLL) {
 #pragma unroll
-    for (int j = 0; j < NPF; ++j) fr[j] = fetch_v(j, SLOT);
+      for (int j = 0; j < NPF; ++j) fr[j] = fetch_v(j, SLOT);
+    }
     finish_pair(7);
     float bsum = bs0 + bs1;
     if constexpr (!FIRST) {
@@ -391,7 +401,6 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
     // fragments and the seed, whose slots are not refilled for another stage; every read of the
     // two slots the request refills has been consumed by an MFMA this wave issued already.
     __builtin_amdgcn_s_barrier();
-    request(b + 1 + F, b + F, (SLOT + 1 + F) % R, (SLOT + F) % R);
   };
   open_stage(std::integral_constant<int, 0>{}, 0);
   stage(yes, std::integral_constant<int, 0>{}, 0, sa, sb);
