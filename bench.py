@@ -10,9 +10,8 @@ GEMMs the kernels really execute).  The decode kernel (B=32 H=12 L=4096 D=64,
 f16) is timed in the same run and reported as achieved HBM GB/s.
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel of the step from
-per-kernel hipEvent times taken in a second pass of the same K steps (event
-pairs between kernels would perturb the headline timing, so that pass is
-separate); `cpu_baseline` is the CPU oracle (a restatement of the reference's
+a pass of its own: one hipEvent pair around K back-to-back launches of that
+kernel; `cpu_baseline` is the CPU oracle (a restatement of the reference's
 materialised CPU path) timed on this box's host cores on a bounded sample.
 """
 from __future__ import annotations
@@ -70,21 +69,31 @@ def bench_train(steps: int, warmup: int, only: str = "all"):
         if only in ("all", "bwd"):
             bwd()
 
-    # first pass: per-kernel device times over at least KERNEL_PASS_MIN_STEPS steps whatever
-    # `steps` is (`roofline` is computed from this pass), after as many untimed steps.  It
-    # runs before the timed region so that the K timed steps see the device in the state a
-    # long job keeps it in: from idle, the first few milliseconds of launches run 5-8 % slower
-    # while the clocks settle, and K = 20 steps are 2 ms in all.
+    # first pass: as many untimed steps as the per-kernel pass has launches, so that the timed
+    # passes see the device in the state a long job keeps it in: from idle, the first few
+    # milliseconds of launches run 5-8 % slower while the clocks settle, and K = 20 steps are
+    # 2 ms in all.
     ksteps = max(steps, KERNEL_PASS_MIN_STEPS)
     for _ in range(ksteps):
         step()
     rocm.sync()
-    rocm.profile_enable(True)
-    for _ in range(ksteps):
-        step()
-    prof = rocm.profile_collect()
-    rocm.profile_enable(False)
-    kernels = {n: {"calls": c, "avg_us": 1e3 * ms / c} for n, (c, ms) in prof.items()}
+    # second pass: per-kernel device time, one event pair around `ksteps` back-to-back launches
+    # of that kernel (`roofline` is computed from this pass; a kernel trace of the same command
+    # gives the same average from the dispatch records)
+    kernels = {}
+    for name, fn in (("attn_fwd_f16", fwd), ("attn_bwd_f16", bwd)):
+        if only not in ("all", name[5:8]):
+            continue
+        for _ in range(10):
+            fn()
+        rocm.sync()
+        t = rocm.Timer()
+        t.start()
+        for _ in range(ksteps):
+            fn()
+        t.stop()
+        rocm.sync()
+        kernels[name] = {"calls": ksteps, "avg_us": 1e3 * t.elapsed_ms() / ksteps}
 
     # the timed region: `warmup` untimed steps, then exactly `steps` steps between two events
     # (and two host clock reads), synchronised on both sides
@@ -110,7 +119,63 @@ def bench_train(steps: int, warmup: int, only: str = "all"):
     rocm.sync()
     per_step = sorted(1e3 * t.elapsed_ms() for t in timers)
     step_us = {"median": per_step[len(per_step) // 2], "min": per_step[0]}
-    return dict(wall_ms=wall_ms, dev_ms=dev_ms, kernels=kernels, step_us=step_us)
+    return dict(wall_ms=wall_ms, dev_ms=dev_ms, kernels=kernels, step_us=step_us,
+                warmup_effective=warmup + 2 * ksteps + 10 * len(kernels))
+
+
+PEAK_F32_TFLOPS = 157.3  # MI355X dense f32 MFMA, published
+
+
+def bench_attention_config(dtype, B, H, T, D, launches=50, sigma=1.0):
+    """Forward, backward and fwd+bwd step of one more attention geometry: each from one event
+    pair around `launches` back-to-back launches, after as many untimed ones."""
+    x = synth.attention_inputs(f"bench-{B}-{H}-{T}-{D}", B, H, T, D, dtype, base_seed=1)
+    if sigma != 1.0:
+        x = {n: (a.astype(np.float32) * sigma).astype(dtype) for n, a in x.items()}
+    q, k, v, do = (rocm.DeviceBuffer.from_numpy(x[n]) for n in ("q", "k", "v", "do"))
+    o = rocm.DeviceBuffer((B, H, T, D), dtype)
+    lse = rocm.DeviceBuffer((B, H, T), np.float32)
+    dq, dk, dv = (rocm.DeviceBuffer((B, H, T, D), dtype) for _ in range(3))
+    scale = rocm.default_scale(D)
+
+    def fwd():
+        rocm.attn_fwd_raw(dtype, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, B, H, T, D, scale)
+
+    def bwd():
+        rocm.attn_bwd_raw(dtype, q.ptr, k.ptr, v.ptr, o.ptr, lse.ptr, do.ptr, dq.ptr, dk.ptr, dv.ptr,
+                          B, H, T, D, scale)
+
+    def both():
+        fwd()
+        bwd()
+
+    us = {}
+    for name, fn in (("fwd", fwd), ("bwd", bwd), ("step", both)):
+        for _ in range(launches):
+            fn()
+        rocm.sync()
+        t = rocm.Timer()
+        t.start()
+        for _ in range(launches):
+            fn()
+        t.stop()
+        rocm.sync()
+        us[name] = 1e3 * t.elapsed_ms() / launches
+    fwd_f, bwd_f = attn_flops(B, H, T, D)
+    peak = PEAK_F16_TFLOPS if np.dtype(dtype) == np.float16 else PEAK_F32_TFLOPS
+    tf = {"fwd": fwd_f / (us["fwd"] * 1e-6) / 1e12, "bwd": bwd_f / (us["bwd"] * 1e-6) / 1e12,
+          "step": (fwd_f + bwd_f) / (us["step"] * 1e-6) / 1e12}
+    return {"workload": f"causal self-attention fwd+bwd, {np.dtype(dtype).name}, B={B} H={H} T={T} D={D}",
+            "launches_timed": launches, "us": us, "tflops": tf,
+            "frac_mfma_peak": {n: v / peak for n, v in tf.items()}, "peak_tflops": peak,
+            "flops_per_step": fwd_f + bwd_f}
+
+
+EXTRA_CONFIGS = {
+    "c1": dict(dtype=np.float32, B=4, H=6, T=256, D=32),                    # BASELINE configs[0]
+    "c3": dict(dtype=np.float16, B=1, H=16, T=8192, D=128, sigma=0.5),      # BASELINE configs[2]
+    "c2_d128": dict(dtype=np.float16, B=8, H=12, T=1024, D=128),            # configs[1] at head width 128
+}
 
 
 def bench_decode(steps: int, warmup: int, rotate: int = 4):
@@ -478,7 +543,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gpt", action="store_true",
                     help="skip the end-to-end GPT training step reported beside the headline")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "decode", "copy", "rope", "log_softmax", "adamw", "gpt", "storage"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "c1", "c3", "c2_d128", "decode", "copy", "rope", "log_softmax", "adamw", "gpt", "storage"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
@@ -506,6 +571,9 @@ def main():
             print(json.dumps({"only": "gpt", **bench_gpt(min(args.steps, 10), min(args.warmup, 3))}))
         elif args.only == "copy":
             print(json.dumps({"only": "copy", **bench_copy(args.steps, args.warmup)}))
+        elif args.only in EXTRA_CONFIGS:
+            print(json.dumps({"only": args.only,
+                              **bench_attention_config(launches=max(50, min(args.steps, 200)), **EXTRA_CONFIGS[args.only])}))
         else:
             tr = bench_train(args.steps, args.warmup, args.only)
             print(json.dumps({"only": args.only, "kernels": tr["kernels"]}))
@@ -550,15 +618,18 @@ def main():
     out = {
         "metric": "causal attn fwd+bwd TFLOP/s & %MFMA peak (T=1024,D=64,f16); decode HBM GB/s",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "warmup": args.warmup, "warmup_effective": tr["warmup_effective"], "ms_per_step": ms_per_step,
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "causal self-attention fwd+bwd, f16 in / f32 accumulate, "
                                "B=8 H=12 T=1024 D=64 (BASELINE configs[1])",
                    "flops_per_step": fwd_f + bwd_f, "flop_convention": "7*B*H*T^2*D"},
         "frac_mfma_peak": tflops / PEAK_F16_TFLOPS,
         "peak_tflops_f16_dense": PEAK_F16_TFLOPS,
-        "timed_region": "`warmup` untimed + exactly `steps` timed fwd+bwd steps, run after the per-kernel pass "
-                        "(2 x %d steps) so that short runs see settled clocks" % max(args.steps, KERNEL_PASS_MIN_STEPS),
+        "timed_region": "`warmup` untimed + exactly `steps` timed fwd+bwd steps, run after the settling pass "
+                        "(%d steps) and the per-kernel pass (%d launches of each kernel between one event pair), "
+                        "so that short runs see settled clocks: `warmup_effective` counts all of them"
+                        % (max(args.steps, KERNEL_PASS_MIN_STEPS), max(args.steps, KERNEL_PASS_MIN_STEPS)),
         "wall_ms_per_step": tr["wall_ms"] / args.steps,
         "step_us_event_pairs": tr["step_us"],
         "kernels": kern,
@@ -570,6 +641,13 @@ def main():
                    "GB/s_whole_call": dec["gbs_call"], "peak_GB/s": PEAK_HBM_GBS,
                    "frac_hbm_peak": dec["gbs_kernel"] / PEAK_HBM_GBS},
     }
+    # BASELINE configs[0] and configs[2] (and configs[1]'s shape at head width 128), reported
+    # beside the headline, never part of `value`
+    for name, cfg in EXTRA_CONFIGS.items():
+        try:
+            out[name] = bench_attention_config(**cfg)
+        except Exception as e:  # the headline line must not depend on them
+            out[name] = {"error": str(e)}
     if not args.no_gpt:
         # BASELINE configs[4], reported beside the headline (never part of `value`)
         try:

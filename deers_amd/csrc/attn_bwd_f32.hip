@@ -750,7 +750,10 @@ static bool launch_bwd_fused_f32_d(const BwdParams& p, int B, hipStream_t stream
   }
   const int n_blocks = (p.T + kBwd32Blk - 1) / kBwd32Blk;
   const Bwd32Items items = bwd32_items(p.T, (int64_t)n_blocks * B * p.H < capacity);
-  if (!items.dev) return false;
+  if (!items.dev) {
+    (void)hipGetLastError();  // the two-pass form stands in: leave no error behind for the caller's check
+    return false;
+  }
   const int64_t rows = (int64_t)B * p.H * p.T;
   constexpr int LPR = D / 4;
   const int64_t threads = rows * LPR;

@@ -266,6 +266,7 @@ static Fwd32Lists fwd32_lists(int n_qtiles, int heads_per_xcd, int T, hipStream_
       cus_per_xcd = prop.multiProcessorCount / 8;
     } else {
       slots = -1;
+      (void)hipGetLastError();  // the plain grid stands in: leave no error behind for the caller's check
     }
   }
   if (slots < 0) return Fwd32Lists{};
@@ -313,10 +314,14 @@ static Fwd32Lists fwd32_lists(int n_qtiles, int heads_per_xcd, int T, hipStream_
     std::vector<int> flat((size_t)wgs * e.max_len, -1);
     for (int w = 0; w < wgs; ++w)
       for (size_t k = 0; k < lists[w].size(); ++k) flat[(size_t)w * e.max_len + k] = lists[w][k];
-    if (hipMalloc(&e.dev, flat.size() * sizeof(int)) != hipSuccess) return Fwd32Lists{};
+    if (hipMalloc(&e.dev, flat.size() * sizeof(int)) != hipSuccess) {
+      (void)hipGetLastError();  // the plain grid stands in
+      return Fwd32Lists{};
+    }
     // the table is read by launches on `stream` only; a synchronous copy keeps `flat` alive
     if (hipMemcpy(e.dev, flat.data(), flat.size() * sizeof(int), hipMemcpyHostToDevice) != hipSuccess) {
       (void)hipFree(e.dev);
+      (void)hipGetLastError();
       return Fwd32Lists{};
     }
     (void)stream;

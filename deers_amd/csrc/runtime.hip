@@ -436,6 +436,10 @@ int deers_rocm_set_handover_mode(int mode) {
   NEED_INIT();
   if (mode != -1 && mode != DEERS_ROCM_HANDOVER_SAME_XCD && mode != DEERS_ROCM_HANDOVER_STREAM_ORDER)
     return fail(DEERS_ROCM_ERR_ARG, "set_handover_mode: mode %d is not -1, 0 or 1", mode);
+  if (mode == DEERS_ROCM_HANDOVER_SAME_XCD && !g_rt.same_xcd_handover)
+    return fail(DEERS_ROCM_ERR_ARG,
+                "set_handover_mode: this device's policy is stream order (partition or CU mask): a hand-over "
+                "through one XCD's L2 is not valid here");
   g_rt.handover_forced = mode;
   return DEERS_ROCM_OK;
 }

@@ -97,17 +97,15 @@ void* deers_rocm_stream(void);
  * (256 compute units) with no CU mask in the environment. */
 int deers_rocm_handover_policy(int cu_count, int cu_mask_set);
 /* The mode in force (after deers_rocm_init; -1 before), and an override: mode -1 returns
- * to the policy's choice for this device.  A caller that captures backward calls into a HIP
- * graph selects STREAM_ORDER first: the single launch's flag epoch is a kernel argument, so
- * a replayed launch would find its flags already set. */
+ * to the policy's choice for this device.  Asking for SAME_XCD on a device whose policy is
+ * STREAM_ORDER is refused with DEERS_ROCM_ERR_ARG (the hand-over through one L2 is not valid
+ * there).  A backward call made while the library stream is being captured into a HIP graph
+ * takes the two-launch form without flags by itself: the single launch's flag epoch is a
+ * kernel argument, so a replayed launch would find its flags already set.  Such a call must
+ * have been made once outside capture with the same geometry (workspace and flags grow
+ * there). */
 int deers_rocm_handover_mode(void);
 int deers_rocm_set_handover_mode(int mode);
-/* Test hook for the bounded wait of the single-launch backward: `spin_limit` polls (the
- * default is 2^20) and, when `skip_producers` is non-zero, backward calls launch only the
- * waiting half of the grid, so that every wait runs out, every kernel still exits, and the
- * next deers_rocm_sync returns DEERS_ROCM_ERR_HANDOVER.  (spin_limit 2^20,
- * skip_producers 0) restores normal operation. */
-int deers_rocm_debug_bwd_wait(int spin_limit, int skip_producers);
 
 /* ---- device memory (the storage backend's alloc / to-device / to_vec) ---- */
 
@@ -565,6 +563,15 @@ int deers_rocm_decode_qkv(int dtype, const void* q, const void* k, const void* v
 int deers_rocm_rope_bwd(int dtype, const void* dy, const int64_t* dy_strides,
                         const void* cos, const void* sin, void* dx,
                         int64_t B, int64_t T, int64_t H, int64_t D);
+
+/* ---- testing only: nothing a binding exposes ---- */
+
+/* Test hook for the bounded wait of the single-launch backward: `spin_limit` polls (the
+ * default is 2^20) and, when `skip_producers` is non-zero, backward calls launch only the
+ * waiting half of the grid, so that every wait runs out, every kernel still exits, and the
+ * next deers_rocm_sync returns DEERS_ROCM_ERR_HANDOVER.  (spin_limit 2^20,
+ * skip_producers 0) restores normal operation.  No counterpart in the reference. */
+int deers_rocm_debug_bwd_wait(int spin_limit, int skip_producers);
 
 #ifdef __cplusplus
 }

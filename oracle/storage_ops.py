@@ -154,3 +154,36 @@ def scatter_add(src: np.ndarray, dim: int, indices: np.ndarray, dst_shape) -> np
 def cat(parts) -> np.ndarray:
     """Compact buffers one after the other (CpuStorage::cat, src/storage/cpu.rs:47-90)."""
     return np.concatenate([np.ascontiguousarray(p).reshape(-1) for p in parts])
+
+
+def index_select_dim(x: np.ndarray, dim: int, indices) -> np.ndarray:
+    """index_select along any dimension: for every leading slab, the rows named by `indices`
+    in their order (index_select_into, src/storage/cpu.rs:936-952)."""
+    indices = np.asarray(indices, dtype=np.int64)
+    if indices.size and (indices.min() < 0 or indices.max() >= x.shape[dim]):
+        raise IndexError("index_select: index out of bounds")
+    left = int(np.prod(x.shape[:dim], dtype=np.int64))
+    right = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    s = np.ascontiguousarray(x).reshape(left, x.shape[dim], right)
+    out = np.empty((left, indices.size, right), x.dtype)
+    for l in range(left):
+        for i, r in enumerate(indices):
+            out[l, i, :] = s[l, r, :]
+    return out.reshape(x.shape[:dim] + (indices.size,) + x.shape[dim + 1:])
+
+
+def index_add_dim(src: np.ndarray, dim: int, indices, dst_shape) -> np.ndarray:
+    """index_add along any dimension into zeros of `dst_shape`: for every leading slab,
+    dst[l, indices[i], :] += src[l, i, :] for i ascending, each `+=` in the storage type
+    (index_add_into, src/storage/cpu.rs:954-975)."""
+    indices = np.asarray(indices, dtype=np.int64)
+    if indices.size and (indices.min() < 0 or indices.max() >= dst_shape[dim]):
+        raise IndexError("index_add: index out of bounds")
+    left = int(np.prod(dst_shape[:dim], dtype=np.int64))
+    right = int(np.prod(dst_shape[dim + 1:], dtype=np.int64))
+    s = np.ascontiguousarray(src).reshape(left, indices.size, right)
+    out = np.zeros((left, int(dst_shape[dim]), right), src.dtype)
+    for l in range(left):
+        for i, r in enumerate(indices):
+            out[l, r, :] = out[l, r, :] + s[l, i, :]
+    return out.reshape(tuple(dst_shape))

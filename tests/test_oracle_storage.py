@@ -235,3 +235,58 @@ def test_scatter_add_f16_order_and_rounding():
 def test_cat():
     a, b = _rand((2, 3), 1), _rand((4,), 2)
     assert np.array_equal(so.cat([a, b]), np.concatenate([a.ravel(), b]))
+
+
+def test_cat_reference_literal():
+    # tests/tensor.rs:1942-1972: two [2, 2] tensors along dim 0
+    lhs, rhs = np.array([1, 2, 3, 4], np.float32).reshape(2, 2), np.array([5, 6, 7, 8], np.float32).reshape(2, 2)
+    assert so.cat([lhs, rhs]).tolist() == [1, 2, 3, 4, 5, 6, 7, 8]
+
+
+# ---- index_select / index_add along any dimension -------------------------------------------
+
+def test_index_select_dim_reference_literals():
+    # tests/tensor.rs:2289-2321 (dim 0) and 2323-2357 (dim 2 of [2, 2, 3])
+    x = np.array([10, 11, 12, 20, 21, 22, 30, 31, 32, 40, 41, 42], np.float32).reshape(4, 3)
+    assert so.index_select_dim(x, 0, [2, 0, 3]).ravel().tolist() == [30, 31, 32, 10, 11, 12, 40, 41, 42]
+    y = np.arange(1, 13, dtype=np.float32).reshape(2, 2, 3)
+    assert so.index_select_dim(y, 2, [2, 0]).ravel().tolist() == [3, 1, 6, 4, 9, 7, 12, 10]
+
+
+@pytest.mark.parametrize("dim", [0, 1, 2])
+def test_index_select_dim_against_libraries(dim):
+    x = _rand((3, 5, 4), 31)
+    idx = np.random.default_rng(32).integers(0, x.shape[dim], 7)
+    got = so.index_select_dim(x, dim, idx)
+    assert np.array_equal(got, np.take(x, idx, axis=dim))
+    assert np.array_equal(got, torch.index_select(torch.from_numpy(x), dim, torch.from_numpy(idx)).numpy())
+    with pytest.raises(IndexError):
+        so.index_select_dim(x, dim, [x.shape[dim]])
+
+
+def test_index_add_dim_reference_literal():
+    # tests/tensor.rs:2359-2385: the gradient of a sum through index_select(0, [2, 0, 2]) of [4, 3]
+    got = so.index_add_dim(np.ones((3, 3), np.float32), 0, [2, 0, 2], (4, 3))
+    assert got.ravel().tolist() == [1, 1, 1, 0, 0, 0, 2, 2, 2, 0, 0, 0]
+
+
+@pytest.mark.parametrize("dim", [0, 1, 2])
+def test_index_add_dim_against_torch_and_the_adjoint(dim):
+    shape = (3, 5, 4)
+    idx = np.random.default_rng(41).integers(0, shape[dim], 9)  # with collisions
+    src_shape = shape[:dim] + (9,) + shape[dim + 1:]
+    src = np.random.default_rng(42).integers(-8, 9, src_shape).astype(np.float32)  # exact sums in any order
+    got = so.index_add_dim(src, dim, idx, shape)
+    want = torch.zeros(shape).index_add_(dim, torch.from_numpy(idx), torch.from_numpy(src)).numpy()
+    assert np.array_equal(got, want)
+    # index_add is the adjoint of index_select: <select(x), s> == <x, add(s)>
+    x = np.random.default_rng(43).integers(-8, 9, shape).astype(np.float32)
+    assert float((so.index_select_dim(x, dim, idx) * src).sum()) == float((x * got).sum())
+
+
+def test_index_add_dim_f16_order():
+    # ascending positions: (2048 + 1) + 1 == 2048 in f16, (1 + 1) + 2048 == 2050
+    src = np.array([[2048.0, 1.0, 1.0]], np.float16).reshape(1, 3, 1)
+    assert so.index_add_dim(src, 1, [0, 0, 0], (1, 2, 1)).ravel().tolist() == [2048.0, 0.0]
+    src = np.array([[1.0, 1.0, 2048.0]], np.float16).reshape(1, 3, 1)
+    assert so.index_add_dim(src, 1, [0, 0, 0], (1, 2, 1)).ravel().tolist() == [2050.0, 0.0]

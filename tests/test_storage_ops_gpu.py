@@ -1,5 +1,6 @@
 """The generic storage kernels (deers_rocm_unary / _binary / _reduce / _log_sum_exp / _gather /
-_scatter_add) against oracle/storage_ops.py, the numpy restatement of src/storage/cpu.rs.
+_scatter_add) and the documented compositions (cat, index_select / index_add along an inner
+dimension) against oracle/storage_ops.py, the numpy restatement of src/storage/cpu.rs.
 
 Bar: bit-exact for everything that is exact arithmetic, a copy or an index operation (neg, relu,
 relu_backward, the scalar ops, add/sub/mul/div/eq, max, short sums, gather, scatter_add); for the
@@ -353,6 +354,87 @@ def test_argument_errors():
     sh0 = (ctypes.c_int64 * 2)(0, 4)
     assert lib.deers_rocm_unary(1, 0, None, 2, sh0, None, ctypes.c_double(0), None) == 0
     rocm.sync()
+
+
+# ---- the compositions: cat, index_select / index_add along an inner dimension -----------------
+# BackendStorage::index_select / index_add with dim > 0 are one deers_rocm_index_select /
+# _index_add call per leading slab (left_len of src/storage/cpu.rs:936-975) with width =
+# right_len; Storage::cat (src/storage.rs:568-607) is one deers_rocm_dtod per part.
+
+def _index_select_dim(x, dim, idx):
+    import ctypes
+    left = int(np.prod(x.shape[:dim], dtype=np.int64))
+    n, right = x.shape[dim], int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    dx, di = _dev(np.ascontiguousarray(x)), _dev(np.asarray(idx, np.int64))
+    out = rocm.DeviceBuffer(x.shape[:dim] + (len(idx),) + x.shape[dim + 1:], x.dtype)
+    for l in range(left):
+        rocm.index_select_raw(x.dtype, _ptr(dx, l * n * right, x.itemsize), di.ptr,
+                              _ptr(out, l * len(idx) * right, x.itemsize), n, len(idx), right)
+    return out.numpy()
+
+
+def _index_add_dim(src, dim, idx, dst_shape):
+    left = int(np.prod(dst_shape[:dim], dtype=np.int64))
+    n, right = dst_shape[dim], int(np.prod(dst_shape[dim + 1:], dtype=np.int64))
+    ds, di = _dev(np.ascontiguousarray(src)), _dev(np.asarray(idx, np.int64))
+    out = rocm.DeviceBuffer(dst_shape, src.dtype, zeros=True)
+    for l in range(left):
+        rocm.index_add_raw(src.dtype, _ptr(ds, l * len(idx) * right, src.itemsize), di.ptr,
+                           _ptr(out, l * n * right, src.itemsize), n, len(idx), right)
+    return out.numpy()
+
+
+def _cat(parts):
+    import ctypes
+    total = sum(p.size for p in parts)
+    out = rocm.DeviceBuffer((total,), parts[0].dtype)
+    at = 0
+    for p in parts:
+        if p.size == 0:
+            continue
+        d = _dev(np.ascontiguousarray(p))
+        rocm._check(rocm.load().deers_rocm_dtod(_ptr(out, at, p.itemsize), d.ptr, ctypes.c_size_t(p.nbytes)))
+        at += p.size
+    return out.numpy()
+
+
+@pytest.mark.gpu
+def test_index_select_and_index_add_reference_literals():
+    # tests/tensor.rs:2289-2385
+    x = np.array([10, 11, 12, 20, 21, 22, 30, 31, 32, 40, 41, 42], np.float32).reshape(4, 3)
+    assert _index_select_dim(x, 0, [2, 0, 3]).ravel().tolist() == [30, 31, 32, 10, 11, 12, 40, 41, 42]
+    y = np.arange(1, 13, dtype=np.float32).reshape(2, 2, 3)
+    assert _index_select_dim(y, 2, [2, 0]).ravel().tolist() == [3, 1, 6, 4, 9, 7, 12, 10]
+    grad = _index_add_dim(np.ones((3, 3), np.float32), 0, [2, 0, 2], (4, 3))
+    assert grad.ravel().tolist() == [1, 1, 1, 0, 0, 0, 2, 2, 2, 0, 0, 0]
+    rocm.sync()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("shape,dim,n_idx", [((3, 5, 4), 1, 7), ((3, 5, 4), 2, 9), ((2, 3, 6, 8), 2, 4),
+                                             ((4, 7, 1), 1, 3), ((1, 300, 33), 1, 1000)])
+def test_index_select_and_index_add_along_an_inner_dimension(dtype, shape, dim, n_idx):
+    rng = np.random.default_rng(100 + dim + n_idx)
+    x = _rand(shape, 50 + n_idx, dtype)
+    idx = rng.integers(0, shape[dim], n_idx)
+    _same(_index_select_dim(x, dim, idx), so.index_select_dim(x, dim, idx), exact=True)
+    src = _rand(shape[:dim] + (n_idx,) + shape[dim + 1:], 60 + n_idx, dtype)
+    # collisions: the sums follow the reference's order, so f16 agrees bit for bit too
+    _same(_index_add_dim(src, dim, idx, shape), so.index_add_dim(src, dim, idx, shape), exact=True)
+    rocm.sync()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int64])
+def test_cat(dtype):
+    # tests/tensor.rs:1942-1972, then ragged parts (one of them a single element, one empty)
+    lhs, rhs = np.array([1, 2, 3, 4]).astype(dtype).reshape(2, 2), np.array([5, 6, 7, 8]).astype(dtype).reshape(2, 2)
+    assert _cat([lhs, rhs]).tolist() == [1, 2, 3, 4, 5, 6, 7, 8]
+    parts = [(np.random.default_rng(70 + i).standard_normal(s) * 4).astype(dtype)
+             for i, s in enumerate([(3, 5), (1,), (0,), (7, 2, 3), (1001,)])]
+    got = _cat(parts)
+    assert got.dtype == np.dtype(dtype) and np.array_equal(got, so.cat(parts))
 
 
 @pytest.mark.gpu
