@@ -11,6 +11,14 @@
 //   D  the forward's wave-iteration (S = K Q^T on 64 keys, online softmax on the results,
 //      O += V^T P) with its memory features switched on one at a time: LDS fragment reads,
 //      the per-iteration barrier, asynchronous global->LDS tile loads; 1, 2, 3 waves per SIMD
+//   E  phase alternation: every wave alternates a matrix phase (16 MFMAs) and a vector phase
+//      (the softmax ops of 32 scores); free running, two wave groups held in opposite phases by
+//      barriers ("ping-pong"), and both groups in the same phase
+//   F  the block-pipelined forward's own loop, compiled in its bench mode
+//   G  one stream of chunks, each one MFMA followed by a given handful of other instructions
+//      (what fits in the 32 clocks of an MFMA, and what each further instruction costs)
+//   H  one or two MFMAs per 1 KiB operand fragment read from LDS, with and without the
+//      softmax's vector ops, and the rate of MFMAs chained through one accumulator
 //
 // Every launch covers all CUs (256 workgroups x waves); times are clock64() deltas from the
 // common start of a CU's waves to the end of its slowest wave, averaged over the CUs, so
@@ -420,6 +428,198 @@ static void run_fwd_bp(int wgs) {
   CK(hipFree(q)); CK(hipFree(k)); CK(hipFree(v)); CK(hipFree(o)); CK(hipFree(lse)); CK(hipFree(clk));
 }
 
+// ---- E: phase alternation ---------------------------------------------------------------------
+// MODE 0: free running; 1: a barrier between the phases, the two wave groups of a workgroup in
+// opposite phases; 2: barriers, all waves in the same phase.  VSET 0: the tile-pipelined
+// loops' vector mix per 32 scores (32 fma, 32 exp, 16 cvt_pk, 16 dot2c, 16 max3, 8 fma); 1:
+// without the fma before each exponential and the maxima.
+template <int MODE, int VSET>
+__global__ __launch_bounds__(1024) void phase_kernel(float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) { a[i] = (half_t)(0.001f * (lane + i)); b[i] = (half_t)(0.002f * (lane - i)); }
+  floatx16 acc0 = ZERO16, acc1 = ZERO16, acc2 = ZERO16, acc3 = ZERO16;
+  float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3, v4 = lane + 4, v5 = lane + 5, v6 = lane + 6, v7 = lane + 7;
+  float c1 = 0.999f, c2 = 0.001f, s0 = 0, s1 = 0, mx0 = 0, mx1 = 0;
+  unsigned h0, h1; const unsigned ones = 0x3c003c00u;
+  const int group = (wave >> 2) & 1;
+  __syncthreads();
+  const long long t0 = clock64();
+  auto phase_m = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { MF(acc0); MF(acc1); MF(acc2); MF(acc3); }
+  };
+  auto phase_v = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {  // 4 scores per round
+      if (VSET == 0) { FM(v0); FM(v1); FM(v2); FM(v3); }
+      EX(v0); EX(v1); EX(v2); EX(v3);
+      CVT(h0, v0, v1); CVT(h1, v2, v3);
+      DOT(s0, h0); DOT(s1, h1);
+      if (VSET == 0) { MX(mx0, v4); MX(mx1, v6); }
+      FM(v4);
+    }
+  };
+  for (int it = 0; it < iters; ++it) {
+    if (MODE == 0) { phase_m(); phase_v(); }
+    if (MODE == 1) {
+      if (group == 0) { phase_m(); __builtin_amdgcn_s_barrier(); phase_v(); __builtin_amdgcn_s_barrier(); }
+      else { phase_v(); __builtin_amdgcn_s_barrier(); phase_m(); __builtin_amdgcn_s_barrier(); }
+    }
+    if (MODE == 2) { phase_m(); __builtin_amdgcn_s_barrier(); phase_v(); __builtin_amdgcn_s_barrier(); }
+  }
+  const long long t1 = clock64();
+  float s = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7 + s0 + s1 + mx0 + mx1;
+  for (int i = 0; i < 16; ++i) s += acc0[i] + acc1[i] + acc2[i] + acc3[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+template <int MODE, int VSET>
+static void run_phase(const char* mode_name) {
+  const int iters = 3000;
+  for (int waves = 4; waves <= 16; waves += 4) {
+    if (MODE != 0 && (waves == 4 || waves == 12)) continue;  // two equal groups
+    phase_kernel<MODE, VSET><<<256, 64 * waves>>>(g_out, g_clk, 50);
+    phase_kernel<MODE, VSET><<<256, 64 * waves>>>(g_out, g_clk, iters);
+    CK(hipDeviceSynchronize());
+    const double per_wave_iter = slowest_wave_clocks(256, 0, waves) / iters;
+    printf("E %-15s vector mix %d, %d wave(s)/SIMD: %5.0f clocks of SIMD time per wave-iteration (its 16 MFMAs alone: 512)\n",
+           mode_name, VSET, waves / 4, per_wave_iter / (waves / 4));
+  }
+}
+
+// ---- G: chunks of one MFMA and a handful of other instructions ------------------------------------
+#define ADDF(v, w) asm volatile("v_add_f32 %0, %0, %1" : "+v"(v) : "v"(w))
+#define MULF(v, w) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(v) : "v"(w))
+template <int ID>
+__global__ __launch_bounds__(1024) void chunk_kernel(float* out, long long* clk, int iters) {
+  __shared__ __attribute__((aligned(16))) char lds[16384];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) { a[i] = (half_t)(0.001f * (lane + i)); b[i] = (half_t)(0.002f * (lane - i)); }
+  floatx16 acc0 = ZERO16, acc1 = ZERO16, acc2 = ZERO16, acc3 = ZERO16;
+  float v0 = lane, v1 = lane + 1, v2 = lane + 2, v3 = lane + 3, v4 = lane + 4, v5 = lane + 5, v6 = lane + 6, v7 = lane + 7;
+  float c1 = 0.999f, c2 = 0.001f, s0 = 0, s1 = 0;
+  unsigned h0 = 0, h1 = 0; const unsigned ones = 0x3c003c00u;
+  for (int i = threadIdx.x; i < 4096; i += blockDim.x) ((float*)lds)[i] = 0.f;
+  const uint32_t la = lds_address(lds) + lane * 16;
+  half8 fr0 = a, fr1 = a;
+  __syncthreads();
+  const long long t0 = clock64();
+#define OPS(x, y, hh, ss, fr)                                                                   \
+  do {                                                                                          \
+    if (ID == 0) { EX(x); EX(y); CVT(hh, x, y); }                                               \
+    if (ID == 1) { EX(x); EX(y); CVT(hh, x, y); ADDF(ss, x); }                                  \
+    if (ID == 2) { EX(x); EX(y); CVT(hh, x, y); ADDF(ss, x); ADDF(ss, y); }                     \
+    if (ID == 3) { EX(x); EX(y); CVT(hh, x, y); DOT(ss, hh); }                                  \
+    if (ID == 4) { EX(x); EX(y); CVT(hh, x, y); FM(v4); FM(v5); FM(v6); FM(v7); }               \
+    if (ID == 5) { EX(x); MULF(v4, x); CVT(hh, x, v4); }                                        \
+    if (ID == 6) { EX(x); EX(y); CVT(hh, x, y); ADDF(ss, x); ADDF(ss, y); fr = lds_read_half8_at(la); } \
+    if (ID == 7) { EX(x); EX(y); CVT(hh, x, y); ADDF(ss, x); ADDF(ss, y);                       \
+                   const half4 lo = lds_read_tr16_at(la), hi = lds_read_tr16_at(la + 2048);     \
+                   fr = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }              \
+    if (ID == 8) { EX(x); MULF(v4, x); CVT(hh, x, v4); fr = lds_read_half8_at(la); }            \
+  } while (0)
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc0) : "v"(fr0), "v"(b)); OPS(v0, v1, h0, s0, fr0);
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc1) : "v"(fr1), "v"(b)); OPS(v2, v3, h1, s1, fr1);
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc2) : "v"(fr0), "v"(b)); OPS(v0, v1, h0, s0, fr0);
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc3) : "v"(fr1), "v"(b)); OPS(v2, v3, h1, s1, fr1);
+    }
+  }
+#undef OPS
+  const long long t1 = clock64();
+  float s = v0 + v1 + v2 + v3 + v4 + v5 + v6 + v7 + s0 + s1 + (float)h0 + (float)h1;
+  for (int i = 0; i < 16; ++i) s += acc0[i] + acc1[i] + acc2[i] + acc3[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+template <int ID>
+static void run_chunk(const char* name) {
+  const int iters = 3000;
+  printf("G MFMA + %-44s", name);
+  for (int waves = 4; waves <= 12; waves += 4) {
+    chunk_kernel<ID><<<256, 64 * waves>>>(g_out, g_clk, 50);
+    chunk_kernel<ID><<<256, 64 * waves>>>(g_out, g_clk, iters);
+    CK(hipDeviceSynchronize());
+    printf("  %d wave(s)/SIMD: %5.1f", waves / 4, slowest_wave_clocks(256, 0, waves) / (iters * 16.0) / (waves / 4));
+  }
+  printf("  clocks of SIMD time per chunk\n");
+}
+
+// ---- H: MFMAs per LDS fragment, and MFMAs chained through one accumulator -----------------------
+// MPR: MFMAs per 1 KiB fragment read (1 or 2); VALU: the softmax ops of two scores per MFMA
+template <int MPR, bool VALU>
+__global__ __launch_bounds__(1024) void reuse_kernel(float* out, long long* clk, int iters) {
+  __shared__ __attribute__((aligned(16))) char lds[65536];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 16384; i += blockDim.x) ((float*)lds)[i] = 1e-4f * (i & 1023);
+  const uint32_t la = lds_address(lds) + (wave & 3) * 8192 + lane * 16;
+  half8 fr[4], b0, b1;
+  for (int i = 0; i < 8; ++i) { b0[i] = (half_t)(0.002f * (lane - i)); b1[i] = (half_t)(0.001f * (lane + i)); }
+  for (int i = 0; i < 4; ++i) fr[i] = b0;
+  floatx16 acc0 = ZERO16, acc1 = ZERO16;
+  float v0 = lane, v1 = lane + 1, s0 = 0;
+  unsigned h0 = 0;
+  __syncthreads();
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      acc0 = mfma_f16(fr[c & 3], b0, acc0);
+      if (VALU) { EX(v0); EX(v1); CVT(h0, v0, v1); ADDF(s0, v0); ADDF(s0, v1); }
+      if (MPR == 2) {
+        acc1 = mfma_f16(fr[c & 3], b1, acc1);
+        if (VALU) { EX(v0); EX(v1); CVT(h0, v0, v1); ADDF(s0, v0); ADDF(s0, v1); }
+      }
+      fr[c & 3] = lds_read_half8_at(opaque(la) + (c & 3) * 1024 + (c >> 2) * 4096);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  const long long t1 = clock64();
+  float r = v0 + v1 + s0 + (float)h0;
+  for (int i = 0; i < 8; ++i) r += (float)fr[0][i] + (float)fr[1][i] + (float)fr[2][i] + (float)fr[3][i];
+  for (int i = 0; i < 16; ++i) r += acc0[i] + acc1[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (lane == 0) clk[blockIdx.x * 16 + wave] = t1 - t0;
+}
+template <int MPR, bool VALU>
+static void run_reuse() {
+  const int iters = 2000;
+  for (int waves = 4; waves <= 12; waves += 4) {
+    reuse_kernel<MPR, VALU><<<256, 64 * waves>>>(g_out, g_clk, 50);
+    reuse_kernel<MPR, VALU><<<256, 64 * waves>>>(g_out, g_clk, iters);
+    CK(hipDeviceSynchronize());
+    printf("H %d MFMA(s) per LDS fragment, softmax ops %s, %d wave(s)/SIMD: %5.1f clocks of SIMD time per MFMA\n", MPR,
+           VALU ? "on " : "off", waves / 4, slowest_wave_clocks(256, 0, waves) / ((double)iters * 8 * MPR * (waves / 4)));
+  }
+}
+template <int DIST>
+__global__ __launch_bounds__(256) void chain_kernel(float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63;
+  half8 a, b;
+  for (int i = 0; i < 8; ++i) { a[i] = (half_t)(0.002f * (lane - i)); b[i] = (half_t)(0.001f * (lane + i)); }
+  floatx16 acc[4] = {ZERO16, ZERO16, ZERO16, ZERO16};
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc[c % DIST] = mfma_f16(a, b, acc[c % DIST]);
+  }
+  const long long t1 = clock64();
+  float r = 0;
+  for (int j = 0; j < 4; ++j) for (int i = 0; i < 16; ++i) r += acc[j][i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (lane == 0) clk[blockIdx.x * 16 + (threadIdx.x >> 6)] = t1 - t0;
+}
+template <int DIST>
+static void run_chain() {
+  chain_kernel<DIST><<<256, 256>>>(g_out, g_clk, 2000);
+  CK(hipDeviceSynchronize());
+  printf("H MFMAs through %d accumulator(s) in turn: %5.1f clocks per MFMA\n", DIST, slowest_wave_clocks(256, 0, 4) / (2000.0 * 16));
+}
+
 int main() {
   CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
   CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
@@ -451,5 +651,22 @@ int main() {
   run_fwd_iteration<true, false, false>(Kg, Vg);
   run_fwd_iteration<true, true, false>(Kg, Vg);
   run_fwd_iteration<true, true, true>(Kg, Vg);
+  run_phase<0, 0>("free running");
+  run_phase<1, 0>("opposite phases");
+  run_phase<2, 0>("same phase");
+  run_phase<0, 1>("free running");
+  run_phase<1, 1>("opposite phases");
+  run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3);
+  run_chunk<0>("2 exp, cvt_pk");
+  run_chunk<1>("2 exp, cvt_pk, add");
+  run_chunk<2>("2 exp, cvt_pk, 2 add");
+  run_chunk<3>("2 exp, cvt_pk, dot2c");
+  run_chunk<4>("2 exp, cvt_pk, 4 fma");
+  run_chunk<5>("exp, mul, cvt_pk");
+  run_chunk<6>("2 exp, cvt_pk, 2 add, ds_read_b128");
+  run_chunk<7>("2 exp, cvt_pk, 2 add, 2 ds_read_b64_tr_b16");
+  run_chunk<8>("exp, mul, cvt_pk, ds_read_b128");
+  run_reuse<1, false>(); run_reuse<2, false>(); run_reuse<1, true>(); run_reuse<2, true>();
+  run_chain<1>(); run_chain<2>(); run_chain<4>();
   return 0;
 }

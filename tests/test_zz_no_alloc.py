@@ -51,7 +51,7 @@ def test_noalloc_decode_matches_decode_on_two_calls_in_a_row():
         assert err <= TOL_F16, f"{name}: max abs err {err:.3e}"
 
 
-def test_noalloc_decode_unsplit_heads_and_oversize_rejection():
+def test_noalloc_decode_unsplit_heads_and_bad_arguments():
     from deers_amd import rocm, synth
     rocm.init(0)
     # enough heads that none is split: the scratch array is not touched at all
