@@ -57,8 +57,9 @@ struct TileOrder {
 // global -> LDS asynchronously into rings, F stages ahead, one barrier per stage; a block has
 // landed one barrier before its first use, so the first V fragments of a stage leave LDS at the
 // end of the stage before it, across the barrier, and the K fragments (needed in the stage's
-// second half) right after it.  Waves skip blocks beyond their rows' diagonal but meet at every
-// barrier and keep issuing their share of the loads.
+// second half) right after it.  Every wave runs every stage of its workgroup, S products
+// included: a branch around a single MFMA costs a lone wave more than the MFMA (eight such
+// branches per stage were 23 % of the stage).
 // Hook for a timestamp-tracing build of this kernel; expands to nothing in the library.
 #ifndef DEERS_TRACE_POINT
 #define DEERS_TRACE_POINT(slot)
@@ -258,7 +259,6 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
     constexpr int NPV = HAS_PV ? 2 * DB : 0, NMS = KS, NM = NPV + NMS;
     constexpr int NPRE = HAS_PV ? NPF : 0;  // fragments already in fr
     constexpr bool ROLL = NM % W == 0;      // a fetched fragment lands in the register its MFMA names
-    const bool has_s = b < bd;    // wave-uniform: the wave needs block b+1
     const bool masked = b >= bd;  // block b is the wave's diagonal block, or lies beyond it
     auto fetch = [&](int mi) -> half8 { return mi < NPV ? fetch_v(mi, VSLOT) : fetch_k(mi - NPV, KSLOT); };
 #pragma unroll
@@ -269,10 +269,8 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
       set_negm();
     }
     if constexpr (FIRST) {
-      if (has_s) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) seed_part(j, nxt);
-      }
+      for (int j = 0; j < 4; ++j) seed_part(j, nxt);
     }
     __builtin_amdgcn_sched_barrier(0);
     uint32_t pw[8];
@@ -297,14 +295,14 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
           oacc[db] = mfma_f16(fr[mi % W], pf[ms], oacc[db]);
         } else {
           const int ks = mi - NPV;
-          if (has_s) nxt = mfma_f16(fr[mi % W], qf[ks], nxt);
+          nxt = mfma_f16(fr[mi % W], qf[ks], nxt);
         }
         if (mi + W < NM)
           fr[mi % W] = fetch(mi + W);
         else if (ROLL && mi + W - NM < NPF)
           fr[mi % W] = fetch_v(mi + W - NM, SLOT);  // the next stage multiplies V(b) by P(b)
       }
-      if (!FIRST && i < 4 && has_s) seed_part(i, nxt);
+      if (!FIRST && i < 4) seed_part(i, nxt);
       if (i >= 1 && i <= LPI) request_part(i - 1, b + 1 + F, b + F, (SLOT + 1 + F) % R, (SLOT + F) % R);
       if constexpr (FIRST) {
         cur[2 * i] = fast_exp2(cur[2 * i] - m);
@@ -361,10 +359,8 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
       lsum *= alpha;
 #pragma unroll
       for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-      if (has_s) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) nxt[r] += shift;
-      }
+      for (int r = 0; r < 16; ++r) nxt[r] += shift;
       set_negm();
       bsum = 0.f;
 #pragma unroll
