@@ -100,6 +100,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   const int blk0 = kv0 / kBwdBpBlk;                       // first query block (the diagonal of wave 0)
   const int last_blk = (T - 1) / kBwdBpBlk;               // holds row T-1: its rows are clamped
   const int n_blk = last_blk - blk0 + 1;                  // query blocks blk0 .. last_blk
+  const unsigned edge_span = (unsigned)max(n_blk - wave - 1, 0);  // stages wave+1 .. n_blk-1 need no mask
   const uint32_t lds0 = lds_address(smem);
   const int sqt = (int)p.sq.t, sdot = (int)p.sdo.t;
 
@@ -318,7 +319,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     // against this lane's key.  Only the wave's first blocks have masked entries.
     // Blocks past the end (the closing stages only consume) are cleared entirely: their slots
     // hold the last block a second time.
-    if (n <= wave || n >= n_blk) {
+    if ((unsigned)(n - wave - 1) >= edge_span) {  // n <= wave or n >= n_blk, one compare
       const int dist = n >= n_blk ? 64 : kvrow - 32 * (blk0 + n) - 4 * g;  // rows below dist are masked
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
