@@ -337,14 +337,17 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(pf[i]), "+v"(dsf[i]));
   };
 
-  // ---- S, dP of block 0 ----
+  // Waves 2 and 3 have nothing in blocks 0 and 1 (every query of those lies before their keys):
+  // they start their pipeline at block 2 and only keep the loads and barriers of stages 0 and 1.
+  const int n0 = wave & 2;
+  // ---- S, dP of block n0 (blocks 0 .. F are in LDS) ----
   floatx16 sa, dpa, sb, dpb;
 #pragma unroll
-  for (int part = 0; part < 8; ++part) seed_part(part, sa, dpa, 0);
+  for (int part = 0; part < 8; ++part) seed_part(part, sa, dpa, n0);
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    sa = mfma_f16(fetch1(2 * ks, 0), kf[ks], sa);
-    dpa = mfma_f16(fetch1(2 * ks + 1, 0), vf[ks], dpa);
+    sa = mfma_f16(fetch1(2 * ks, n0), kf[ks], sa);
+    dpa = mfma_f16(fetch1(2 * ks + 1, n0), vf[ks], dpa);
   }
   // ---- stage n: barrier n retires the reads of block n-2, whose slot request(n) refills with
   // block n+1+F, and makes block n+1 (requested F stages ago) visible ----
@@ -357,8 +360,12 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
   DEERS_TRACE_POINT(2);
+  for (int i = 0; i < n0; ++i) {  // stages without work: their loads and barrier
+    open_stage();
+    request(i + 1 + F, (uint32_t)(i + 1 + F) % R);
+  }
   open_stage();
-  stage(yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
+  stage(yes, (uint32_t)(n0 + R - 1) % R, (uint32_t)n0, (uint32_t)n0 + 1, n0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
     const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
@@ -373,7 +380,8 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   // a value.  (Leaving the unrolled loop from its middle instead made the register allocator
   // copy whole accumulators at every exit: 168 spilled values.)
   const int n_total = (n_blk + 1) & ~1;
-  int n = 1;
+  int n = n0 + 1;
+  for (; n % R != 1 && n <= n_total; n += 2) two_stages((uint32_t)n % R, n);  // up to the ring's start
   for (; n + R - 1 <= n_total; n += R) {
     two_stages(1, n);
     two_stages(3, n + 2);
@@ -638,13 +646,20 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   // a value.  (Leaving the unrolled loop from its middle instead made the register allocator
   // copy whole accumulators at every exit: 168 spilled values.)
   const int n_total = (n_blk + 1) & ~1;
+  // A wave's last block is its diagonal block bd, consumed in stage bd + 1: the pairs after that
+  // stage have nothing for it but the barriers (the loads of those stages are never consumed).
+  const int n_live = min(n_total, (bd + 2) & ~1);
   int n = 1;
-  for (; n + R - 1 <= n_total; n += R) {
+  for (; n + R - 1 <= n_live; n += R) {
     two_stages(1, n);
     two_stages(3, n + 2);
     two_stages(5, n + 4);
   }
-  for (; n <= n_total; n += 2) two_stages((uint32_t)n % R, n);
+  for (; n <= n_live; n += 2) two_stages((uint32_t)n % R, n);
+  for (; n <= n_total; n += 2) {
+    open_stage();
+    open_stage();
+  }
   DEERS_TRACE_POINT(4);
 
   if (qrow < T) {
