@@ -254,14 +254,15 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   // fetch of a fragment W MFMAs ahead (rolling into the next stage's consumers, which read
   // block n), by one of the eight seed reads, by one of the loads that refill the slot of
   // block n-2 with block n+1+F, and by the exponential, product and packing of block n.
-  auto stage = [&](auto first_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s, floatx16& dp,
-                   floatx16& sn, floatx16& dpn) {
+  auto stage = [&](auto first_c, auto produce_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s,
+                   floatx16& dp, floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
-    constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + NM1;
+    constexpr bool PRODUCE = decltype(produce_c)::value;  // false: block n+1 lies past the end
+    constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + (PRODUCE ? NM1 : 0);
     constexpr int NPRE = NM2 < W ? NM2 : W;  // fragments a stage finds fetched
     // whether the fetches can roll on into the next stage (a fragment must land in the register
     // its MFMA names, which is the one just freed only if the counts are multiples of W)
-    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0;
+    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0 && NMS % W == 0;
     const uint32_t RSLOT = (SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
     if constexpr (FIRST) {
@@ -302,7 +303,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
         else if (ROLL && mi + W - NMS < NPRE)
           fr[mi % W] = fetch2(mi + W - NMS, SLOT);
       }
-      if (!FIRST && i < 8) seed_part(i, sn, dpn, NSLOT);
+      if (!FIRST && PRODUCE && i < 8) seed_part(i, sn, dpn, NSLOT);
       if (i >= 1 && i <= LPI) request_part(i - 1, n + 1 + F, RSLOT);
       s[i] = fast_exp2(s[i]);
       if (i > 0) dp[i - 1] = s[i - 1] * dp[i - 1];
@@ -365,14 +366,21 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     request(i + 1 + F, (uint32_t)(i + 1 + F) % R);
   }
   open_stage();
-  stage(yes, (uint32_t)(n0 + R - 1) % R, (uint32_t)n0, (uint32_t)n0 + 1, n0, sa, dpa, sb, dpb);
+  stage(yes, yes, (uint32_t)(n0 + R - 1) % R, (uint32_t)n0, (uint32_t)n0 + 1, n0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
     const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
     open_stage();
-    stage(no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    stage(no, yes, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
     open_stage();
-    stage(no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
+    stage(no, yes, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
+  };
+  auto last_two_stages = [&](uint32_t slot, int n) {  // the same without the products of blocks n+1, n+2
+    const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
+    open_stage();
+    stage(no, no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    open_stage();
+    stage(no, no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
   // Stages 1 .. n_blk, rounded up to an even count (the closing stages only consume: their own
   // blocks lie past the end and are cleared).  Whole turns of the ring run with every LDS
@@ -380,14 +388,16 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   // a value.  (Leaving the unrolled loop from its middle instead made the register allocator
   // copy whole accumulators at every exit: 168 spilled values.)
   const int n_total = (n_blk + 1) & ~1;
+  // The last pair produces nothing: the blocks after it lie past the end.
   int n = n0 + 1;
-  for (; n % R != 1 && n <= n_total; n += 2) two_stages((uint32_t)n % R, n);  // up to the ring's start
-  for (; n + R - 1 <= n_total; n += R) {
+  for (; n % R != 1 && n + 2 <= n_total; n += 2) two_stages((uint32_t)n % R, n);  // up to the ring's start
+  for (; n + R + 1 <= n_total; n += R) {
     two_stages(1, n);
     two_stages(3, n + 2);
     two_stages(5, n + 4);
   }
-  for (; n <= n_total; n += 2) two_stages((uint32_t)n % R, n);
+  for (; n + 2 <= n_total; n += 2) two_stages((uint32_t)n % R, n);
+  if (n <= n_total) last_two_stages((uint32_t)n % R, n);
   DEERS_TRACE_POINT(4);
 
   if (kvrow < T) {
@@ -553,12 +563,13 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   // One stage, spread over 16 chunks as in the dK/dV role: the consumers of block n-1 (dQ), the
   // producers of block n+1 (S^T, dP^T), the rolling fragment fetches, the loads that refill the
   // slot of block n-2, and the vector ops of block n.
-  auto stage = [&](auto first_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s, floatx16& dp,
-                   floatx16& sn, floatx16& dpn) {
+  auto stage = [&](auto first_c, auto produce_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s,
+                   floatx16& dp, floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
-    constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + NM1;
+    constexpr bool PRODUCE = decltype(produce_c)::value;  // false: block n+1 lies past the wave's diagonal
+    constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + (PRODUCE ? NM1 : 0);
     constexpr int NPRE = NM2 < W ? NM2 : W;
-    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0;
+    constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0 && NMS % W == 0;
     const uint32_t RSLOT = (SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
 #pragma unroll
@@ -631,14 +642,21 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   constexpr std::false_type no{};
   DEERS_TRACE_POINT(2);
   open_stage();
-  stage(yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
+  stage(yes, yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
     const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
     open_stage();
-    stage(no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    stage(no, yes, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
     open_stage();
-    stage(no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
+    stage(no, yes, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
+  };
+  auto last_two_stages = [&](uint32_t slot, int n) {  // the same without the products of blocks n+1, n+2
+    const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
+    open_stage();
+    stage(no, no, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    open_stage();
+    stage(no, no, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
   // Stages 1 .. n_blk, rounded up to an even count (the closing stages only consume: their own
   // blocks lie past the end and are cleared).  Whole turns of the ring run with every LDS
@@ -649,13 +667,18 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   // A wave's last block is its diagonal block bd, consumed in stage bd + 1: the pairs after that
   // stage have nothing for it but the barriers (the loads of those stages are never consumed).
   const int n_live = min(n_total, (bd + 2) & ~1);
+  // Its last live pair produces nothing: the blocks after it lie past its diagonal.
   int n = 1;
-  for (; n + R - 1 <= n_live; n += R) {
+  for (; n + R + 1 <= n_live; n += R) {
     two_stages(1, n);
     two_stages(3, n + 2);
     two_stages(5, n + 4);
   }
-  for (; n <= n_live; n += 2) two_stages((uint32_t)n % R, n);
+  for (; n + 2 <= n_live; n += 2) two_stages((uint32_t)n % R, n);
+  if (n <= n_live) {
+    last_two_stages((uint32_t)n % R, n);
+    n += 2;
+  }
   for (; n <= n_total; n += 2) {
     open_stage();
     open_stage();
