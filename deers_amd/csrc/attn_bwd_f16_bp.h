@@ -284,7 +284,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
 #pragma unroll
-      for (int mi = i * NMS / 16; mi < (i + 1) * NMS / 16; ++mi) {
+      for (int mi = (i * NMS + 15) / 16; mi < ((i + 1) * NMS + 15) / 16; ++mi) {  // an MFMA leads every run of chunks
         if (mi < N2) {
           const int st = mi / (2 * DB), db = (mi >> 1) % DB;
           if (mi & 1)
@@ -583,7 +583,7 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
 #pragma unroll
-      for (int mi = i * NMS / 16; mi < (i + 1) * NMS / 16; ++mi) {
+      for (int mi = (i * NMS + 15) / 16; mi < ((i + 1) * NMS + 15) / 16; ++mi) {  // an MFMA leads every run of chunks
         if (mi < N2) {
           const int st = mi / DB, db = mi % DB;
           dqacc[db] = mfma_f16(fr[mi % W], dsf[st], dqacc[db]);
