@@ -5,9 +5,9 @@
 // materialises the [T,T] score tensor.
 //
 // Two kernels share this decomposition: the tile-pipelined one described below (two
-// workgroups per CU; head width 128 and small launches) and, for D <= 64 launches with
-// more than two tiles per CU, the block-pipelined one of attn_fwd_f16_bp.h at three
-// workgroups per CU, whose workgroups are all resident from the start when they fit.
+// workgroups per CU; small launches) and, for launches with more than two tiles per CU, the
+// block-pipelined one of attn_fwd_f16_bp.h (three workgroups per CU at head widths 32 and
+// 64, two at 128), whose workgroups are all resident from the start when they fit.
 //
 // Work decomposition
 //   grid  = one workgroup per (head, 128-row query tile), dealt to the XCDs so a
@@ -35,7 +35,6 @@
 // of their use so HBM/L2 latency is off the critical path; tiles are unpadded and
 // XOR-swizzled by 16-byte chunk.  One barrier per iteration.
 #include <algorithm>
-#include <cstdlib>
 #include <map>
 #include <tuple>
 #include <type_traits>
@@ -469,7 +468,9 @@ static const TileOrder* resident_order(int heads_per_xcd, int T, bool* use_resid
   const int n_qtiles = (T + kFwdBM - 1) / kFwdBM;
   const int n_items = heads_per_xcd * n_qtiles;
   // launches that fit the pipelined kernel's two workgroups per CU are faster there
-  entry.resident = per_cu > 2 && n_items > 2 * n_cu;
+  // (head width 128: both kernels hold two workgroups per CU and the block-pipelined one is the
+  // faster from the same size on: 1x16x8192x128 267 against 296 us)
+  entry.resident = (D == 128 ? per_cu >= 2 : per_cu > 2) && n_items > 2 * n_cu;
   *use_resident_kernel = entry.resident;
   if (!entry.resident || n_items > n_cu * per_cu || n_items > kMaxResidentTiles) return nullptr;
   std::vector<long> load(n_cu, 0);
@@ -502,15 +503,19 @@ static void launch_fwd_f16_d(const FwdParams& p, int B, hipStream_t stream) {
   const int heads_per_xcd = (BH + 7) / 8;
   const size_t lds = FwdCfg<D>::kLds;
   static bool attr_set = false;  // launches are serialised by the caller
-  if (!attr_set && lds > 64 * 1024) {
-    (void)hipFuncSetAttribute((const void*)attn_fwd_f16_kernel<D>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (!attr_set) {
+    if (lds > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_fwd_f16_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds);
+    if (BpCfg<D>::kLds > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)attn_fwd_f16_bp_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)BpCfg<D>::kLds);
     attr_set = true;
   }
   LaunchScope scope("attn_fwd_f16", stream);
-  if constexpr (D <= 64) {
+  {
     // More tiles than the tile-pipelined kernel holds at once (two workgroups per CU): the
-    // block-pipelined kernel at three workgroups per CU.  While they all fit, every workgroup
+    // block-pipelined kernel, at three workgroups per CU for head widths 32 and 64.  While they all fit, every workgroup
     // is resident from the start, placed for even CU totals, and nothing is left to a tail of
     // late, short workgroups; beyond that the dispatcher hands out each XCD's list longest
     // first.  Smaller launches are faster on the tile-pipelined kernel (2x12x2048x64: 33.6
