@@ -100,13 +100,13 @@ def test_config2_f16_full_size():
 
 @pytest.mark.parametrize("B,H,T,D", [(5, 16, 1000, 64), (3, 25, 897, 64), (4, 12, 2048, 64),
                                      (8, 12, 1024, 32), (10, 12, 1001, 32), (16, 12, 1024, 64),
-                                     (9, 13, 1500, 64)])
+                                     (9, 13, 1500, 64), (2, 8, 4100, 128), (3, 9, 2500, 128)])
 def test_forward_on_the_plain_kernel(B, H, T, D):
-    """f16 geometries with more than two query tiles per CU and XCD: the forward takes the kernel
-    with three (D=64) or four (D=32) workgroups per CU, with the placement table while all
-    workgroups fit at once (ragged last tile, a head count that does not fill the last round of
-    XCDs, the 2048-token case) and with the dispatcher's longest-first order beyond (the last two
-    cases).  The oracle runs on the first and last batch entries; the whole output is checked for
+    """f16 geometries with more than two query tiles per CU and XCD: the forward takes the
+    block-pipelined kernel (three workgroups per CU at D = 32 and 64, two at D = 128), with the
+    placement table while all workgroups fit at once (ragged last tile, a head count that does
+    not fill the last round of XCDs, the 2048-token case) and with the dispatcher's longest-first
+    order beyond (the last four cases; the D = 128 ones end in a partial 32-key block).  The oracle runs on the first and last batch entries; the whole output is checked for
     finiteness, the first row, and bit-reproducibility."""
     x = synth.attention_inputs(f"resident-{B}-{H}-{T}-{D}", B, H, T, D, np.float16, base_seed=3)
     o, lse, dq, dk, dv = check_case(x, 5e-3, f"resident B{B} H{H} T{T}", heads=[0, B - 1])
