@@ -1,5 +1,5 @@
 // Block-pipelined causal attention backward (f16 storage, f32 accumulate, gfx950): the two role
-// bodies of the single-launch backward for head widths 32 and 64.
+// bodies of the single-launch backward (attn_bwd_f16.hip) for head widths 32, 64 and 128.
 //
 //     P  = exp(S*scale + mask - LSE)        dV = P^T dO
 //     dP = dO V^T                           dS = P o (dP - delta),  delta = rowsum(dO o O)
@@ -7,10 +7,9 @@
 // (the reference's backward bodies: src/ops.rs:1089-1101, 422-425, 210-214, 777-799, 1162-1175,
 // 638-643, walked by src/backprop.rs:52-66).
 //
-// Same decomposition as the tile kernels of attn_bwd_f16.hip (a dQ workgroup owns 128 queries
-// and walks the keys up to the diagonal, a dK/dV workgroup owns 128 keys and walks the queries
-// from the diagonal on; the dQ role publishes the row statistics the dK/dV role needs), but
-// the loops follow what the SIMD rewards (see attn_fwd_f16_bp.h): the unit is a 32-row block of
+// A dQ workgroup owns 128 queries and walks the keys up to the diagonal, a dK/dV workgroup owns
+// 128 keys and walks the queries from the diagonal on; the dQ role publishes the row statistics
+// the dK/dV role needs.  The loops follow what the SIMD rewards (see attn_fwd_f16_bp.h): the unit is a 32-row block of
 // the streamed operand, and in stage n a wave issues the MFMAs that consume block n-1's
 // probabilities (dV, dK, or dQ) and those that produce block n+1's scores (S, dP) between the
 // vector ops of block n, one MFMA per score register: exponential, multiply and the f16 packing
@@ -78,7 +77,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   constexpr int NM2 = 4 * DB;               // MFMAs that consume a block: (dV, dK) x 2 steps x DB
   constexpr int NM1 = 2 * KS;               // MFMAs that produce a block: (S, dP) x KS
   constexpr int W = 4;                      // operand fragments in flight ahead of their MFMA
-  static_assert(D == 64 || D == 32, "head widths 32 and 64");
+  static_assert(D == 128 || D == 64 || D == 32, "head widths 32, 64 and 128");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
