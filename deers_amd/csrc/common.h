@@ -286,16 +286,6 @@ __device__ __forceinline__ bool map_block(int block_id, int n_blocks, int heads_
   return *bh < BH;
 }
 
-// Long blocks are the critical path of a causal launch: waves of the longest
-// blocks ask the instruction arbiter for priority over the short blocks that share
-// their SIMD, which then fill the gaps.
-__device__ __forceinline__ void set_block_priority(int rank, int n_blocks) {
-  const int q = (4 * rank) / max(n_blocks, 1);  // 0 = longest quarter
-  if (q == 0) __builtin_amdgcn_s_setprio(3);
-  else if (q == 1) __builtin_amdgcn_s_setprio(2);
-  else if (q == 2) __builtin_amdgcn_s_setprio(1);
-}
-
 // Brackets one kernel launch with a hipEvent pair when per-kernel profiling is
 // switched on (deers_rocm_profile_enable); a no-op otherwise.  Defined in
 // runtime.hip.
