@@ -67,7 +67,8 @@ SHAPES = [
     (np.float16, 1, 2, 64, 64), (np.float16, 1, 2, 65, 64), (np.float16, 2, 3, 127, 64),
     (np.float16, 1, 2, 128, 64), (np.float16, 1, 2, 129, 64), (np.float16, 1, 2, 300, 64),
     (np.float16, 1, 2, 513, 64), (np.float16, 2, 2, 100, 32), (np.float16, 1, 2, 257, 128),
-    (np.float16, 1, 1, 1024, 128),
+    (np.float16, 1, 1, 1024, 128), (np.float16, 1, 2, 31, 128), (np.float16, 2, 3, 333, 128),
+    (np.float16, 1, 1, 640, 128), (np.float16, 3, 3, 200, 128), (np.float16, 1, 3, 700, 32),
 ]
 
 
@@ -186,11 +187,12 @@ def test_causality_and_linearity_properties():
     assert max_err(gk[:, :, -1], dk[:, :, -1]) <= 5e-3 and max_err(gv[:, :, -1], dv[:, :, -1]) <= 5e-3
 
 
-def test_strided_head_interleaved_layout():
+@pytest.mark.parametrize("D", [64, 128])
+def test_strided_head_interleaved_layout(D):
     """v reaches the reference's matmul as a [B,H,T,D] view of [B,T,H,D] memory
     (strides [T*C, D, C, 1], src/models/gpt.rs:137); the ABI takes such views by stride."""
-    B, H, T, D = 2, 3, 150, 64
-    x = synth.attention_inputs("strided", B, H, T, D, np.float16, base_seed=5)
+    B, H, T = 2, 3, 150
+    x = synth.attention_inputs(f"strided{D}", B, H, T, D, np.float16, base_seed=5)
     want_o, want_lse, want_dq, want_dk, want_dv = rocm.attn_fwd_bwd(x["q"], x["k"], x["v"], x["do"])
     C = H * D
     st = (T * C, D, C, 1)
