@@ -19,6 +19,8 @@
 //      (what fits in the 32 clocks of an MFMA, and what each further instruction costs)
 //   H  one or two MFMAs per 1 KiB operand fragment read from LDS, with and without the
 //      softmax's vector ops, and the rate of MFMAs chained through one accumulator
+//   P  a bare MFMA stream again, on operands of zeros, a constant, and random values: the
+//      device is power limited and the clock it sustains depends on the data
 //
 // Every launch covers all CUs (256 workgroups x waves); times are clock64() deltas from the
 // common start of a CU's waves to the end of its slowest wave, averaged over the CUs, so
@@ -27,6 +29,7 @@
 // microbench; run: deers_amd/csrc/microbench/simd_mfma_valu.
 #include <cstdio>
 #include <cstdlib>
+#include <vector>
 
 #include "../attn_fwd_f16_bp.h"
 #include "../common.h"
@@ -392,39 +395,60 @@ static void run_fwd_iteration(const half_t* Kg, const half_t* Vg) {
 
 
 // ---- F: the block-pipelined forward's own loop (attn_fwd_f16_bp.h compiled in its bench mode) ----
-template <int OCC>
+template <int OCC, int DH>
 __global__ __launch_bounds__(256, OCC) void fwd_bp_bench_kernel(FwdParams p, int BH, int n_qtiles, int heads_per_xcd,
                                                                 TileOrder order, int stages, long long* clk) {
-  attn_fwd_f16_bp_body<64, true>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
+  attn_fwd_f16_bp_body<DH, true>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
 }
-template <int OCC>
+template <int OCC, int DH = 64>
 static void run_fwd_bp(int wgs) {
   const int stages = 4000, T = 1024, n_qtiles = 8, heads_per_xcd = 4 * wgs, BH = 8 * heads_per_xcd;
-  const size_t elems = (size_t)BH * T * 64;
+  const size_t elems = (size_t)BH * T * DH;
   half_t *q, *k, *v, *o;
   float* lse;
   long long* clk;
   CK(hipMalloc(&q, elems * 2)); CK(hipMalloc(&k, elems * 2)); CK(hipMalloc(&v, elems * 2)); CK(hipMalloc(&o, elems * 2));
   CK(hipMalloc(&lse, (size_t)BH * T * 4));
   CK(hipMalloc(&clk, 256 * 4 * 4 * sizeof(long long)));
-  CK(hipMemset(q, 0, elems * 2)); CK(hipMemset(k, 0, elems * 2)); CK(hipMemset(v, 0, elems * 2));
+  {  // random operands (sigma 0.25, scores stay small): the clock the loop sustains depends on the data
+    static std::vector<_Float16> h;
+    h.resize(elems);
+    unsigned s = 99;
+    for (size_t i = 0; i < elems; ++i) {
+      float u = 0;
+      for (int j = 0; j < 4; ++j) { s = s * 1664525u + 1013904223u; u += (s >> 8) / 16777216.0f; }
+      h[i] = (_Float16)((u - 2.0f) * 1.73f * 0.25f);
+    }
+    CK(hipMemcpy(q, h.data(), elems * 2, hipMemcpyHostToDevice));
+    CK(hipMemcpy(k, h.data(), elems * 2, hipMemcpyHostToDevice));
+    CK(hipMemcpy(v, h.data(), elems * 2, hipMemcpyHostToDevice));
+  }
   FwdParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
-  p.sq = p.sk = p.sv = p.so = Strides3{(int64_t)T * 64, (int64_t)T * 64, 64};  // B = BH "batches" of one head
+  p.sq = p.sk = p.sv = p.so = Strides3{(int64_t)T * DH, (int64_t)T * DH, DH};  // B = BH "batches" of one head
   p.H = 1; p.T = T; p.scale_log2 = 0.18f;
   TileOrder order{};
   order.code[0] = -1;
-  const size_t lds = BpCfg<64>::kLds;
-  fwd_bp_bench_kernel<OCC><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, 100, clk);
-  fwd_bp_bench_kernel<OCC><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
+  const size_t lds = BpCfg<DH>::kLds;
+  if (lds > 64 * 1024)
+    CK(hipFuncSetAttribute((const void*)fwd_bp_bench_kernel<OCC, DH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  fwd_bp_bench_kernel<OCC, DH><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, 100, clk);
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+  CK(hipEventRecord(e0));
+  fwd_bp_bench_kernel<OCC, DH><<<256 * wgs, 256, lds>>>(p, BH, n_qtiles, heads_per_xcd, order, stages, clk);
+  CK(hipEventRecord(e1));
   CK(hipDeviceSynchronize());
+  float ms = 0;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  CK(hipEventDestroy(e0)); CK(hipEventDestroy(e1));
   static long long h[256 * 4 * 4];
   CK(hipMemcpy(h, clk, sizeof(long long) * 256 * wgs * 4, hipMemcpyDeviceToHost));
   double s = 0;
   for (int i = 0; i < 256 * wgs * 4; ++i) s += (double)h[i];
   const double per_stage = s / (256.0 * wgs * 4) / stages;
-  printf("F block-pipelined forward (launch bound %d), %d workgroup(s) = wave(s)/SIMD per CU: %5.0f clocks per wave-stage (32 keys) = %4.0f of SIMD time (its 8 MFMAs alone: 256)\n",
-         OCC, wgs, per_stage, per_stage / wgs);
+  printf("F block-pipelined forward, head width %d (launch bound %d), %d workgroup(s) = wave(s)/SIMD per CU: %5.0f clocks per wave-stage (32 keys) = %4.0f of SIMD time (its %d MFMAs alone: %d); %.2f GHz\n",
+         DH, OCC, wgs, per_stage, per_stage / wgs, DH / 8, DH * 4, per_stage * stages / (ms * 1e6));
   CK(hipFree(q)); CK(hipFree(k)); CK(hipFree(v)); CK(hipFree(o)); CK(hipFree(lse)); CK(hipFree(clk));
 }
 
@@ -620,14 +644,72 @@ static void run_chain() {
   printf("H MFMAs through %d accumulator(s) in turn: %5.1f clocks per MFMA\n", DIST, slowest_wave_clocks(256, 0, 4) / (2000.0 * 16));
 }
 
+// ---- P: what the operand DATA does to a bare MFMA stream (the device is power limited) --------
+// Eight A and four B fragments read once from memory, then only MFMAs, ~5 ms per run on every
+// CU.  Rate by events; shader clock = wave clocks / event time.
+__global__ __launch_bounds__(256) void mfma_data_kernel(const half8* src, float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63;
+  half8 a[8], b[4];
+  for (int i = 0; i < 8; ++i) a[i] = src[i * 64 + lane];
+  for (int i = 0; i < 4; ++i) b[i] = src[(8 + i) * 64 + lane];
+  floatx16 acc[4] = {ZERO16, ZERO16, ZERO16, ZERO16};
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc[c & 3] = mfma_f16(a[c & 7], b[(c >> 1) & 3], acc[c & 3]);
+    if ((it & 63) == 63)  // keeps the accumulators finite without touching the operands
+      for (int j = 0; j < 4; ++j)
+        for (int e = 0; e < 16; ++e) acc[j][e] *= 0.0009765625f;
+  }
+  const long long t1 = clock64();
+  float r = 0;
+  for (int j = 0; j < 4; ++j)
+    for (int e = 0; e < 16; ++e) r += acc[j][e];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (threadIdx.x == 0) clk[blockIdx.x] = t1 - t0;
+}
+static void run_mfma_data() {
+  half8* src;
+  CK(hipMalloc(&src, 12 * 64 * sizeof(half8)));
+  static _Float16 h[12 * 64 * 8];
+  const char* names[] = {"zeros", "the constant 0.5", "random values, sigma 1", "random values, sigma 1, every other lane zero"};
+  for (int mode = 0; mode < 4; ++mode) {
+    unsigned s = 12345;
+    for (int i = 0; i < 12 * 64 * 8; ++i) {
+      float u = 0;
+      for (int j = 0; j < 4; ++j) { s = s * 1664525u + 1013904223u; u += (s >> 8) / 16777216.0f; }
+      const float g = (u - 2.0f) * 1.73f;  // sum of four uniforms, unit variance
+      h[i] = (_Float16)(mode == 0 ? 0.f : mode == 1 ? 0.5f : (mode == 3 && ((i / 8) & 1)) ? 0.f : g);
+    }
+    CK(hipMemcpy(src, h, sizeof(h), hipMemcpyHostToDevice));
+    const int iters = 20000;
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    mfma_data_kernel<<<256, 256>>>(src, g_out, g_clk, 200);
+    CK(hipEventRecord(e0));
+    mfma_data_kernel<<<256, 256>>>(src, g_out, g_clk, iters);
+    CK(hipEventRecord(e1));
+    CK(hipDeviceSynchronize());
+    float ms = 0;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    long long c0 = 0;
+    CK(hipMemcpy(&c0, g_clk, 8, hipMemcpyDeviceToHost));
+    printf("P bare MFMA stream, operands = %-46s: %5.0f TFLOP/s, shader clock %.2f GHz\n", names[mode],
+           256.0 * 4 * iters * 16.0 * 32768.0 / (ms * 1e-3) / 1e12, (double)c0 / (ms * 1e6));
+    CK(hipEventDestroy(e0)); CK(hipEventDestroy(e1));
+  }
+  CK(hipFree(src));
+}
+
 int main() {
   CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
   CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
   if (getenv("MICROBENCH_ONLY_F")) {
-    run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3); run_fwd_bp<2>(1); run_fwd_bp<2>(2);
+    run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3); run_fwd_bp<2, 128>(1); run_fwd_bp<2, 128>(2);
     return 0;
   }
   run_mfma_stream();
+  run_mfma_data();
   run_valu_rate<0>("v_fma_f32 independent");
   run_valu_rate<1>("v_fma_f32 dependent");
   run_valu_rate<2>("v_exp_f32");
@@ -657,6 +739,7 @@ int main() {
   run_phase<0, 1>("free running");
   run_phase<1, 1>("opposite phases");
   run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3);
+  run_fwd_bp<2, 128>(1); run_fwd_bp<2, 128>(2);
   run_chunk<0>("2 exp, cvt_pk");
   run_chunk<1>("2 exp, cvt_pk, add");
   run_chunk<2>("2 exp, cvt_pk, 2 add");
