@@ -57,9 +57,11 @@ struct TileOrder {
 // global -> LDS asynchronously into rings, F stages ahead, one barrier per stage; a block has
 // landed one barrier before its first use, so the first V fragments of a stage leave LDS at the
 // end of the stage before it, across the barrier, and the K fragments (needed in the stage's
-// second half) right after it.  Every wave runs every stage of its workgroup, S products
-// included: a branch around a single MFMA costs a lone wave more than the MFMA (eight such
-// branches per stage were 23 % of the stage).
+// second half) right after it.  Inside a stage nothing is conditional (a branch around a single
+// MFMA costs a lone wave more than the MFMA: eight such branches per stage were 23 % of the
+// stage); what a wave leaves out it leaves out in whole stages at the end of its walk: the
+// pair of stages at its diagonal block forms no further scores, and after it the wave only
+// keeps the workgroup's barriers and its share of the loads.
 // Hook for a timestamp-tracing build of this kernel; expands to nothing in the library.
 #ifndef DEERS_TRACE_POINT
 #define DEERS_TRACE_POINT(slot)
@@ -252,11 +254,12 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
   // refill the slots of K(b) and V(b-2), and the exponentials, sums and packing of block b.
   // One body serves every position of a wave: variants per position made the register
   // allocator spill hundreds of values.
-  auto stage = [&](auto first_c, auto slot_c, int b, floatx16& cur, floatx16& nxt) {
+  auto stage = [&](auto first_c, auto produce_c, auto slot_c, int b, floatx16& cur, floatx16& nxt) {
     constexpr bool FIRST = decltype(first_c)::value, HAS_PV = !FIRST;
-    constexpr int SLOT = decltype(slot_c)::value;
-    constexpr uint32_t KSLOT = (SLOT + 1) % R, VSLOT = (SLOT + R - 1) % R;
-    constexpr int NPV = HAS_PV ? 2 * DB : 0, NMS = KS, NM = NPV + NMS;
+    constexpr bool PRODUCE = decltype(produce_c)::value;  // false: block b + 1 lies past the wave's diagonal
+    const uint32_t SLOT = (uint32_t)slot_c;  // a constant in the unrolled ring, a value in the last pair
+    const uint32_t KSLOT = (SLOT + 1) % R, VSLOT = (SLOT + R - 1) % R;
+    constexpr int NPV = HAS_PV ? 2 * DB : 0, NMS = PRODUCE ? KS : 0, NM = NPV + NMS;
     constexpr int NPRE = HAS_PV ? NPF : 0;  // fragments already in fr
     constexpr bool ROLL = NM % W == 0;      // a fetched fragment lands in the register its MFMA names
     const bool masked = b >= bd;  // block b is the wave's diagonal block, or lies beyond it
@@ -302,7 +305,7 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
         else if (ROLL && mi + W - NM < NPF)
           fr[mi % W] = fetch_v(mi + W - NM, SLOT);  // the next stage multiplies V(b) by P(b)
       }
-      if (!FIRST && i < 4) seed_part(i, nxt);
+      if (!FIRST && PRODUCE && i < 4) seed_part(i, nxt);
       if (i >= 1 && i <= LPI) request_part(i - 1, b + 1 + F, b + F, (SLOT + 1 + F) % R, (SLOT + F) % R);
       if constexpr (FIRST) {
         cur[2 * i] = fast_exp2(cur[2 * i] - m);
@@ -390,39 +393,52 @@ __device__ __forceinline__ void attn_fwd_f16_bp_body(const FwdParams& p, int BH,
   // ---- stage b: barrier b retires the reads of K(b) and V(b-2), whose slots request(b) refills
   // (with K(b+1+F) and V(b+F); both rings have F + 2 slots), and makes K(b+1) and V(b), requested
   // F stages ago, visible ----
-  auto open_stage = [&](auto slot_c, int b) {
-    constexpr int SLOT = decltype(slot_c)::value;
+  auto open_stage = [&]() {
     wait_vmcnt<(F - 1) * LPI>();
     // A bare barrier: no wait for the LDS reads in flight.  Those are the next stage's first V
     // fragments and the seed, whose slots are not refilled for another stage; every read of the
     // two slots the request refills has been consumed by an MFMA this wave issued already.
     __builtin_amdgcn_s_barrier();
   };
-  open_stage(std::integral_constant<int, 0>{}, 0);
-  stage(yes, std::integral_constant<int, 0>{}, 0, sa, sb);
+  open_stage();
+  stage(yes, yes, std::integral_constant<int, 0>{}, 0, sa, sb);
   DEERS_TRACE_POINT(2);
   [[maybe_unused]] const long long bench_t0 = BENCH ? clock64() : 0;
-  // Every wave runs every stage of the workgroup, two at a time (an odd count runs one more,
-  // fully masked stage): past its diagonal block a wave sees masked blocks, probabilities 0.
-  // Skipping those stages per wave was measured in the compiler, not on the device: any path
-  // around a stage body made the register allocator spill 100-700 values.  The loop body is one
-  // turn of the ring, so that every LDS address is a fixed register plus an instruction offset.
-  auto two_stages = [&](auto slot_c, int b) {  // stages b (odd) and b + 1
-    constexpr int SLOT = decltype(slot_c)::value;
-    open_stage(std::integral_constant<int, SLOT>{}, b);
-    stage(no, std::integral_constant<int, SLOT>{}, b, sb, sa);
-    open_stage(std::integral_constant<int, (SLOT + 1) % R>{}, b + 1);
-    stage(no, std::integral_constant<int, (SLOT + 1) % R>{}, b + 1, sa, sb);
+  // Stages come two at a time (an odd count runs one more, fully masked stage).  A wave's last
+  // block is its diagonal block bd, consumed in stage bd + 1: after the pair that holds that
+  // stage the wave only keeps the workgroup's barriers and its share of the loads.  (Any path
+  // AROUND a stage body inside the walk made the register allocator spill 100-700 values; leaving
+  // the walk early does not.)  The loop body is one turn of the ring, so that every LDS address
+  // is a fixed register plus an instruction offset.
+  auto two_stages = [&](auto produce_c, auto slot_c, int b) {  // stages b (odd) and b + 1
+    const uint32_t slot = (uint32_t)slot_c;
+    open_stage();
+    stage(no, produce_c, slot_c, b, sb, sa);
+    open_stage();
+    if constexpr (std::is_integral_v<decltype(slot_c)>)
+      stage(no, produce_c, (slot + 1) % R, b + 1, sa, sb);
+    else
+      stage(no, produce_c, std::integral_constant<int, (decltype(slot_c)::value + 1) % R>{}, b + 1, sa, sb);
     DEERS_TRACE_POINT(3 + (b >> 1));
   };
-  for (int b = 1; b <= n_blk; b += R) {
-    two_stages(std::integral_constant<int, 1>{}, b);
-    if (b + 2 > n_blk) break;
-    two_stages(std::integral_constant<int, 3 % R>{}, b + 2);
-    if constexpr (R == 6) {
-      if (b + 4 > n_blk) break;
-      two_stages(std::integral_constant<int, 5>{}, b + 4);
-    }
+  const int n_total = (n_blk + 1) & ~1;                              // the workgroup's last stage
+  const int n_live = BENCH ? n_total : min(n_total, (bd + 2) & ~1);  // this wave's last stage with work
+  // The wave's last pair of stages, (n_live - 1, n_live), lies at or past its diagonal block:
+  // it forms no further scores.
+  const int b_last = BENCH ? n_live + 1 : n_live - 1;
+  // Whole turns of the ring run with constant slots; the remaining pairs take the slot as a
+  // value.  (Leaving the unrolled turn from its middle made the register allocator spill.)
+  int b = 1;
+  for (; b + R <= b_last; b += R) {
+    two_stages(yes, std::integral_constant<int, 1>{}, b);
+    two_stages(yes, std::integral_constant<int, 3 % R>{}, b + 2);
+    if constexpr (R == 6) two_stages(yes, std::integral_constant<int, 5>{}, b + 4);
+  }
+  for (; b < b_last; b += 2) two_stages(yes, (uint32_t)b % R, b);
+  if constexpr (!BENCH) two_stages(no, (uint32_t)b_last % R, b_last);
+  for (b = n_live + 1; b <= n_total; ++b) {  // stages without work: the barrier and the loads
+    open_stage();
+    request(b + 1 + F, b + F, (uint32_t)(b + 1 + F) % R, (uint32_t)(b + F) % R);
   }
   if constexpr (BENCH) {
     if (lane == 0) bench_clk[blockIdx.x * 4 + wave] = clock64() - bench_t0;

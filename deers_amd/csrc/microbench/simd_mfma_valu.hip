@@ -668,6 +668,60 @@ __global__ __launch_bounds__(256) void mfma_data_kernel(const half8* src, float*
   out[blockIdx.x * blockDim.x + threadIdx.x] = r;
   if (threadIdx.x == 0) clk[blockIdx.x] = t1 - t0;
 }
+// The f32 matrix instruction (v_mfma_f32_32x32x2_f32, 64 clocks) the same way.
+__global__ __launch_bounds__(256) void mfma_f32_data_kernel(const float* src, float* out, long long* clk, int iters) {
+  const int lane = threadIdx.x & 63;
+  float a[8], b[4];
+  for (int i = 0; i < 8; ++i) a[i] = src[i * 64 + lane];
+  for (int i = 0; i < 4; ++i) b[i] = src[(8 + i) * 64 + lane];
+  floatx16 acc[4] = {ZERO16, ZERO16, ZERO16, ZERO16};
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c)
+      acc[c & 3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c & 7], b[(c >> 1) & 3], acc[c & 3], 0, 0, 0);
+    if ((it & 63) == 63)
+      for (int j = 0; j < 4; ++j)
+        for (int e = 0; e < 16; ++e) acc[j][e] *= 0.0009765625f;
+  }
+  const long long t1 = clock64();
+  float r = 0;
+  for (int j = 0; j < 4; ++j)
+    for (int e = 0; e < 16; ++e) r += acc[j][e];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (threadIdx.x == 0) clk[blockIdx.x] = t1 - t0;
+}
+static void run_mfma_f32_data() {
+  float* src;
+  CK(hipMalloc(&src, 12 * 64 * sizeof(float)));
+  static float h[12 * 64];
+  const char* names[] = {"zeros", "random values, sigma 1"};
+  for (int mode = 0; mode < 2; ++mode) {
+    unsigned s = 777;
+    for (int i = 0; i < 12 * 64; ++i) {
+      float u = 0;
+      for (int j = 0; j < 4; ++j) { s = s * 1664525u + 1013904223u; u += (s >> 8) / 16777216.0f; }
+      h[i] = mode == 0 ? 0.f : (u - 2.0f) * 1.73f;
+    }
+    CK(hipMemcpy(src, h, sizeof(h), hipMemcpyHostToDevice));
+    const int iters = 10000;
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    mfma_f32_data_kernel<<<256, 256>>>(src, g_out, g_clk, 200);
+    CK(hipEventRecord(e0));
+    mfma_f32_data_kernel<<<256, 256>>>(src, g_out, g_clk, iters);
+    CK(hipEventRecord(e1));
+    CK(hipDeviceSynchronize());
+    float ms = 0;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    long long c0 = 0;
+    CK(hipMemcpy(&c0, g_clk, 8, hipMemcpyDeviceToHost));
+    printf("P bare f32 MFMA stream (32x32x2), operands = %-30s: %5.1f TFLOP/s, shader clock %.2f GHz\n", names[mode],
+           256.0 * 4 * iters * 16.0 * 4096.0 / (ms * 1e-3) / 1e12, (double)c0 / (ms * 1e6));
+    CK(hipEventDestroy(e0)); CK(hipEventDestroy(e1));
+  }
+  CK(hipFree(src));
+}
 static void run_mfma_data() {
   half8* src;
   CK(hipMalloc(&src, 12 * 64 * sizeof(half8)));
@@ -704,12 +758,18 @@ static void run_mfma_data() {
 int main() {
   CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
   CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
+  if (getenv("MICROBENCH_ONLY_P")) {
+    run_mfma_data();
+    run_mfma_f32_data();
+    return 0;
+  }
   if (getenv("MICROBENCH_ONLY_F")) {
     run_fwd_bp<3>(1); run_fwd_bp<3>(2); run_fwd_bp<3>(3); run_fwd_bp<2, 128>(1); run_fwd_bp<2, 128>(2);
     return 0;
   }
   run_mfma_stream();
   run_mfma_data();
+  run_mfma_f32_data();
   run_valu_rate<0>("v_fma_f32 independent");
   run_valu_rate<1>("v_fma_f32 dependent");
   run_valu_rate<2>("v_exp_f32");
