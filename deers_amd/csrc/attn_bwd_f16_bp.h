@@ -57,6 +57,19 @@ struct BwdBpCfg {
   static constexpr size_t kLds = kLdsDkdv > kLdsDq ? kLdsDkdv : kLdsDq;
 };
 
+// A ring slot is either a value or, in the unrolled turns of the ring, a compile-time constant.
+template <uint32_t N>
+using SlotC = std::integral_constant<uint32_t, N>;
+template <class S>
+constexpr bool kConstSlot = !std::is_integral_v<S>;
+template <int R, int K, class S>
+__device__ __forceinline__ auto slot_plus(S s) {
+  if constexpr (kConstSlot<S>)
+    return SlotC<(S::value + K) % R>{};
+  else
+    return (uint32_t)((s + K) % R);
+}
+
 // Packs two f32 into an f16 pair (round to nearest even).
 __device__ __forceinline__ uint32_t pack_pair_f16(float a, float b) {
   return __builtin_bit_cast(uint32_t, half2v{(half_t)a, (half_t)b});
@@ -196,6 +209,37 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     }
   }
   const uint32_t va = vec_dst + 16 * g;  // this wave's vectors: rows 4g .. (+32 rq)
+  // A ring of more than 64 KB does not fit the 16-bit offset of an LDS instruction: the upper
+  // half of its slots is addressed from a second set of base registers (where the slot is a
+  // constant of the unrolled ring; a slot held in a register is added to the base).
+  constexpr bool SPLIT = (size_t)R * SLOT_B > 65536;
+  constexpr uint32_t HALF_B = (R / 2) * SLOT_B;
+  uint32_t aa_hi[SPLIT ? KS : 1], ta_lo_hi[SPLIT ? DB : 1], ta_hi_hi[SPLIT ? DB : 1];
+  if constexpr (SPLIT) {  // (opaque, or the compiler recomputes each of them at every use)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      aa_hi[ks] = aa[ks] + HALF_B;
+      asm volatile("" : "+v"(aa_hi[ks]));
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      ta_lo_hi[db] = ta_lo[db] + HALF_B;
+      ta_hi_hi[db] = ta_hi[db] + HALF_B;
+      asm volatile("" : "+v"(ta_lo_hi[db]), "+v"(ta_hi_hi[db]));
+    }
+  }
+  uint32_t va_lo[1] = {va}, va_hi[1] = {va + HALF_B};
+  if constexpr (SPLIT) asm volatile("" : "+v"(va_hi[0]));
+  auto slot_addr = [&](const uint32_t* lo, [[maybe_unused]] const uint32_t* hi, int idx, auto slot) -> uint32_t {
+    if constexpr (SPLIT && kConstSlot<decltype(slot)>) {
+      if constexpr (decltype(slot)::value >= (uint32_t)(R / 2))
+        return hi[idx] + (decltype(slot)::value - R / 2) * SLOT_B;
+      else
+        return lo[idx] + decltype(slot)::value * SLOT_B;
+    } else {
+      return lo[idx] + (uint32_t)slot * SLOT_B;
+    }
+  };
 
   floatx16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -218,23 +262,23 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
 
   // fragment mi of the MFMAs that consume the block in `slot`: (step st, output block db, dV|dK)
   // = (mi / (2 DB), (mi / 2) % DB, mi % 2); dV reads dO^T, dK reads Q^T
-  auto fetch2 = [&](int mi, uint32_t slot) -> half8 {
+  auto fetch2 = [&](int mi, auto slot) -> half8 {
     const int st = mi / (2 * DB), db = (mi >> 1) % DB;
-    const uint32_t off = slot * SLOT_B + ((mi & 1) ? 0 : TB) + 16 * st * RB;
-    const half4 lo = lds_read_tr16_at(ta_lo[db] + off);
-    const half4 hi = lds_read_tr16_at(ta_hi[db] + off);
+    const uint32_t off = ((mi & 1) ? 0 : TB) + 16 * st * RB;
+    const half4 lo = lds_read_tr16_at(slot_addr(ta_lo, ta_lo_hi, db, slot) + off);
+    const half4 hi = lds_read_tr16_at(slot_addr(ta_hi, ta_hi_hi, db, slot) + off);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
   // fragment mi of the MFMAs that produce the block in `slot`: (contraction step, S|dP) = (mi / 2, mi % 2)
-  auto fetch1 = [&](int mi, uint32_t slot) -> half8 {
-    return lds_read_half8_at(aa[mi >> 1] + slot * SLOT_B + ((mi & 1) ? TB : 0));
+  auto fetch1 = [&](int mi, auto slot) -> half8 {
+    return lds_read_half8_at(slot_addr(aa, aa_hi, mi >> 1, slot) + ((mi & 1) ? TB : 0));
   };
   // accumulator seeds of the block in `slot`: S from -lse2, dP from -delta (row values)
   // One eighth of the accumulator seeds of the block in `slot`: part 2 rq gives S rows from
   // -lse2, part 2 rq + 1 gives dP rows from -delta (row values, the same for every lane of a half)
-  auto seed_part = [&](int part, floatx16& s, floatx16& dp, uint32_t slot) {
+  auto seed_part = [&](int part, floatx16& s, floatx16& dp, auto slot) {
     const int rq = part >> 1;
-    const floatx4 a = lds_read_float4_at(va + slot * SLOT_B + ((part & 1) ? VEC_B : 0) + 32 * rq);
+    const floatx4 a = lds_read_float4_at(slot_addr(va_lo, va_hi, 0, slot) + ((part & 1) ? VEC_B : 0) + 32 * rq);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (part & 1)
@@ -253,7 +297,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   // fetch of a fragment W MFMAs ahead (rolling into the next stage's consumers, which read
   // block n), by one of the eight seed reads, by one of the loads that refill the slot of
   // block n-2 with block n+1+F, and by the exponential, product and packing of block n.
-  auto stage = [&](auto first_c, auto produce_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s,
+  auto stage = [&](auto first_c, auto produce_c, auto PSLOT, auto SLOT, auto NSLOT, int n, floatx16& s,
                    floatx16& dp, floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
     constexpr bool PRODUCE = decltype(produce_c)::value;  // false: block n+1 lies past the end
@@ -262,7 +306,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     // whether the fetches can roll on into the next stage (a fragment must land in the register
     // its MFMA names, which is the one just freed only if the counts are multiples of W)
     constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0 && NMS % W == 0;
-    const uint32_t RSLOT = (SLOT + 1 + F) % R;
+    const uint32_t RSLOT = ((uint32_t)SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
     if constexpr (FIRST) {
 #pragma unroll
@@ -367,10 +411,11 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   open_stage();
   stage(yes, yes, (uint32_t)(n0 + R - 1) % R, (uint32_t)n0, (uint32_t)n0 + 1, n0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
-  auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
-    const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
+  auto two_stages = [&](auto slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
+    const auto s1 = slot_plus<R, 1>(slot);
+    const auto s2 = slot_plus<R, 2>(slot);
     open_stage();
-    stage(no, yes, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    stage(no, yes, slot_plus<R, R - 1>(slot), slot, s1, n, sb, dpb, sa, dpa);
     open_stage();
     stage(no, yes, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
@@ -391,9 +436,9 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   int n = n0 + 1;
   for (; n % R != 1 && n + 2 <= n_total; n += 2) two_stages((uint32_t)n % R, n);  // up to the ring's start
   for (; n + R + 1 <= n_total; n += R) {
-    two_stages(1, n);
-    two_stages(3, n + 2);
-    two_stages(5, n + 4);
+    two_stages(SlotC<1>{}, n);
+    two_stages(SlotC<3>{}, n + 2);
+    two_stages(SlotC<5>{}, n + 4);
   }
   for (; n + 2 <= n_total; n += 2) two_stages((uint32_t)n % R, n);
   if (n <= n_total) last_two_stages((uint32_t)n % R, n);
@@ -528,6 +573,33 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
       ta_hi[db] = lds0 + (lrow + 8) * RB + ((chunk ^ lds_swizzle<CH>(lrow + 8)) << 4) + (c4 & 1) * 8;
     }
   }
+  // (as in the dK/dV role: a second set of base registers for the upper half of a ring over 64 KB)
+  constexpr bool SPLIT = (size_t)R * SLOT_B > 65536;
+  constexpr uint32_t HALF_B = (R / 2) * SLOT_B;
+  uint32_t aa_hi[SPLIT ? KS : 1], ta_lo_hi[SPLIT ? DB : 1], ta_hi_hi[SPLIT ? DB : 1];
+  if constexpr (SPLIT) {  // (opaque, or the compiler recomputes each of them at every use)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      aa_hi[ks] = aa[ks] + HALF_B;
+      asm volatile("" : "+v"(aa_hi[ks]));
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      ta_lo_hi[db] = ta_lo[db] + HALF_B;
+      ta_hi_hi[db] = ta_hi[db] + HALF_B;
+      asm volatile("" : "+v"(ta_lo_hi[db]), "+v"(ta_hi_hi[db]));
+    }
+  }
+  auto slot_addr = [&](const uint32_t* lo, [[maybe_unused]] const uint32_t* hi, int idx, auto slot) -> uint32_t {
+    if constexpr (SPLIT && kConstSlot<decltype(slot)>) {
+      if constexpr (decltype(slot)::value >= (uint32_t)(R / 2))
+        return hi[idx] + (decltype(slot)::value - R / 2) * SLOT_B;
+      else
+        return lo[idx] + decltype(slot)::value * SLOT_B;
+    } else {
+      return lo[idx] + (uint32_t)slot * SLOT_B;
+    }
+  };
   floatx16 dqacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) dqacc[i] = ZERO16;
@@ -548,28 +620,28 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   if (tid == 0)
     __hip_atomic_store(p.ready + (int64_t)bh * n_own + qtile, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-  auto fetch2 = [&](int mi, uint32_t slot) -> half8 {  // dQ: (step, output block) = (mi / DB, mi % DB), K^T
+  auto fetch2 = [&](int mi, auto slot) -> half8 {  // dQ: (step, output block) = (mi / DB, mi % DB), K^T
     const int st = mi / DB, db = mi % DB;
-    const uint32_t off = slot * SLOT_B + 16 * st * RB;
-    const half4 lo = lds_read_tr16_at(ta_lo[db] + off);
-    const half4 hi = lds_read_tr16_at(ta_hi[db] + off);
+    const uint32_t off = 16 * st * RB;
+    const half4 lo = lds_read_tr16_at(slot_addr(ta_lo, ta_lo_hi, db, slot) + off);
+    const half4 hi = lds_read_tr16_at(slot_addr(ta_hi, ta_hi_hi, db, slot) + off);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
-  auto fetch1 = [&](int mi, uint32_t slot) -> half8 {  // (contraction step, S|dP) = (mi / 2, mi % 2): K rows | V rows
-    return lds_read_half8_at(aa[mi >> 1] + slot * SLOT_B + ((mi & 1) ? TB : 0));
+  auto fetch1 = [&](int mi, auto slot) -> half8 {  // (contraction step, S|dP) = (mi / 2, mi % 2): K rows | V rows
+    return lds_read_half8_at(slot_addr(aa, aa_hi, mi >> 1, slot) + ((mi & 1) ? TB : 0));
   };
 
   // One stage, spread over 16 chunks as in the dK/dV role: the consumers of block n-1 (dQ), the
   // producers of block n+1 (S^T, dP^T), the rolling fragment fetches, the loads that refill the
   // slot of block n-2, and the vector ops of block n.
-  auto stage = [&](auto first_c, auto produce_c, uint32_t PSLOT, uint32_t SLOT, uint32_t NSLOT, int n, floatx16& s,
+  auto stage = [&](auto first_c, auto produce_c, auto PSLOT, auto SLOT, auto NSLOT, int n, floatx16& s,
                    floatx16& dp, floatx16& sn, floatx16& dpn) {
     constexpr bool FIRST = decltype(first_c)::value;
     constexpr bool PRODUCE = decltype(produce_c)::value;  // false: block n+1 lies past the wave's diagonal
     constexpr int N2 = FIRST ? 0 : NM2, NMS = N2 + (PRODUCE ? NM1 : 0);
     constexpr int NPRE = NM2 < W ? NM2 : W;
     constexpr bool ROLL = (NM2 + NM1) % W == 0 && NM1 % W == 0 && NMS % W == 0;
-    const uint32_t RSLOT = (SLOT + 1 + F) % R;
+    const uint32_t RSLOT = ((uint32_t)SLOT + 1 + F) % R;
     auto fetch = [&](int mi) -> half8 { return mi < N2 ? fetch2(mi, PSLOT) : fetch1(mi - N2, NSLOT); };
 #pragma unroll
     for (int mi = FIRST ? 0 : NPRE; mi < W && mi < NMS; ++mi) fr[mi] = fetch(mi);
@@ -643,10 +715,11 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   open_stage();
   stage(yes, yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
-  auto two_stages = [&](uint32_t slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
-    const uint32_t s1 = (slot + 1) % R, s2 = (slot + 2) % R;
+  auto two_stages = [&](auto slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1
+    const auto s1 = slot_plus<R, 1>(slot);
+    const auto s2 = slot_plus<R, 2>(slot);
     open_stage();
-    stage(no, yes, (slot + R - 1) % R, slot, s1, n, sb, dpb, sa, dpa);
+    stage(no, yes, slot_plus<R, R - 1>(slot), slot, s1, n, sb, dpb, sa, dpa);
     open_stage();
     stage(no, yes, slot, s1, s2, n + 1, sa, dpa, sb, dpb);
   };
@@ -669,9 +742,9 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   // Its last live pair produces nothing: the blocks after it lie past its diagonal.
   int n = 1;
   for (; n + R + 1 <= n_live; n += R) {
-    two_stages(1, n);
-    two_stages(3, n + 2);
-    two_stages(5, n + 4);
+    two_stages(SlotC<1>{}, n);
+    two_stages(SlotC<3>{}, n + 2);
+    two_stages(SlotC<5>{}, n + 4);
   }
   for (; n + 2 <= n_live; n += 2) two_stages((uint32_t)n % R, n);
   if (n <= n_live) {
