@@ -200,20 +200,18 @@ def bench_decode(steps: int, warmup: int, rotate: int = 4):
     for i in range(warmup):
         call(i)
     rocm.sync()
-    rocm.profile_enable(True)
+    # one event pair around all the calls, as for the attention kernels: a pair per launch adds
+    # about 5 us of command-processor work to each
+    timer = rocm.Timer()
+    timer.start()
     for i in range(steps):
         call(i)
-    prof = rocm.profile_collect()
-    rocm.profile_enable(False)
-    calls, ms = prof["attn_decode_f16"]
+    timer.stop()
+    rocm.sync()
     nbytes = 2.0 * B * H * L * D * 2 + 2 * B * H * D * 2
-    main_us = 1e3 * ms / calls
-    total_us = main_us
-    if "attn_decode_merge" in prof:  # only launched when a head is split over workgroups
-        mcalls, mms = prof["attn_decode_merge"]
-        total_us += 1e3 * mms / mcalls
-    return dict(bytes=nbytes, kernel_us=main_us, call_us=total_us,
-                gbs_kernel=nbytes / (main_us * 1e-6) / 1e9,
+    total_us = 1e3 * timer.elapsed_ms() / steps  # the whole call: main kernel (+ merge when a head is split)
+    return dict(bytes=nbytes, kernel_us=total_us, call_us=total_us,
+                gbs_kernel=nbytes / (total_us * 1e-6) / 1e9,
                 gbs_call=nbytes / (total_us * 1e-6) / 1e9)
 
 
@@ -613,7 +611,8 @@ def main():
                 "flops_per_launch": algorithmic_flops.get(dom),
                 "executed_flops_per_launch": executed_flops.get(dom)}
 
-    dec = bench_decode(args.steps, args.warmup)
+    dec_calls = max(args.steps, 50)
+    dec = bench_decode(dec_calls, max(args.warmup, 10))
 
     out = {
         "metric": "causal attn fwd+bwd TFLOP/s & %MFMA peak (T=1024,D=64,f16); decode HBM GB/s",
@@ -636,6 +635,7 @@ def main():
         "roofline": roofline,
         "decode": {"workload": "decode f16 B=32 H=12 L=4096 D=64 (BASELINE configs[3]), "
                                "4 KV caches in rotation",
+                   "timing": "one event pair around %d back-to-back calls" % dec_calls,
                    "bytes_per_call": dec["bytes"], "kernel_us": dec["kernel_us"],
                    "call_us": dec["call_us"], "GB/s": dec["gbs_kernel"],
                    "GB/s_whole_call": dec["gbs_call"], "peak_GB/s": PEAK_HBM_GBS,
