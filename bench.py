@@ -175,6 +175,7 @@ EXTRA_CONFIGS = {
     "c1": dict(dtype=np.float32, B=4, H=6, T=256, D=32),                    # BASELINE configs[0]
     "c3": dict(dtype=np.float16, B=1, H=16, T=8192, D=128, sigma=0.5),      # BASELINE configs[2]
     "c2_d128": dict(dtype=np.float16, B=8, H=12, T=1024, D=128),            # configs[1] at head width 128
+    "c5_attn": dict(dtype=np.float32, B=8, H=12, T=1024, D=64),             # one layer's attention of configs[4]
 }
 
 
@@ -541,7 +542,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gpt", action="store_true",
                     help="skip the end-to-end GPT training step reported beside the headline")
-    ap.add_argument("--only", choices=["all", "fwd", "bwd", "c1", "c3", "c2_d128", "decode", "copy", "rope", "log_softmax", "adamw", "gpt", "storage"], default="all",
+    ap.add_argument("--only", choices=["all", "fwd", "bwd", "c1", "c3", "c2_d128", "c5_attn", "decode", "copy", "rope", "log_softmax", "adamw", "gpt", "storage"], default="all",
                     help="profiling aid: launch only this part and print its kernel times "
                          "(the headline JSON line needs the default, all)")
     args = ap.parse_args()
