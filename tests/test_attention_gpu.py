@@ -159,6 +159,13 @@ def test_config3_long_context_f16():
         say(f"C3 head {hsel}: " + " ".join(f"{n}={e:.2e}" for n, e in errs.items()))
         for n, e in errs.items():
             assert e <= 5e-3, f"C3 head {hsel} {n}: {e:.3e}"
+    # size-independent properties on the full problem
+    for a in (o, lse, dq, dk, dv):
+        assert np.isfinite(a.astype(np.float32)).all()
+    np.testing.assert_array_equal(o[:, :, 0], v[:, :, 0])             # first row attends to itself
+    o2, lse2, dq2, dk2, dv2 = rocm.attn_fwd_bwd(q, k, v, do)
+    for a, b in ((o, o2), (lse, lse2), (dq, dq2), (dk, dk2), (dv, dv2)):
+        np.testing.assert_array_equal(a, b)                           # no atomics: bit-reproducible
 
 
 def test_causality_and_linearity_properties():
