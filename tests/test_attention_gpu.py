@@ -80,6 +80,32 @@ def test_ragged_shapes_match_oracle(dtype, B, H, T, D):
     check_case(x, TOL[np.dtype(dtype)], name)
 
 
+def _random_shapes(n, seed):
+    """n seeded (dtype, B, H, T, D) draws: lengths on and around the 32-, 64- and 128-row
+    boundaries of the kernels' blocks, and B * H on both sides of a multiple of 8 (the XCDs)."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        D = int(rng.choice([32, 64, 128]))
+        dtype = np.float32 if i % 6 == 5 else np.float16
+        base = int(rng.choice([32, 64, 96, 128, 160, 256, 384, 512, 640]))
+        T = max(1, base + int(rng.integers(-2, 3)) * int(rng.choice([0, 1, 15, 31])))
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+        out.append((dtype, B, H, T, D))
+    return out
+
+
+RANDOM_SHAPES = _random_shapes(30, seed=2024)
+
+
+@pytest.mark.parametrize("dtype,B,H,T,D", RANDOM_SHAPES,
+                         ids=[f"{np.dtype(s[0]).name}-b{s[1]}h{s[2]}t{s[3]}d{s[4]}" for s in RANDOM_SHAPES])
+def test_random_shapes_match_oracle(dtype, B, H, T, D):
+    name = f"rand-{np.dtype(dtype).name}-{B}-{H}-{T}-{D}"
+    x = synth.attention_inputs(name, B, H, T, D, dtype, base_seed=13)
+    check_case(x, TOL[np.dtype(dtype)], name)
+
+
 def test_config1_f32_full():
     """B=4 H=6 T=256 D=32 f32: the reference's own CPU-runnable case."""
     x = synth.attention_inputs("c1", 4, 6, 256, 32, np.float32, base_seed=0)
@@ -101,14 +127,20 @@ def test_config2_f16_full_size():
 
 @pytest.mark.parametrize("B,H,T,D", [(5, 16, 1000, 64), (3, 25, 897, 64), (4, 12, 2048, 64),
                                      (8, 12, 1024, 32), (10, 12, 1001, 32), (16, 12, 1024, 64),
-                                     (9, 13, 1500, 64), (2, 8, 4100, 128), (3, 9, 2500, 128)])
+                                     (9, 13, 1500, 64), (2, 8, 4100, 128), (3, 9, 2500, 128),
+                                     (8, 12, 705, 64), (8, 12, 992, 64), (8, 12, 1025, 64),
+                                     (8, 12, 1056, 64), (12, 8, 801, 32), (4, 12, 1440, 128)])
 def test_forward_on_the_plain_kernel(B, H, T, D):
     """f16 geometries with more than two query tiles per CU and XCD: the forward takes the
     block-pipelined kernel (three workgroups per CU at D = 32 and 64, two at D = 128), with the
     placement table while all workgroups fit at once (ragged last tile, a head count that does
     not fill the last round of XCDs, the 2048-token case) and with the dispatcher's longest-first
-    order beyond (the last four cases; the D = 128 ones end in a partial 32-key block).  The oracle runs on the first and last batch entries; the whole output is checked for
-    finiteness, the first row, and bit-reproducibility."""
+    order beyond (9x13x1500 and the first two D = 128 cases, which end in a partial 32-key block).
+    The last six cases vary the number of 32-key blocks of the last tile (even, odd, one row into
+    a new block, a tile of a single block): a wave leaves its walk after the pair of stages at
+    its diagonal block and only keeps barriers and loads from there on.  The oracle runs on the
+    first and last batch entries; the whole output is checked for finiteness, the first row, and
+    bit-reproducibility."""
     x = synth.attention_inputs(f"resident-{B}-{H}-{T}-{D}", B, H, T, D, np.float16, base_seed=3)
     o, lse, dq, dk, dv = check_case(x, 5e-3, f"resident B{B} H{H} T{T}", heads=[0, B - 1])
     assert np.isfinite(o.astype(np.float32)).all() and np.isfinite(lse).all()
