@@ -25,7 +25,7 @@
 //             rows through the block's flag.
 // Recomputing S and dP in both roles costs 7 tile GEMMs instead of 5 but keeps every product
 // in registers and needs no dQ accumulation buffer.  Head widths 32 and 64 run two workgroups
-// per CU; head width 128 needs 226 + 160 registers and runs one.
+// per CU; head width 128 needs more than 256 registers (213 + 160 accumulation registers) and runs one.
 #include <type_traits>
 
 
