@@ -16,13 +16,14 @@
 //             publishes, for the rows it owns, negdelta[b,h,t] = -sum_d dO*O and
 //             lse2 = -LSE*log2(e) as f32 in a workspace whose rows are padded to a multiple of
 //             64 per head (lse2 = -inf and negdelta = 0 in the padding, so padded query rows get
-//             probability exactly 0), then sets the block's flag.
+//             probability exactly 0) and its queries scaled by scale*log2(e) as f16 (the
+//             values it and the forward form their scores from), then sets the block's flag.
 //   dK/dV   : a workgroup owns 128 key rows (32 per wave, K^T and V^T held in registers as B
 //             operands) and walks the query blocks at or below the diagonal.  Orientation
 //             S[q,kv] (one key column per lane) so P and dS leave the accumulators directly as
 //             B operands of dV^T += dO^T P and dK^T += Q^T dS; dO^T / Q^T fragments come from
-//             the row-major LDS blocks via ds_read_b64_tr_b16.  It waits for a query block's
-//             rows through the block's flag.
+//             the row-major LDS blocks via ds_read_b64_tr_b16.  The queries it streams are the
+//             dQ role's scaled ones; it waits for a query block's rows through the block's flag.
 // Recomputing S and dP in both roles costs 7 tile GEMMs instead of 5 but keeps every product
 // in registers and needs no dQ accumulation buffer.  Head widths 32 and 64 run two workgroups
 // per CU; head width 128 needs more than 256 registers (213 + 160 accumulation registers) and runs one.

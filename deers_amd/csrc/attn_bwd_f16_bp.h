@@ -14,8 +14,12 @@
 // probabilities (dV, dK, or dQ) and those that produce block n+1's scores (S, dP) between the
 // vector ops of block n, one MFMA per score register: exponential, multiply and the f16 packing
 // ride in the MFMA's shadow.  Nothing else is left on the vector pipe:
-//   * scale*log2(e) is folded into the register-resident f16 operand of the S product (K in the
-//     dK/dV role, Q in the dQ role);
+//   * scale*log2(e) is folded into the f16 queries, once, by the dQ role, which keeps them in
+//     registers and also writes them to the workspace; the dK/dV role streams these scaled
+//     queries (its dK sum is rescaled by ln 2 at the end).  The forward folds the scale into its
+//     queries the same way, so all three kernels exponentiate bit-identical scores: with the
+//     scale folded into K in the dK/dV role instead, its scores differed from the forward's by up
+//     to |S| * 2^-11, a dominant probability by 0.2 %, and dK of a peaked row by 6e-3;
 //   * the S accumulator starts from -LSE*log2(e) and the dP accumulator from -delta (row values
 //     read from LDS straight into the accumulator registers in the dK/dV role, 16-register
 //     constants in the dQ role), so P = exp2(S) and dS = P * dP;
@@ -98,7 +102,8 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   const int T = p.T;
   DEERS_TRACE_POINT(0);  // key block 0 walks the most queries
   const int b_ = bh / p.H, h_ = bh % p.H;
-  const half_t* Q = (const half_t*)p.q + b_ * p.sq.b + h_ * p.sq.h;
+  // the queries as the dQ role scaled them (f16(Q * scale * log2(e)), compact rows)
+  const half_t* Q = (const half_t*)p.qs + (int64_t)bh * p.t_pad * D;
   const half_t* K = (const half_t*)p.k + b_ * p.sk.b + h_ * p.sk.h;
   const half_t* V = (const half_t*)p.v + b_ * p.sv.b + h_ * p.sv.h;
   const half_t* dO = (const half_t*)p.d_o + b_ * p.sdo.b + h_ * p.sdo.h;
@@ -114,7 +119,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   const int n_blk = last_blk - blk0 + 1;                  // query blocks blk0 .. last_blk
   const unsigned edge_span = (unsigned)max(n_blk - wave - 1, 0);  // stages wave+1 .. n_blk-1 need no mask
   const uint32_t lds0 = lds_address(smem);
-  const int sqt = (int)p.sq.t, sdot = (int)p.sdo.t;
+  const int sqt = D, sdot = (int)p.sdo.t;
 
   // ---- this wave's loads of a stage: NLT of the 2 * TB / 1024 tile loads (waves 0 and 1 fetch
   // the Q block, waves 2 and 3 the dO block; a load covers RPW rows) and its two row vectors.
@@ -156,7 +161,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     for (int part = 0; part < LPI; ++part) request_part(part, nb, slot);
   };
 
-  // K^T (scaled) and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.  Rows past
+  // K^T and V^T as B operands: lane holds row kvrow, halfs 16ks+8g .. +7.  Rows past
   // T-1 read row T-1: their keys are masked for every valid query and their rows are not stored.
   half8 kf[KS], vf[KS];
   {
@@ -251,13 +256,6 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
   half8 pf[2], dsf[2];  // P and dS of the previous block as B operands (rows 0-15, 16-31)
   half8 fr[W];          // operand fragments on their way from LDS
   wait_all_vmem();
-  {  // fold scale * log2(e) into K (one rounding to f16)
-    const float c = p.scale_log2;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) kf[ks][e] = (half_t)((float)kf[ks][e] * c);
-  }
   __syncthreads();
 
   // fragment mi of the MFMAs that consume the block in `slot`: (step st, output block db, dV|dK)
@@ -449,7 +447,7 @@ __device__ __forceinline__ void bwd_dkdv_f16_bp_body(const BwdParams& p, int bh,
     half_t* dvrow = dV + (int64_t)kvrow * p.sdv.t;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      store_block_f16(dkrow + 32 * db, dkacc[db], p.scale, g);
+      store_block_f16(dkrow + 32 * db, dkacc[db], kLn2, g);  // sum of dS * Q * scale * log2(e)
       store_block_f16(dvrow + 32 * db, dvacc[db], 1.f, g);
     }
   }
@@ -614,11 +612,16 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
 #pragma unroll
       for (int e = 0; e < 8; ++e) qf[ks][e] = (half_t)((float)qf[ks][e] * c);
   }
-  __syncthreads();
-  // every wave drained its stores of the statistics before this barrier: the rows are in the
-  // XCD's L2, tell the dK/dV workgroups
-  if (tid == 0)
-    __hip_atomic_store(p.ready + (int64_t)bh * n_own + qtile, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // The scaled queries go to the workspace: the dK/dV role forms its scores from these very
+  // values, as the forward did, so that all three exponentiate identical scores (with the
+  // scale folded into K there instead, scores differed by up to |S| * 2^-11 and a dominant
+  // probability by 0.2 %).
+  if (qrow < T) {
+    half_t* qs = (half_t*)p.qs + ((int64_t)bh * p.t_pad + qrow) * D + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) *(half8*)(qs + 16 * ks) = qf[ks];
+  }
+  __syncthreads();  // every wave's first blocks have landed (the stores drain under the first products)
 
   auto fetch2 = [&](int mi, auto slot) -> half8 {  // dQ: (step, output block) = (mi / DB, mi % DB), K^T
     const int st = mi / DB, db = mi % DB;
@@ -712,7 +715,13 @@ __device__ __forceinline__ void bwd_dq_f16_bp_body(const BwdParams& p, int bh, i
   constexpr std::true_type yes{};
   constexpr std::false_type no{};
   DEERS_TRACE_POINT(2);
-  open_stage();
+  // The first stage's barrier doubles as the hand-over: every wave has drained its stores of the
+  // statistics and of the scaled queries before it, the rows are in the XCD's L2, tell the
+  // dK/dV workgroups.
+  wait_all_vmem();
+  __builtin_amdgcn_s_barrier();
+  if (tid == 0)
+    __hip_atomic_store(p.ready + (int64_t)bh * n_own + qtile, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   stage(yes, yes, R - 1, 0, 1, 0, sa, dpa, sb, dpb);
   DEERS_TRACE_POINT(3);
   auto two_stages = [&](auto slot, int n) {  // stages n (odd, ring slot `slot`) and n + 1

@@ -233,9 +233,12 @@ inline bool bwd_dq_short_first(int group_wgs, int capacity) { return 8 * group_w
 struct BwdParams {
   const void* q; const void* k; const void* v; const void* o; const void* d_o;
   const float* lse; float* delta;  // delta: [B,H,T] workspace, rowsum(dO o O)
-  // f16 path workspace, rows padded to a multiple of 64 per head (t_pad):
-  // lse2 = LSE*log2(e) (+inf in the padding), negdelta = -rowsum(dO o O) (0 in the padding)
-  float* lse2; float* negdelta; int t_pad;
+  // f16 path workspace, rows padded to a multiple of 64 per head (t_pad), written by the dQ
+  // role and read by the dK/dV role: lse2 = -LSE*log2(e) (-inf in the padding), negdelta =
+  // -rowsum(dO o O) (0 in the padding), and qs = f16(Q * scale * log2(e)), [B*H][t_pad][D]
+  // compact: the scaled queries the forward and the dQ role form their scores from, so that
+  // all three kernels exponentiate the same scores
+  float* lse2; float* negdelta; void* qs; int t_pad;
   // ready[bh * n_blocks + q_block] == epoch once the lse2 / negdelta rows of that 128-row
   // query block are published (f16 path, hand-over inside one launch); epoch 0: the flags
   // are not used (two launches in stream order).  *error is set to 1 by a workgroup whose

@@ -697,7 +697,9 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   // f16: + 64 floats, the block-pipelined dK/dV role loads row vectors 64 floats at a time
   const size_t ws_floats = dtype == DEERS_ROCM_F16 ? (size_t)(2 * B * H * t_pad + 64) : (size_t)(B * H * T);
   void* ws = nullptr;
-  if (int rc = workspace(ws_floats * sizeof(float), &ws)) return rc;
+  // f16: behind them the dQ role's scaled queries, [B*H][t_pad][D] f16
+  const size_t ws_qs = dtype == DEERS_ROCM_F16 ? (size_t)(B * H * t_pad * D) * 2 : 0;
+  if (int rc = workspace(ws_floats * sizeof(float) + ws_qs, &ws)) return rc;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse;
   p.delta = static_cast<float*>(ws);
   // A launch that is being captured into a graph gets no fresh epoch on replay: it takes the
@@ -736,6 +738,7 @@ int deers_rocm_attn_bwd(int dtype, const void* q, const int64_t* q_strides, cons
   const bool single_launch = !capturing && same_xcd_handover_now();
   p.lse2 = static_cast<float*>(ws);
   p.negdelta = static_cast<float*>(ws) + B * H * t_pad;
+  p.qs = static_cast<float*>(ws) + ws_floats;
   p.t_pad = (int)t_pad;
   p.dq = dq; p.dk = dk; p.dv = dv;
   p.H = (int)H; p.T = (int)T;

@@ -17,7 +17,7 @@
  *    1598-1602).
  *  - The caller owns every buffer it passes.  The library keeps no pointer past
  *    the call and never frees caller memory.  Internal workspace (softmax
- *    statistics of the backward pass, split partial results of decode) is owned
+ *    statistics and scaled queries of the backward pass, split partial results of decode) is owned
  *    and cached by the library.
  *  - Entry points may be called from any thread; they serialise on an internal
  *    mutex.
