@@ -603,7 +603,7 @@ def main():
     # HBM bytes per launch at this shape: rocprofv3 FETCH_SIZE / WRITE_SIZE passes, scaled by
     # what the same counters read for a copy of known size.  A profiler measurement kept in
     # the named file, not taken in this run.
-    measured_traffic = {"attn_bwd_f16": 146.6e6, "attn_fwd_f16": 51.0e6}
+    measured_traffic = {"attn_bwd_f16": 161.4e6, "attn_fwd_f16": 51.0e6}
     roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                 "unit": "TFLOP/s", "frac": (achieved / PEAK_F16_TFLOPS) if achieved else None,
                 "traffic": measured_traffic.get(dom),
