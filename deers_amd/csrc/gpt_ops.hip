@@ -176,9 +176,10 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const T* x, T* y, int
   }
 }
 
-// dx = inv * dy - x * (inv^3 / n) * sum(dy * x)
+// dx = inv * dy - x * (inv^3 / n) * sum(dy * x), plus `addend` where one is given: the
+// gradient is rounded to the storage type before the addition, as a separate add would see it
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const T* x, const T* dy, T* dx,
+__global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const T* x, const T* dy, const T* addend, T* dx,
                                                            int64_t outer, int width, float eps) {
   constexpr int kEpc = 16 / sizeof(T);
   const int lane = threadIdx.x & 63;
@@ -187,6 +188,7 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const T* x, const T* 
   const T* row = x + r * width;
   const T* grow = dy + r * width;
   T* orow = dx + r * width;
+  const T* arow = addend ? addend + r * width : nullptr;
   const float inv = 1.0f / sqrtf(row_sum_prod<T, VEC>(row, row, width, lane) / (float)width + eps);
   const float dot = row_sum_prod<T, VEC>(row, grow, width, lane);
   const float k = dot * inv * inv * inv / (float)width;
@@ -196,10 +198,18 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const T* x, const T* 
       Vec16<T> o;
 #pragma unroll
       for (int e = 0; e < kEpc; ++e) o.e[e] = (T)((float)vg.e[e] * inv - (float)vx.e[e] * k);
+      if (arow) {
+        const Vec16<T> va = load16(arow + c * kEpc);
+#pragma unroll
+        for (int e = 0; e < kEpc; ++e) o.e[e] = (T)((float)va.e[e] + (float)o.e[e]);
+      }
       store16(o, orow + c * kEpc);
     }
   } else {
-    for (int c = lane; c < width; c += 64) orow[c] = (T)((float)grow[c] * inv - (float)row[c] * k);
+    for (int c = lane; c < width; c += 64) {
+      const T g = (T)((float)grow[c] * inv - (float)row[c] * k);
+      orow[c] = arow ? (T)((float)arow[c] + (float)g) : g;
+    }
   }
 }
 
@@ -532,17 +542,17 @@ void launch_index_add(int dtype_f16, const void* src, const int64_t* idx, void* 
 }
 
 template <typename T>
-static void rms_norm_t(const T* x, const T* dy, T* out, int64_t outer, int width, float eps, bool bwd,
-                       hipStream_t stream) {
-  const bool vec = aligned16(x) && aligned16(out) && (!bwd || aligned16(dy)) &&
+static void rms_norm_t(const T* x, const T* dy, const T* addend, T* out, int64_t outer, int width, float eps,
+                       bool bwd, hipStream_t stream) {
+  const bool vec = aligned16(x) && aligned16(out) && (!bwd || aligned16(dy)) && aligned16(addend) &&
                    (width * sizeof(T)) % 16 == 0;
   const dim3 grid((unsigned)((outer + 3) / 4));
   if (bwd) {
     if (vec)
-      hipLaunchKernelGGL((rms_norm_bwd_kernel<T, true>), grid, dim3(256), 0, stream, x, dy, out, outer,
-                         width, eps);
+      hipLaunchKernelGGL((rms_norm_bwd_kernel<T, true>), grid, dim3(256), 0, stream, x, dy, addend, out,
+                         outer, width, eps);
     else
-      hipLaunchKernelGGL((rms_norm_bwd_kernel<T, false>), grid, dim3(256), 0, stream, x, dy, out,
+      hipLaunchKernelGGL((rms_norm_bwd_kernel<T, false>), grid, dim3(256), 0, stream, x, dy, addend, out,
                          outer, width, eps);
   } else {
     if (vec)
@@ -554,13 +564,15 @@ static void rms_norm_t(const T* x, const T* dy, T* out, int64_t outer, int width
   }
 }
 
-void launch_rms_norm(int dtype_f16, const void* x, const void* dy, void* out, int64_t outer, int width,
-                     float eps, int bwd, hipStream_t stream) {
+void launch_rms_norm(int dtype_f16, const void* x, const void* dy, const void* addend, void* out, int64_t outer,
+                     int width, float eps, int bwd, hipStream_t stream) {
   LaunchScope scope(bwd ? "rms_norm_bwd" : "rms_norm_fwd", stream);
   if (dtype_f16)
-    rms_norm_t((const half_t*)x, (const half_t*)dy, (half_t*)out, outer, width, eps, bwd != 0, stream);
+    rms_norm_t((const half_t*)x, (const half_t*)dy, (const half_t*)addend, (half_t*)out, outer, width, eps,
+               bwd != 0, stream);
   else
-    rms_norm_t((const float*)x, (const float*)dy, (float*)out, outer, width, eps, bwd != 0, stream);
+    rms_norm_t((const float*)x, (const float*)dy, (const float*)addend, (float*)out, outer, width, eps,
+               bwd != 0, stream);
 }
 
 template <typename T, bool BWD>

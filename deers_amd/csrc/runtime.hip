@@ -58,8 +58,8 @@ void launch_index_select(int dtype_f16, const void* table, const int64_t* idx, v
                          int64_t n_rows, int64_t n_idx, int width, int* flag, hipStream_t stream);
 void launch_index_add(int dtype_f16, const void* src, const int64_t* idx, void* dst, int64_t n_rows,
                       int64_t n_idx, int width, int* flag, hipStream_t stream);
-void launch_rms_norm(int dtype_f16, const void* x, const void* dy, void* out, int64_t outer, int width,
-                     float eps, int bwd, hipStream_t stream);
+void launch_rms_norm(int dtype_f16, const void* x, const void* dy, const void* addend, void* out, int64_t outer,
+                     int width, float eps, int bwd, hipStream_t stream);
 void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int64_t n, int bwd,
                     hipStream_t stream);
 void launch_argmax_rows(int dtype_f16, const void* x, int64_t* out, int64_t outer, int width,
@@ -1023,7 +1023,7 @@ int deers_rocm_rms_norm_fwd(int dtype, const void* x, void* y, int64_t outer, in
   if (int rc = rows_check("rms_norm_fwd", dtype, outer, inner)) return rc;
   if (outer == 0) return DEERS_ROCM_OK;
   if (!x || !y) return fail(DEERS_ROCM_ERR_ARG, "rms_norm_fwd: null pointer");
-  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, nullptr, y, outer, (int)inner, (float)eps, 0,
+  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, nullptr, nullptr, y, outer, (int)inner, (float)eps, 0,
                          g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
@@ -1036,7 +1036,20 @@ int deers_rocm_rms_norm_bwd(int dtype, const void* x, const void* dy, void* dx, 
   if (int rc = rows_check("rms_norm_bwd", dtype, outer, inner)) return rc;
   if (outer == 0) return DEERS_ROCM_OK;
   if (!x || !dy || !dx) return fail(DEERS_ROCM_ERR_ARG, "rms_norm_bwd: null pointer");
-  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, dy, dx, outer, (int)inner, (float)eps, 1,
+  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, dy, nullptr, dx, outer, (int)inner, (float)eps, 1,
+                         g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_rms_norm_bwd_add(int dtype, const void* x, const void* dy, const void* addend, void* dx,
+                                int64_t outer, int64_t inner, double eps) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = rows_check("rms_norm_bwd_add", dtype, outer, inner)) return rc;
+  if (outer == 0) return DEERS_ROCM_OK;
+  if (!x || !dy || !addend || !dx) return fail(DEERS_ROCM_ERR_ARG, "rms_norm_bwd_add: null pointer");
+  deers::launch_rms_norm(dtype == DEERS_ROCM_F16, x, dy, addend, dx, outer, (int)inner, (float)eps, 1,
                          g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
@@ -1438,6 +1451,7 @@ int deers_rocm_matmul_tune(int on) {
   return DEERS_ROCM_OK;
 }
 
+constexpr size_t kTuneScratchMax = (size_t)256 << 20;  // largest output a tuned product with an addend may have
 constexpr int kSkinnyCounters = 4096;  // column blocks a K-split launch of the few-rows GEMM may have
 
 // The few-rows GEMM on operands skinny_gemm_takes() accepted; prologue 0 none, 1 rms_norm
@@ -1465,19 +1479,25 @@ static int skinny_locked(const void* x, int64_t ldx, const void* w, int64_t ldw,
   return DEERS_ROCM_OK;
 }
 
-// c = a @ b (accumulate = false) or c += a @ b (true); the caller holds g_mu
+// c = a @ b (addend null) or c = a @ b + addend (compact like c; may be c itself); the
+// caller holds g_mu
 static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
-                         const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
-                         int64_t batch, int64_t m, int64_t n, int64_t k, bool accumulate) {
+                         const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, const void* addend,
+                         void* c, int64_t batch, int64_t m, int64_t n, int64_t k) {
   NEED_INIT();
+  const bool accumulate = addend != nullptr;
   if (int rc = check_dtype(dtype)) return rc;
   if (batch < 0 || m < 0 || n < 0 || k < 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX ||
       batch > INT32_MAX)
     return fail(DEERS_ROCM_ERR_ARG, "matmul: sizes must be in [0, 2^31)");
   if (batch == 0 || m == 0 || n == 0) return DEERS_ROCM_OK;
   if (!a || !b || !c) return fail(DEERS_ROCM_ERR_ARG, "matmul: null pointer");
+  const size_t c_bytes = (size_t)(batch * m * n) * (dtype == DEERS_ROCM_F16 ? 2 : 4);
   if (k == 0) {  // empty sum
-    if (accumulate) return DEERS_ROCM_OK;
+    if (accumulate) {
+      if (addend != c) HIP_TRY(hipMemcpyAsync(c, addend, c_bytes, hipMemcpyDeviceToDevice, g_rt.stream));
+      return DEERS_ROCM_OK;
+    }
     deers::launch_fill(dtype == DEERS_ROCM_F16, c, (size_t)(batch * m * n), 0.f, g_rt.stream);
     HIP_TRY(hipGetLastError());
     return DEERS_ROCM_OK;
@@ -1500,7 +1520,7 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
                 (long long)a_rs, (long long)a_cs, (long long)b_rs, (long long)b_cs);
   // a few rows against a weight matrix (a generation step's projections): one streaming
   // pass over the weights instead of a library GEMM
-  if (dtype == DEERS_ROCM_F16 && batch == 1 && !a_t && !b_t &&
+  if (dtype == DEERS_ROCM_F16 && batch == 1 && !a_t && !b_t && (!accumulate || addend == c) &&
       deers::skinny_gemm_takes(m, n, k, lda, ldb, n, a, b, c))
     return skinny_locked(a, lda, b, ldb, c, m, n, k, accumulate, 0, 0.f, false);
   g_rt.skinny_next = deers::SkinnyPrefetch{};  // a pending prefetch hint does not outlive this product
@@ -1517,35 +1537,42 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
   const float alpha = 1.f, beta = accumulate ? 1.f : 0.f;
   const rocblas_operation op_b = b_t ? rocblas_operation_transpose : rocblas_operation_none;
   const rocblas_operation op_a = a_t ? rocblas_operation_transpose : rocblas_operation_none;
-  auto run = [&](int solution) {
+  const void* c_in = accumulate ? addend : c;
+  auto run_into = [&](int solution, void* out) {
     return rocblas_gemm_strided_batched_ex(
         g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
-        (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n, m * n, c,
+        (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c_in, ty, (rocblas_int)n, m * n, out,
         ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
         solution ? rocblas_gemm_algo_solution_index : rocblas_gemm_algo_standard, solution, 0);
   };
+  auto run = [&](int solution) { return run_into(solution, c); };
   int solution = 0;
   if (g_rt.tune_gemm) {
     const std::vector<int64_t> key{dtype, (int64_t)b_t, (int64_t)a_t, n, m, k, ldb, lda, b_bs, a_bs, batch};
     auto hit = g_rt.gemm_choice.find(key);
     if (hit != g_rt.gemm_choice.end()) {
       solution = hit->second;
-    } else if (!accumulate) {  // the trial runs would add into c again and again
-      // Times the default and every listed kernel on the caller's own operands (the
-      // output is overwritten by the real call below): one warm-up and one timed run
-      // each, a second timed run for those within 20 % of the best so far.
+    } else if (!accumulate || c_bytes <= kTuneScratchMax) {
+      // Times the default and every listed kernel on the caller's own operands: one
+      // warm-up and one timed run each, a second timed run for those within 20 % of the
+      // best so far.  A plain product's trial runs write the output the real call below
+      // overwrites; a product with an addend writes its trials into the workspace, since
+      // the addend may be the output itself.
+      void* trial_out = c;
+      if (accumulate)
+        if (int rc = workspace(c_bytes, &trial_out)) return rc;
       rocblas_int count = 0;
       std::vector<rocblas_int> list;
       if (rocblas_gemm_strided_batched_ex_get_solutions(
               g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
-              (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n,
+              (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c_in, ty, (rocblas_int)n,
               m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
               rocblas_gemm_algo_solution_index, 0, nullptr, &count) == rocblas_status_success &&
           count > 0) {
         list.resize(count);
         if (rocblas_gemm_strided_batched_ex_get_solutions(
                 g_rt.blas, op_b, op_a, (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha, b, ty,
-                (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c, ty, (rocblas_int)n,
+                (rocblas_int)ldb, b_bs, a, ty, (rocblas_int)lda, a_bs, &beta, c_in, ty, (rocblas_int)n,
                 m * n, c, ty, (rocblas_int)n, m * n, (rocblas_int)batch, rocblas_datatype_f32_r,
                 rocblas_gemm_algo_solution_index, 0, list.data(), &count) != rocblas_status_success)
           list.clear();
@@ -1555,7 +1582,7 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
       HIP_TRY(hipEventCreate(&e1));
       auto time_one = [&](int sol, float* ms) -> bool {
         HIP_TRY_BOOL(hipEventRecord(e0, g_rt.stream));
-        if (run(sol) != rocblas_status_success) return false;
+        if (run_into(sol, trial_out) != rocblas_status_success) return false;
         HIP_TRY_BOOL(hipEventRecord(e1, g_rt.stream));
         HIP_TRY_BOOL(hipEventSynchronize(e1));
         HIP_TRY_BOOL(hipEventElapsedTime(ms, e0, e1));
@@ -1594,14 +1621,22 @@ int deers_rocm_matmul(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int6
                       const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
                       int64_t batch, int64_t m, int64_t n, int64_t k) {
   std::lock_guard<std::mutex> lock(g_mu);
-  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, batch, m, n, k, false);
+  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, nullptr, c, batch, m, n, k);
 }
 
 int deers_rocm_matmul_acc(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
                           const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, void* c,
                           int64_t batch, int64_t m, int64_t n, int64_t k) {
   std::lock_guard<std::mutex> lock(g_mu);
-  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, batch, m, n, k, true);
+  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, c, c, batch, m, n, k);
+}
+
+int deers_rocm_matmul_add(int dtype, const void* a, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+                          const void* b, int64_t b_rs, int64_t b_cs, int64_t b_bs, const void* addend,
+                          void* c, int64_t batch, int64_t m, int64_t n, int64_t k) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!addend && batch > 0 && m > 0 && n > 0) return fail(DEERS_ROCM_ERR_ARG, "matmul_add: null addend");
+  return matmul_locked(dtype, a, a_rs, a_cs, a_bs, b, b_rs, b_cs, b_bs, addend, c, batch, m, n, k);
 }
 
 int deers_rocm_decode_linear(int dtype, int prologue, float eps, const void* x, int64_t ldx, const void* w,

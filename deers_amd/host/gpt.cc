@@ -29,10 +29,11 @@ MLP::MLP(Tensor up_proj, Tensor down_proj) : up_(std::move(up_proj)), down_(std:
     throw std::logic_error("MLP weights must be [n_embd, hidden] and [hidden, n_embd]");
 }
 
-Tensor MLP::forward(const Tensor& x) const {
+Tensor MLP::forward(const Tensor& x, const Tensor* residual) const {
   if (x.layout().ndim() != 3) throw std::logic_error("MLP expects input shape [B, T, C]");
   const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
   const Tensor y = relu_sq(x.reshape({B * T, C}).matmul(up_));  // [B*T, H]
+  if (residual) return matmul_add(y, down_, residual->reshape({B * T, C})).reshape({B, T, C});
   return y.matmul(down_).reshape({B, T, C});
 }
 
@@ -65,8 +66,10 @@ Block::Block(CausalSelfAttention attn, MLP mlp, double eps)
     : attn_(std::move(attn)), mlp_(std::move(mlp)), eps_(eps) {}
 
 Tensor Block::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const {
-  const Tensor h = x.add(attn_.forward(rms_norm(x, eps_), cos, sin));
-  return h.add(mlp_.forward(rms_norm(h, eps_)));
+  // x + attn(norm(x)) and h + mlp(norm(h)) (src/models/gpt.rs:237-239), each sum riding on
+  // the branch's last product
+  const Tensor h = attn_.forward(rms_norm(x, eps_), cos, sin, &x);
+  return mlp_.forward(rms_norm(h, eps_), &h);
 }
 
 Tensor Block::decode_step(const Tensor& x_t, KvCache& cache, const Tensor& cos, const Tensor& sin,

@@ -27,7 +27,9 @@ class Embedding {
 class MLP {
  public:
   MLP(Tensor up_proj, Tensor down_proj);
-  Tensor forward(const Tensor& x) const;  // [B,T,C] -> [B,T,C]
+  // [B,T,C] -> [B,T,C]; with `residual` the result is residual + mlp(x), the sum riding on the
+  // down projection
+  Tensor forward(const Tensor& x, const Tensor* residual = nullptr) const;
   // residual ([B,T,C], compact) += forward(x), the addition riding on the down projection
   // (inference: the residual's storage is updated in place)
   // With `norm_eps` x is the un-normalised stream and its RMSNorm is folded into the up

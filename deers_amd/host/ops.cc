@@ -1,6 +1,7 @@
 // Operators of the C++ host side; see ops.h for the reference ops each follows.
 #include "ops.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -166,8 +167,10 @@ bool gemm_view(const Tensor& t, int64_t* rs, int64_t* cs, int64_t* bs) {
 }
 }  // namespace
 
-Tensor MatMul::forward(std::unique_ptr<MatMul> self) {
-  Tensor a = self->a_, b = self->b_;
+namespace {
+// a @ b, plus `addend` (compact, the product's shape and type) where one is given, into
+// fresh storage
+Tensor run_product(Tensor a, Tensor b, const Tensor* addend) {
   int64_t ars, acs, abs_, brs, bcs, bbs;
   if (!gemm_view(a, &ars, &acs, &abs_)) { a = a.detach().compact(); gemm_view(a, &ars, &acs, &abs_); }
   if (!gemm_view(b, &brs, &bcs, &bbs)) { b = b.detach().compact(); gemm_view(b, &brs, &bcs, &bbs); }
@@ -179,15 +182,64 @@ Tensor MatMul::forward(std::unique_ptr<MatMul> self) {
   out_shape.push_back(m);
   out_shape.push_back(n);
   Tensor out = empty(out_shape, a.dtype(), backed(a));
-  if (backed(a))
+  if (addend && (!addend->is_compact() || addend->shape() != out_shape || addend->dtype() != a.dtype()))
+    throw std::logic_error("matmul_add: the addend must be a compact tensor of the product's shape and type");
+  if (backed(a) && addend)
+    check(deers_rocm_matmul_add((int)a.dtype(), a.data(), ars, acs, abs_, b.data(), brs, bcs, bbs,
+                                addend->data(), out.data(), batch, m, n, k));
+  else if (backed(a))
     check(deers_rocm_matmul((int)a.dtype(), a.data(), ars, acs, abs_, b.data(), brs, bcs, bbs,
                             out.data(), batch, m, n, k));
+  return out;
+}
+
+// GradientStore::accumulate of the product a @ b (src/backprop.rs:101-112 after
+// src/ops.rs:1089-1101): where `target` already holds a gradient the sum rides on the
+// product, into fresh storage, since another entry may share the held tensor.
+void accumulate_product(GradientStore& grads, const Tensor& target, const Tensor& a, const Tensor& b) {
+  const Tensor* held = grads.get(target.id());
+  if (held && held->is_compact() && held->dtype() == a.dtype() && held->shape().size() == a.shape().size() &&
+      std::equal(held->shape().begin(), held->shape().end() - 2, a.shape().begin()) &&
+      held->shape()[held->shape().size() - 2] == a.shape()[a.shape().size() - 2] &&
+      held->shape().back() == b.shape().back()) {
+    const Tensor addend = *held;
+    grads.insert(target.id(), matmul_add(a, b, addend));
+  } else {
+    grads.accumulate(target, a.matmul(b));
+  }
+}
+}  // namespace
+
+Tensor MatMul::forward(std::unique_ptr<MatMul> self) {
+  const Tensor out = run_product(self->a_, self->b_, nullptr);
   return Tensor(out.storage(), out.layout(), false, std::move(self));
 }
 
 void MatMul::backward(GradientStore& grads, const Tensor& out_grad) const {
-  grads.accumulate(a_, out_grad.matmul(b_.transpose()));
-  grads.accumulate(b_, a_.transpose().matmul(out_grad));
+  accumulate_product(grads, a_, out_grad, b_.transpose());
+  accumulate_product(grads, b_, a_.transpose(), out_grad);
+}
+
+// ---- MatMulAdd ----
+MatMulAdd::MatMulAdd(Tensor a, Tensor b, Tensor c) : a_(std::move(a)), b_(std::move(b)), c_(c.compact()) {
+  const size_t nd = a_.layout().ndim();
+  if (nd < 2 || nd != b_.layout().ndim() || a_.shape()[nd - 1] != b_.shape()[nd - 2])
+    throw std::logic_error("matmul_add: a [..,M,K] and b [..,K,N] of equal rank");
+  for (size_t i = 0; i + 2 < nd; ++i)
+    if (a_.shape()[i] != b_.shape()[i]) throw std::logic_error("matmul_add: batch dimension mismatch");
+  if (a_.dtype() != b_.dtype() || a_.dtype() != c_.dtype()) throw std::logic_error("matmul_add: dtypes differ");
+}
+Tensor MatMulAdd::forward(std::unique_ptr<MatMulAdd> self) {
+  const Tensor out = run_product(self->a_, self->b_, &self->c_);
+  return Tensor(out.storage(), out.layout(), false, std::move(self));
+}
+void MatMulAdd::backward(GradientStore& grads, const Tensor& out_grad) const {
+  grads.accumulate(c_, out_grad);
+  accumulate_product(grads, a_, out_grad, b_.transpose());
+  accumulate_product(grads, b_, a_.transpose(), out_grad);
+}
+Tensor matmul_add(const Tensor& a, const Tensor& b, const Tensor& c) {
+  return MatMulAdd::forward(std::make_unique<MatMulAdd>(a, b, c));
 }
 
 // ---- Tensor conveniences that build ops ----
@@ -299,6 +351,15 @@ void RmsNorm::backward(GradientStore& grads, const Tensor& out_grad) const {
   int64_t outer, inner;
   rows_of(arg_, &outer, &inner);
   Tensor dx = empty(arg_.shape(), arg_.dtype(), backed(arg_));
+  // a gradient the input already holds (the residual branch's) is added in the same pass
+  const Tensor* held = grads.get(arg_.id());
+  if (held && held->is_compact() && held->shape() == arg_.shape() && held->dtype() == arg_.dtype()) {
+    if (backed(arg_))
+      check(deers_rocm_rms_norm_bwd_add((int)arg_.dtype(), arg_.data(), g.data(), held->data(), dx.data(), outer,
+                                        inner, eps_));
+    grads.insert(arg_.id(), dx);
+    return;
+  }
   if (backed(arg_))
     check(deers_rocm_rms_norm_bwd((int)arg_.dtype(), arg_.data(), g.data(), dx.data(), outer, inner, eps_));
   grads.accumulate(arg_, dx);
@@ -574,7 +635,8 @@ CausalSelfAttention::CausalSelfAttention(int64_t n_embd, int64_t n_head, Tensor 
       throw std::logic_error("projection weights must be [n_embd, n_embd]");
 }
 
-Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const {
+Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Tensor& sin,
+                                    const Tensor* residual) const {
   if (x.layout().ndim() != 3) throw std::logic_error("attention expects input shape [B, T, C]");
   const int64_t B = x.shape()[0], T = x.shape()[1], C = x.shape()[2];
   if (C != n_head_ * head_dim_) throw std::logic_error("input channel size must match attention width");
@@ -587,6 +649,8 @@ Tensor CausalSelfAttention::forward(const Tensor& x, const Tensor& cos, const Te
   const Tensor kh = rotary_heads(k, cos, sin);
   const Tensor vh = v.permute({0, 2, 1, 3});           // a view; the kernels read it by stride
   const Tensor y = causal_self_attention(qh, kh, vh).permute({0, 2, 1, 3}).reshape({B * T, C});
+  // the block's `x + attn(..)` (src/models/gpt.rs:237-239) rides on the output projection
+  if (residual) return matmul_add(y, wo_, residual->reshape({B * T, C})).reshape({B, T, C});
   return y.matmul(wo_).reshape({B, T, C});
 }
 

@@ -95,6 +95,22 @@ class MatMul : public TensorOp {
   Tensor a_, b_;
 };
 
+// a @ b + c in one launch: a MatMul followed by an EWiseAdd in the reference (the residual
+// connections of a block, src/models/gpt.rs:237-239); backward as those two ops
+// (src/ops.rs:1089-1101 and the binary add's pass-through).
+class MatMulAdd : public TensorOp {
+ public:
+  MatMulAdd(Tensor a, Tensor b, Tensor c);
+  static Tensor forward(std::unique_ptr<MatMulAdd> self);
+  void backward(GradientStore& grads, const Tensor& out_grad) const override;
+  std::vector<const Tensor*> dependencies() const override { return {&a_, &b_, &c_}; }
+  const char* name() const override { return "MatMulAdd"; }
+
+ private:
+  Tensor a_, b_, c_;  // c_ compacted by the constructor
+};
+Tensor matmul_add(const Tensor& a, const Tensor& b, const Tensor& c);
+
 // y = softmax(q k^T * scale + causal mask) v for q, k, v logical [B,H,T,D] (views
 // welcome: any strides with a unit D stride go to the kernels as they are, other
 // views are compacted first, as FusedLogSoftmax::forward compacts its argument,
@@ -282,7 +298,9 @@ class CausalSelfAttention {
  public:
   CausalSelfAttention(int64_t n_embd, int64_t n_head, Tensor wq, Tensor wk, Tensor wv, Tensor wo);
   // x [B,T,C] with the RoPE tables of precompute_rotary_embeddings -> [B,T,C]
-  Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin) const;
+  // with `residual` ([B,T,C]) the result is residual + attention(x), the sum riding on the
+  // output projection
+  Tensor forward(const Tensor& x, const Tensor& cos, const Tensor& sin, const Tensor* residual = nullptr) const;
   // One generation step (inference, no autograd): x_t [B,1,C] is the token at position
   // cache.len; its rotated key and its value are appended to the cache and the query
   // attends to all cache.len+1 positions through the decode kernel.  Returns [B,1,C],

@@ -288,6 +288,12 @@ def rms_norm_bwd_raw(dtype, x, dy, dx, outer, inner, eps):
                                           ctypes.c_double(eps)))
 
 
+def rms_norm_bwd_add_raw(dtype, x, dy, addend, dx, outer, inner, eps):
+    _check(load().deers_rocm_rms_norm_bwd_add(ctypes.c_int(dtype_code(dtype)), x, dy, addend, dx,
+                                              ctypes.c_int64(outer), ctypes.c_int64(inner),
+                                              ctypes.c_double(eps)))
+
+
 def relu_sq_fwd_raw(dtype, x, y, n):
     _check(load().deers_rocm_relu_sq_fwd(ctypes.c_int(dtype_code(dtype)), x, y, ctypes.c_int64(n)))
 
@@ -416,6 +422,15 @@ def matmul_acc_raw(dtype, a, a_strides, b, b_strides, c, batch, m, n, k):
     _check(load().deers_rocm_matmul_acc(
         ctypes.c_int(dtype_code(dtype)), a, i64(a_strides[0]), i64(a_strides[1]), i64(a_strides[2]),
         b, i64(b_strides[0]), i64(b_strides[1]), i64(b_strides[2]), c, i64(batch), i64(m), i64(n),
+        i64(k)))
+
+
+def matmul_add_raw(dtype, a, a_strides, b, b_strides, addend, c, batch, m, n, k):
+    """deers_rocm_matmul_add: c[batch,m,n] = a @ b + addend; strides are (row, col, batch) in elements."""
+    i64 = ctypes.c_int64
+    _check(load().deers_rocm_matmul_add(
+        ctypes.c_int(dtype_code(dtype)), a, i64(a_strides[0]), i64(a_strides[1]), i64(a_strides[2]),
+        b, i64(b_strides[0]), i64(b_strides[1]), i64(b_strides[2]), addend, c, i64(batch), i64(m), i64(n),
         i64(k)))
 
 

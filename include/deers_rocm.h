@@ -381,6 +381,13 @@ int deers_rocm_rms_norm_fwd(int dtype, const void* x, void* y, int64_t outer, in
                             double eps);
 int deers_rocm_rms_norm_bwd(int dtype, const void* x, const void* dy, void* dx, int64_t outer,
                             int64_t inner, double eps);
+/* dx = addend + rms_norm_bwd(x, dy): RMSNorm's backward followed by GradientStore::accumulate
+ * onto a gradient its input already holds (src/backprop.rs:101-112; in a block, the
+ * residual branch's, src/models/gpt.rs:237-239) in one pass.  The gradient is rounded to
+ * the storage type before the addition: same bits as deers_rocm_rms_norm_bwd followed by
+ * deers_rocm_add.  addend may be dx. */
+int deers_rocm_rms_norm_bwd_add(int dtype, const void* x, const void* dy, const void* addend, void* dx,
+                                int64_t outer, int64_t inner, double eps);
 /* y = relu(x)^2, the MLP activation `y.relu(); &y * &y` (src/models/gpt.rs:196-197), and
  * its backward dx = dy * 2 * relu(x). */
 int deers_rocm_relu_sq_fwd(int dtype, const void* x, void* y, int64_t n);
@@ -474,6 +481,14 @@ int deers_rocm_matmul_acc(int dtype,
                           const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
                           const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
                           void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
+/* c = a @ b + addend, addend compact like c (it may be c: then this is
+ * deers_rocm_matmul_acc).  The out-of-place form serves an autograd graph, where the
+ * addend (the residual stream, or a gradient another consumer also holds) must stay
+ * as it is.  Same rounding as deers_rocm_matmul_acc. */
+int deers_rocm_matmul_add(int dtype,
+                          const void* a, int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride,
+                          const void* b, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
+                          const void* addend, void* c, int64_t batch, int64_t m, int64_t n, int64_t k);
 /* y[m,n] (+)= f(x)[m,k] @ w[k,n] for the few rows of a generation step (m <= 32), f16 only,
  * one streaming pass over w by a kernel of this library; x, w, y row-major with row strides
  * ldx, ldw and n.  `prologue` picks f:

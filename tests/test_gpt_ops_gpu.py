@@ -106,6 +106,29 @@ def test_rms_norm_fwd_bwd(dtype, outer, inner):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("outer,inner", [(1, 3), (5, 48), (7, 191), (33, 768), (3, 4100), (8192, 768)])
+def test_rms_norm_bwd_add_is_the_backward_followed_by_an_add(dtype, outer, inner):
+    """deers_rocm_rms_norm_bwd_add: RMSNorm's backward and the accumulation onto the gradient its
+    input already holds (src/backprop.rs:101-112) in one pass, bit for bit what
+    deers_rocm_rms_norm_bwd followed by the oracle's add gives; the addend stays as it is unless
+    it is the output."""
+    x = synth.normal((outer, inner), synth.tensor_seed(73, "rms", "x"), 2.0).astype(dtype)
+    dy = synth.normal((outer, inner), synth.tensor_seed(73, "rms", "dy"), 1.0).astype(dtype)
+    acc = synth.normal((outer, inner), synth.tensor_seed(73, "rms", "acc"), 1.0).astype(dtype)
+    dx_, dd, da = _dev(x), _dev(dy), _dev(acc)
+    g = rocm.DeviceBuffer((outer, inner), dtype)
+    rocm.rms_norm_bwd_raw(dtype, dx_.ptr, dd.ptr, g.ptr, outer, inner, 1e-5)
+    want = (acc.astype(np.float32) + g.numpy().astype(np.float32)).astype(dtype)
+    out = rocm.DeviceBuffer((outer, inner), dtype)
+    rocm.rms_norm_bwd_add_raw(dtype, dx_.ptr, dd.ptr, da.ptr, out.ptr, outer, inner, 1e-5)
+    assert np.array_equal(out.numpy(), want)
+    assert np.array_equal(da.numpy(), acc)
+    rocm.rms_norm_bwd_add_raw(dtype, dx_.ptr, dd.ptr, da.ptr, da.ptr, outer, inner, 1e-5)
+    assert np.array_equal(da.numpy(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("n,skew", [(1, 0), (5, 0), (4099, 0), (1 << 20, 0), (1000, 1), (1000, 3)])
 def test_relu_sq_is_bit_exact(dtype, n, skew):
     item = np.dtype(dtype).itemsize

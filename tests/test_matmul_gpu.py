@@ -152,6 +152,43 @@ def test_matmul_acc_adds_the_product_into_c(dtype, tol, batch, m, n, k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tune", [False, True])
+@pytest.mark.parametrize("dtype,tol", [(np.float16, None), (np.float32, 1e-4)])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 256, 768, 768), (1, 32, 768, 768), (2, 7, 33, 64), (1, 5, 3, 1)])
+def test_matmul_add_writes_product_plus_addend_elsewhere(dtype, tol, batch, m, n, k, tune):
+    """deers_rocm_matmul_add: c = a @ b + addend with the addend left as it is (the residual
+    stream of src/models/gpt.rs:237-239 inside an autograd graph, or a gradient that another
+    entry of the store shares, src/backprop.rs:101-112), what deers_rocm_matmul_acc gives on a
+    copy of the addend; with the kernel picked by timing as well, whose trial runs must
+    touch neither the addend nor the output's final value; k = 0 copies the addend."""
+    rng = np.random.default_rng(batch * 1000 + m + n)
+    a = rng.standard_normal((batch, m, k)).astype(dtype)
+    b = (rng.standard_normal((batch, k, n)) / np.sqrt(k)).astype(dtype)
+    c0 = rng.standard_normal((batch, m, n)).astype(dtype)
+    da, db, dadd, dacc = (rocm.DeviceBuffer.from_numpy(x) for x in (a, b, c0, c0))
+    dc = rocm.DeviceBuffer((batch, m, n), dtype)
+    rocm.matmul_tune(tune)
+    try:
+        for _ in range(2):  # the second call of a tuned problem takes the remembered kernel
+            rocm.matmul_add_raw(dtype, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dadd.ptr, dc.ptr, batch, m, n, k)
+            assert np.array_equal(dadd.numpy(), c0)
+            want = oracle.matmul(a.astype(np.float32), b.astype(np.float32)) + c0.astype(np.float32)
+            ftol = None if tol is None else tol * max(1.0, float(np.abs(want).max()))
+            assert _close(dc.numpy(), want, dtype, ftol)
+        rocm.matmul_acc_raw(dtype, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dacc.ptr, batch, m, n, k)
+        # (a few f16 rows against a weight matrix accumulate in place on the library's own kernel,
+        # out of place on the BLAS: one rounding either way, not always the same bits)
+        assert _close(dc.numpy(), dacc.numpy().astype(np.float32), dtype, ftol)
+        # the addend may be the output
+        rocm.matmul_add_raw(dtype, da.ptr, (k, 1, m * k), db.ptr, (n, 1, k * n), dadd.ptr, dadd.ptr, batch, m, n, k)
+        assert np.array_equal(dadd.numpy(), dacc.numpy())
+        rocm.matmul_add_raw(dtype, da.ptr, (1, 1, 1), db.ptr, (n, 1, 1), dacc.ptr, dc.ptr, batch, m, n, 0)
+        assert np.array_equal(dc.numpy(), dacc.numpy())
+    finally:
+        rocm.matmul_tune(False)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("m,n,k", [(32, 768, 768), (32, 3072, 768), (32, 768, 3072), (7, 2304, 768),
                                    (1, 768, 256), (32, 776, 512), (5, 8, 256), (31, 40, 1024)])
 def test_few_rows_against_a_weight_matrix_take_the_streaming_kernel(m, n, k):
