@@ -33,6 +33,13 @@
 #include "common.h"
 #include "bwd_delta.h"
 
+// Hooks for a timing harness that includes this file (phase stamps of the one-pass kernel);
+// empty in the library.
+#ifndef DEERS_PHASE
+#define DEERS_PHASE(k)
+#define DEERS_PHASE_STATE
+#endif
+
 namespace deers {
 
 constexpr int kBwd32Blk = 128;
@@ -457,7 +464,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
   const int T = p.T;
   int bh, rank;
   if (!map_block(blockIdx.x, n_items, heads_per_xcd, BH, &bh, &rank)) return;
-  const Bwd32Item it = items[rank];  // items are listed longest first
+  // items are listed longest first; the fields are the same in every lane: held in scalar
+  // registers, so that what derives from them (trip counts, the causal tests) is scalar too
+  Bwd32Item it = items[rank];
+  it.kvblk = __builtin_amdgcn_readfirstlane(it.kvblk);
+  it.tile_begin = __builtin_amdgcn_readfirstlane(it.tile_begin);
+  it.tile_end = __builtin_amdgcn_readfirstlane(it.tile_end);
+  it.shared = __builtin_amdgcn_readfirstlane(it.shared);
   const int kvblk = it.kvblk;
   const int b = bh / p.H, h = bh % p.H;
 
@@ -551,10 +564,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
   const int my_kv = KPW * (wave / DB);  // first key (within the block) of this wave's dQ share
 
   prefetch(first_tile);
+  DEERS_PHASE_STATE;
+  DEERS_PHASE(9);
   for (int j = first_tile; j < n_tiles; ++j) {
     __syncthreads();  // the previous tile's readers (Qs, dOs, dSs) are done
+    DEERS_PHASE(0);
     commit();
+    DEERS_PHASE(1);
     __syncthreads();
+    DEERS_PHASE(2);
     if (j + 1 < n_tiles) prefetch(j + 1);
 
     const int qb0 = j * STEP;
@@ -573,6 +591,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
         }
       }
 
+      DEERS_PHASE(3);
       const bool need_mask = (qb0 < kvw0 + 31);
       float* ds_row = dSs + (32 * wave + (lane & 31)) * LDS_DS + 4 * g;
 #pragma unroll
@@ -594,6 +613,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
         }
         *(floatx4*)(ds_row + 8 * rq) = out;
       }
+      DEERS_PHASE(4);
 
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -607,20 +627,34 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
         }
       }
     }
+    DEERS_PHASE(5);
     __syncthreads();  // scale * dS^T of this tile is complete
+    DEERS_PHASE(6);
 
     // dQ[q, d-block] += sum over this wave's keys of dS[q, kv] K[kv, d]; key sub-blocks
     // whose wave skipped the tile hold no data: only the first live_kv keys do
     {
+      // live keys come in whole 32-key sub-blocks: the products go in runs of 16, each
+      // run's operand reads issued ahead of its MFMAs
       const int live_kv = min(kBwd32Blk, qb0 + 32 - kv0);
-      const int n_pairs = max(0, min(KPW, live_kv - my_kv)) / 2;
+      const int n_runs = max(0, min(KPW, live_kv - my_kv)) / 32;
       floatx16 acc = ZERO16;
       const float* a_p = dSs + (my_kv + g) * LDS_DS + (lane & 31);
       const float* b_p = Ks + (my_kv + g) * LD + 32 * my_db + (lane & 31);
-#pragma unroll 8
-      for (int t = 0; t < n_pairs; ++t)
-        acc = mfma_f32(a_p[2 * t * LDS_DS], b_p[2 * t * LD], acc);
-      if (n_pairs > 0) {
+      for (int run = 0; run < n_runs; ++run) {
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+          acc = mfma_f32(a_p[(32 * run + 2 * t) * LDS_DS], b_p[(32 * run + 2 * t) * LD], acc);
+      }
+      DEERS_PHASE(7);
+      if (n_runs > 0 && qb0 + 32 <= T) {
+        float* dst = dQ + (int64_t)(qb0 + 4 * g) * p.sdq.t + 32 * my_db + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qo = 8 * (r >> 2) + (r & 3);
+          unsafeAtomicAdd(dst + (int64_t)qo * p.sdq.t, acc[r]);
+        }
+      } else if (n_runs > 0) {
         float* dst = dQ + (int64_t)(qb0 + 4 * g) * p.sdq.t + 32 * my_db + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -629,6 +663,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_fused_f32_kernel(
         }
       }
     }
+    DEERS_PHASE(8);
   }
 
   if (it.shared) {
