@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5;
   const int T = p.T;
 
@@ -68,7 +68,9 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
       return;
     }
     for (; item < max_len; ++item) {
-      const int code = lists[(blockIdx.x >> 3) * max_len + item];
+      // the same in every lane: a scalar, so that the trip counts and causal tests that
+      // derive from it are scalar too
+      const int code = __builtin_amdgcn_readfirstlane(lists[(blockIdx.x >> 3) * max_len + item]);
       if (code < 0) return;
       const int head = (code >> 16) * 8 + (blockIdx.x & 7);
       if (head < BH) {
@@ -106,13 +108,15 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
     }
   };
   float qf[KH];
-  auto load_q = [&](const float* Q, int qrow) {  // this lane's half of its query row
+  // this lane's half of its query row, times scale * log2(e): the scores then come out of the
+  // MFMAs in the exponent's base-2 domain
+  auto load_q = [&](const float* Q, int qrow) {
 #pragma unroll
     for (int c = 0; c < KH / 4; ++c) {
       floatx4 t = floatx4{0, 0, 0, 0};
       if (qrow < T) t = *(const floatx4*)(Q + (int64_t)qrow * p.sq.t + g * KH + 4 * c);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) qf[4 * c + e] = t[e];
+      for (int e = 0; e < 4; ++e) qf[4 * c + e] = t[e] * p.scale_log2;
     }
   };
 
@@ -183,19 +187,24 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
                next_qtile * kFwd32BM + 32 * wave + (lane & 31));
       if (!active) continue;
 
-      const bool need_mask = (kv0 + BN - 1 > qw0);
+      // only the tiles on the diagonal pay for the mask: a branch of its own (the empty asm
+      // keeps the compiler from turning it into sixty-four selects on every tile)
+      if (kv0 + BN - 1 > qw0) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kv = kv0 + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (kv > qrow) s[mb][r] = -INFINITY;
+          }
+      }
       float mloc = -INFINITY;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float x = s[mb][r] * p.scale_log2;
-          if (need_mask) {
-            const int kv = kv0 + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (kv > qrow) x = -INFINITY;
-          }
-          s[mb][r] = x;
-          mloc = fmaxf(mloc, x);
+          mloc = fmaxf(mloc, s[mb][r]);
         }
       mloc = fmaxf(mloc, swap32(mloc));
       const float m_new = fmaxf(m, mloc);
