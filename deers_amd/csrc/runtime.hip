@@ -9,6 +9,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -1592,15 +1593,28 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
       float t = 0.f;
       if (!time_one(0, &t) || !time_one(0, &best)) best = 1e30f;  // warm-up, then the default
       list.insert(list.begin(), 0);
+      std::vector<std::pair<float, int>> close{{best, 0}};  // (time, kernel) of the contenders
       for (size_t i = 1; i < list.size(); ++i) {
         float t1 = 0.f, t2 = 0.f;
         if (!time_one(list[i], &t1) || !time_one(list[i], &t1)) continue;  // warm-up, timed
         if (t1 > 1.2f * best) continue;
         if (!time_one(list[i], &t2)) continue;
         const float tt = t1 < t2 ? t1 : t2;
-        if (tt < best) {
-          best = tt;
-          solution = list[i];
+        close.emplace_back(tt, (int)list[i]);
+        if (tt < best) best = tt;
+      }
+      // a single run's time wanders by a few percent, as much as the best kernels differ: the
+      // four fastest are run four more times each and the smallest time decides
+      std::sort(close.begin(), close.end());
+      if (close.size() > 4) close.resize(4);
+      best = 1e30f;
+      for (const auto& cand : close) {
+        float tmin = cand.first;
+        for (int rep = 0; rep < 4; ++rep)
+          if (time_one(cand.second, &t) && t < tmin) tmin = t;
+        if (tmin < best) {
+          best = tmin;
+          solution = cand.second;
         }
       }
       (void)hipEventDestroy(e0);

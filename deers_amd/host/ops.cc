@@ -434,16 +434,27 @@ FusedCausalAttention::FusedCausalAttention(Tensor q, Tensor k, Tensor v, double 
     throw std::logic_error("FusedCausalAttention: dtypes differ");
 }
 
+namespace {
+// Logical [B,H,T,D] over fresh [B,T,H,D] memory.
+Tensor heads_interleaved(int64_t B, int64_t H, int64_t T, int64_t D, DType dtype) {
+  const Tensor bthd = empty({B, T, H, D}, dtype, true);
+  return Tensor(bthd.storage(), bthd.layout().permute({0, 2, 1, 3}), false, nullptr);
+}
+}  // namespace
+
 Tensor FusedCausalAttention::forward(std::unique_ptr<FusedCausalAttention> self) {
   if (!fused_kernels_take(self->q_.shape()[3])) return forward_composed(std::move(self));
   const Tensor q = kernel_ready(self->q_), k = kernel_ready(self->k_), v = kernel_ready(self->v_);
   const auto& s = q.shape();
   const int64_t B = s[0], H = s[1], T = s[2], D = s[3];
-  Tensor o = empty(s, q.dtype(), true);
+  // The heads are written interleaved, [B,T,H,D] in memory under the logical [B,H,T,D]: the
+  // module's `y.permute([0,2,1,3]).reshape([B*T, C])` (src/models/gpt.rs:145) is then a view
+  // of compact memory and costs no copy.
+  const Tensor o = heads_interleaved(B, H, T, D, q.dtype());
   Tensor lse = empty({B, H, T}, DType::F32, true);
   check(deers_rocm_attn_fwd((int)q.dtype(), q.data(), q.layout().strides.data(), k.data(),
                             k.layout().strides.data(), v.data(), v.layout().strides.data(), o.data(),
-                            nullptr, (float*)lse.data(), B, H, T, D, (float)self->scale_));
+                            o.layout().strides.data(), (float*)lse.data(), B, H, T, D, (float)self->scale_));
   self->saved_o_ = o;
   self->saved_lse_ = lse;
   return Tensor(o.storage(), o.layout(), false, std::move(self));
@@ -545,12 +556,16 @@ void FusedCausalAttention::backward(GradientStore& grads, const Tensor& out_grad
   const Tensor g = kernel_ready(out_grad);
   const auto& s = q.shape();
   const int64_t B = s[0], H = s[1], T = s[2], D = s[3];
-  Tensor dq = empty(s, q.dtype(), true), dk = empty(s, q.dtype(), true), dv = empty(s, q.dtype(), true);
+  Tensor dq = empty(s, q.dtype(), true), dk = empty(s, q.dtype(), true);
+  // v usually is the permuted view of a [B,T,H,D] projection: its gradient is written in the
+  // same memory order, so that the permute's and the reshape's backward are views too
+  const bool v_interleaved = v.layout().strides[1] == D && v.layout().strides[2] == H * D;
+  const Tensor dv = v_interleaved ? heads_interleaved(B, H, T, D, q.dtype()) : empty(s, q.dtype(), true);
   check(deers_rocm_attn_bwd((int)q.dtype(), q.data(), q.layout().strides.data(), k.data(),
                             k.layout().strides.data(), v.data(), v.layout().strides.data(),
-                            saved_o_.data(), nullptr, (const float*)saved_lse_.data(), g.data(),
-                            g.layout().strides.data(), dq.data(), nullptr, dk.data(), nullptr,
-                            dv.data(), nullptr, B, H, T, D, (float)scale_));
+                            saved_o_.data(), saved_o_.layout().strides.data(), (const float*)saved_lse_.data(),
+                            g.data(), g.layout().strides.data(), dq.data(), nullptr, dk.data(), nullptr,
+                            const_cast<void*>(dv.data()), dv.layout().strides.data(), B, H, T, D, (float)scale_));
   grads.accumulate(q_, dq);
   grads.accumulate(k_, dk);
   grads.accumulate(v_, dv);

@@ -114,9 +114,10 @@ Tensor matmul_add(const Tensor& a, const Tensor& b, const Tensor& c);
 // y = softmax(q k^T * scale + causal mask) v for q, k, v logical [B,H,T,D] (views
 // welcome: any strides with a unit D stride go to the kernels as they are, other
 // views are compacted first, as FusedLogSoftmax::forward compacts its argument,
-// src/ops.rs:1205).  Returns a compact [B,H,T,D] tensor and keeps (O, LSE) for the
-// backward, which overwrites fresh dq/dk/dv buffers and hands them to
-// GradientStore::accumulate.
+// src/ops.rs:1205).  Returns a [B,H,T,D] tensor whose memory is [B,T,H,D], so that the
+// module's permute + reshape (src/models/gpt.rs:145) is a view, and keeps (O, LSE) for the
+// backward, which overwrites fresh dq/dk/dv buffers (dv in v's memory order) and hands
+// them to GradientStore::accumulate.
 // Head widths the fused kernels do not take (they take 32, 64, 128; the reference's own GPT
 // test runs head_dim 2, tests/gpt.rs:38-49) go through the reference's op chain on the
 // device instead, kernel by kernel (src/models/gpt.rs:139-144 forward; the backward bodies of
