@@ -109,14 +109,16 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
   };
   float qf[KH];
   // this lane's half of its query row, times scale * log2(e): the scores then come out of the
-  // MFMAs in the exponent's base-2 domain
+  // MFMAs in the exponent's base-2 domain (head width 128 scales the scores instead: with
+  // 64 query registers scaled in place its 256 registers no longer suffice)
+  constexpr bool kScaledQ = D != 128;
   auto load_q = [&](const float* Q, int qrow) {
 #pragma unroll
     for (int c = 0; c < KH / 4; ++c) {
       floatx4 t = floatx4{0, 0, 0, 0};
       if (qrow < T) t = *(const floatx4*)(Q + (int64_t)qrow * p.sq.t + g * KH + 4 * c);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) qf[4 * c + e] = t[e] * p.scale_log2;
+      for (int e = 0; e < 4; ++e) qf[4 * c + e] = kScaledQ ? t[e] * p.scale_log2 : t[e];
     }
   };
 
@@ -187,9 +189,12 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
                next_qtile * kFwd32BM + 32 * wave + (lane & 31));
       if (!active) continue;
 
-      // only the tiles on the diagonal pay for the mask: a branch of its own (the empty asm
-      // keeps the compiler from turning it into sixty-four selects on every tile)
-      if (kv0 + BN - 1 > qw0) {
+      // At head width 64 only the tiles on the diagonal pay for the mask: a branch of its own
+      // (the empty asm keeps the compiler from turning it into sixty-four selects on every
+      // tile).  The other widths have no registers to spare for it and keep the selects.
+      constexpr bool kMaskBranch = D == 64;
+      const bool need_mask = kv0 + BN - 1 > qw0;
+      if (kMaskBranch && need_mask) {
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -204,6 +209,11 @@ __global__ __launch_bounds__(256, (D == 32 ? 3 : 2)) void attn_fwd_f32_kernel(Fw
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
+          if (!kMaskBranch && need_mask) {
+            const int kv = kv0 + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (kv > qrow) s[mb][r] = -INFINITY;
+          }
+          if (!kScaledQ) s[mb][r] *= p.scale_log2;
           mloc = fmaxf(mloc, s[mb][r]);
         }
       mloc = fmaxf(mloc, swap32(mloc));
