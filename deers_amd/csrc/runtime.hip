@@ -1581,14 +1581,17 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
       hipEvent_t e0, e1;
       HIP_TRY(hipEventCreate(&e0));
       HIP_TRY(hipEventCreate(&e1));
-      auto time_one = [&](int sol, float* ms) -> bool {
+      auto time_runs = [&](int sol, int runs, float* ms) -> bool {  // mean of back-to-back launches
         HIP_TRY_BOOL(hipEventRecord(e0, g_rt.stream));
-        if (run_into(sol, trial_out) != rocblas_status_success) return false;
+        for (int i = 0; i < runs; ++i)
+          if (run_into(sol, trial_out) != rocblas_status_success) return false;
         HIP_TRY_BOOL(hipEventRecord(e1, g_rt.stream));
         HIP_TRY_BOOL(hipEventSynchronize(e1));
         HIP_TRY_BOOL(hipEventElapsedTime(ms, e0, e1));
+        *ms /= (float)runs;
         return true;
       };
+      auto time_one = [&](int sol, float* ms) -> bool { return time_runs(sol, 1, ms); };
       float best = 0.f;
       float t = 0.f;
       if (!time_one(0, &t) || !time_one(0, &best)) best = 1e30f;  // warm-up, then the default
@@ -1604,19 +1607,17 @@ static int matmul_locked(int dtype, const void* a, int64_t a_rs, int64_t a_cs, i
         if (tt < best) best = tt;
       }
       // a single run's time wanders by a few percent, as much as the best kernels differ: the
-      // four fastest are run four more times each and the smallest time decides
+      // four fastest go again, eight back-to-back launches between one pair of events, three
+      // times over, and the smallest mean decides
       std::sort(close.begin(), close.end());
       if (close.size() > 4) close.resize(4);
       best = 1e30f;
-      for (const auto& cand : close) {
-        float tmin = cand.first;
-        for (int rep = 0; rep < 4; ++rep)
-          if (time_one(cand.second, &t) && t < tmin) tmin = t;
-        if (tmin < best) {
-          best = tmin;
-          solution = cand.second;
-        }
-      }
+      for (int round = 0; round < 3; ++round)
+        for (const auto& cand : close)
+          if (time_runs(cand.second, 8, &t) && t < best) {
+            best = t;
+            solution = cand.second;
+          }
       (void)hipEventDestroy(e0);
       (void)hipEventDestroy(e1);
       g_rt.gemm_choice[key] = solution;
