@@ -176,6 +176,40 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const T* x, T* y, int
   }
 }
 
+// The forward for rows of at most 64 * RES 16-byte chunks (aligned): the row stays in the
+// wave's registers between the sum of squares and the scaling.  Same bits as the general kernel.
+template <typename T, int RES>
+__global__ __launch_bounds__(256) void rms_norm_fwd_resident_kernel(const T* x, T* y, int64_t outer, int width,
+                                                                    float eps) {
+  constexpr int kEpc = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= outer) return;
+  const T* row = x + r * width;
+  T* orow = y + r * width;
+  const int n_chunks = width / kEpc;
+  Vec16<T> v[RES];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < RES; ++i) {
+    const int c = lane + 64 * i;
+    if (c < n_chunks) {
+      v[i] = load16(row + c * kEpc);
+#pragma unroll
+      for (int e = 0; e < kEpc; ++e) s = fmaf((float)v[i].e[e], (float)v[i].e[e], s);
+    }
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(s) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < RES; ++i) {
+    const int c = lane + 64 * i;
+    if (c >= n_chunks) continue;
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) v[i].e[e] = (T)((float)v[i].e[e] * inv);
+    store16(v[i], orow + c * kEpc);
+  }
+}
+
 // dx = inv * dy - x * (inv^3 / n) * sum(dy * x), plus `addend` where one is given: the
 // gradient is rounded to the storage type before the addition, as a separate add would see it
 template <typename T, bool VEC>
@@ -210,6 +244,62 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const T* x, const T* 
       const T g = (T)((float)grow[c] * inv - (float)row[c] * k);
       orow[c] = arow ? (T)((float)arow[c] + (float)g) : g;
     }
+  }
+}
+
+// The same for rows of at most 64 * RES 16-byte chunks (aligned): a wave keeps its row of x
+// and dy in registers, so each is read once instead of three and two times.  Sums run in
+// the order of the general kernel: same bits.
+template <typename T, int RES>
+__global__ __launch_bounds__(256) void rms_norm_bwd_resident_kernel(const T* x, const T* dy, const T* addend,
+                                                                    T* dx, int64_t outer, int width, float eps) {
+  constexpr int kEpc = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= outer) return;
+  const T* row = x + r * width;
+  const T* grow = dy + r * width;
+  T* orow = dx + r * width;
+  const T* arow = addend ? addend + r * width : nullptr;
+  const int n_chunks = width / kEpc;
+  Vec16<T> vx[RES], vg[RES];
+#pragma unroll
+  for (int i = 0; i < RES; ++i) {
+    const int c = lane + 64 * i;
+    if (c < n_chunks) {
+      vx[i] = load16(row + c * kEpc);
+      vg[i] = load16(grow + c * kEpc);
+    } else {
+#pragma unroll
+      for (int e = 0; e < kEpc; ++e) {
+        vx[i].e[e] = (T)0.f;
+        vg[i].e[e] = (T)0.f;
+      }
+    }
+  }
+  float sxx = 0.f, sxg = 0.f;
+#pragma unroll
+  for (int i = 0; i < RES; ++i)
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) {
+      sxx = fmaf((float)vx[i].e[e], (float)vx[i].e[e], sxx);
+      sxg = fmaf((float)vx[i].e[e], (float)vg[i].e[e], sxg);
+    }
+  const float inv = 1.0f / sqrtf(wave_sum(sxx) / (float)width + eps);
+  const float k = wave_sum(sxg) * inv * inv * inv / (float)width;
+#pragma unroll
+  for (int i = 0; i < RES; ++i) {
+    const int c = lane + 64 * i;
+    if (c >= n_chunks) continue;
+    Vec16<T> o;
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) o.e[e] = (T)((float)vg[i].e[e] * inv - (float)vx[i].e[e] * k);
+    if (arow) {
+      const Vec16<T> va = load16(arow + c * kEpc);
+#pragma unroll
+      for (int e = 0; e < kEpc; ++e) o.e[e] = (T)((float)va.e[e] + (float)o.e[e]);
+    }
+    store16(o, orow + c * kEpc);
   }
 }
 
@@ -547,13 +637,20 @@ static void rms_norm_t(const T* x, const T* dy, const T* addend, T* out, int64_t
   const bool vec = aligned16(x) && aligned16(out) && (!bwd || aligned16(dy)) && aligned16(addend) &&
                    (width * sizeof(T)) % 16 == 0;
   const dim3 grid((unsigned)((outer + 3) / 4));
-  if (bwd) {
+  constexpr int kResident = 4;  // 16-byte chunks per lane the resident backward holds of x and of dy
+  if (bwd && vec && width / (int)(16 / sizeof(T)) <= 64 * kResident) {
+    hipLaunchKernelGGL((rms_norm_bwd_resident_kernel<T, kResident>), grid, dim3(256), 0, stream, x, dy, addend,
+                       out, outer, width, eps);
+  } else if (bwd) {
     if (vec)
       hipLaunchKernelGGL((rms_norm_bwd_kernel<T, true>), grid, dim3(256), 0, stream, x, dy, addend, out,
                          outer, width, eps);
     else
       hipLaunchKernelGGL((rms_norm_bwd_kernel<T, false>), grid, dim3(256), 0, stream, x, dy, addend, out,
                          outer, width, eps);
+  } else if (vec && width / (int)(16 / sizeof(T)) <= 64 * kResident) {
+    hipLaunchKernelGGL((rms_norm_fwd_resident_kernel<T, kResident>), grid, dim3(256), 0, stream, x, out, outer,
+                       width, eps);
   } else {
     if (vec)
       hipLaunchKernelGGL((rms_norm_fwd_kernel<T, true>), grid, dim3(256), 0, stream, x, out, outer,
