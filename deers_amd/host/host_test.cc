@@ -147,9 +147,45 @@ static void test_backward_accumulates_diamond_grads() {
   std::printf("ok backward_accumulates_diamond_grads\n");
 }
 
+// matmul_add(a, b, c) against a.matmul(b).add(c): values and all three gradients; a is used by
+// two products, so its second gradient rides on a product as well (accumulate of a MatMul's
+// gradient onto one the store already holds, src/backprop.rs:101-112).
+static void test_matmul_add_matches_matmul_then_add() {
+  const int64_t M = 6, K = 8, N = 5;
+  std::vector<float> ha(M * K), hb(K * N), hc(M * N), hb2(K * N);
+  for (size_t i = 0; i < ha.size(); ++i) ha[i] = 0.25f * (float)((int)(i * 7 % 11) - 5);
+  for (size_t i = 0; i < hb.size(); ++i) hb[i] = 0.5f * (float)((int)(i * 5 % 7) - 3);
+  for (size_t i = 0; i < hb2.size(); ++i) hb2[i] = 0.125f * (float)((int)(i * 3 % 13) - 6);
+  for (size_t i = 0; i < hc.size(); ++i) hc[i] = (float)((int)(i % 9) - 4);
+  std::vector<std::vector<float>> got[2];
+  for (int fused = 0; fused < 2; ++fused) {
+    Tensor a = Tensor::from_host(ha.data(), {M, K}, DType::F32).attach();
+    Tensor b = Tensor::from_host(hb.data(), {K, N}, DType::F32).attach();
+    Tensor b2 = Tensor::from_host(hb2.data(), {K, N}, DType::F32).attach();
+    Tensor c = Tensor::from_host(hc.data(), {M, N}, DType::F32).attach();
+    const Tensor y = fused ? matmul_add(a, b, c) : a.matmul(b).add(c);
+    const Tensor z = y.add(a.matmul(b2));  // a second product through a
+    GradientStore grads = z.backward();
+    std::vector<float> hy(M * N);
+    y.to_host(hy.data());
+    got[fused].push_back(hy);
+    for (const Tensor* t : {&a, &b, &b2, &c}) {
+      const Tensor* g = grads.get(t->id());
+      EXPECT(g != nullptr && g->shape() == t->shape());
+      std::vector<float> hg(t->layout().size(), -1.f);
+      if (g) g->to_host(hg.data());
+      got[fused].push_back(hg);
+    }
+  }
+  for (size_t k = 0; k < got[0].size(); ++k)
+    for (size_t i = 0; i < got[0][k].size(); ++i) EXPECT(got[0][k][i] == got[1][k][i]);  // small integers over 8: exact
+  std::printf("ok matmul_add_matches_matmul_then_add\n");
+}
+
 static int run_gpu(const std::string& dir) {
   check(deers_rocm_init(0));
   test_backward_accumulates_diamond_grads();
+  test_matmul_add_matches_matmul_then_add();
 
   // case.txt: dtype B H T D L   (dtype 0 = f16, 1 = f32; L = decode cache length or 0)
   int dt, B, H, T, D, L;
