@@ -55,6 +55,7 @@ def test_host_fused_attention_matches_oracle(tmp_path, dtype, B, H, T, D, L, tol
     r = _run("gpu", str(tmp_path))
     assert r.returncode == 0, r.stdout + r.stderr
     assert "ok backward_accumulates_diamond_grads" in r.stdout and "all passed" in r.stdout
+    assert "ok matmul_add_matches_matmul_then_add" in r.stdout
 
     def out(name, shape=(B, T, H, D)):
         return np.fromfile(tmp_path / name, dtype=dtype).reshape(shape).astype(np.float64)
