@@ -21,6 +21,10 @@
 //      softmax's vector ops, and the rate of MFMAs chained through one accumulator
 //   P  a bare MFMA stream again, on operands of zeros, a constant, and random values: the
 //      device is power limited and the clock it sustains depends on the data
+//   Q  v_mfma_f32_32x32x2_f32 (the f32 attention kernels' instruction) with every A operand
+//      read from LDS, 1..8 reads in flight, through one or four accumulation chains, at one and
+//      two waves per SIMD: whether a chain of dependent products or an LDS read per product
+//      slows the pipe
 //
 // Every launch covers all CUs (256 workgroups x waves); times are clock64() deltas from the
 // common start of a CU's waves to the end of its slowest wave, averaged over the CUs, so
@@ -755,12 +759,84 @@ static void run_mfma_data() {
   CK(hipFree(src));
 }
 
+// ---- Q: f32 MFMA, A operand from LDS, AHEAD reads in flight, NCHAIN accumulators ----
+template <int AHEAD, int NCHAIN>
+__global__ void mfma_f32_lds_kernel(float* out, const float* in, int iters) {
+  __shared__ float lds[64 * 68];
+  for (int i = threadIdx.x; i < 64 * 68; i += blockDim.x) lds[i] = in[i & 1023];
+  __syncthreads();
+  floatx16 acc[NCHAIN];
+  for (int c = 0; c < NCHAIN; ++c)
+    for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+  const float b = in[threadIdx.x & 63];
+  const float* base = lds + (threadIdx.x & 31) + 4 * 68 * ((threadIdx.x >> 5) & 1);
+  for (int it = 0; it < iters; ++it) {
+    float a[AHEAD];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) a[u] = base[(u % 8) * 68 * 8 + (u / 8)];
+#pragma unroll
+    for (int u = 0; u < 64; ++u) {
+      const float cur = a[u % AHEAD];
+      if (u + AHEAD < 64) a[u % AHEAD] = base[((u + AHEAD) % 8) * 68 * 8 + ((u + AHEAD) / 8)];
+      acc[u % NCHAIN] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur, b, acc[u % NCHAIN], 0, 0, 0);
+    }
+  }
+  float s = 0.f;
+  for (int c = 0; c < NCHAIN; ++c)
+    for (int i = 0; i < 16; ++i) s += acc[c][i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+template <int AHEAD, int NCHAIN>
+static void run_mfma_f32_lds_one(int threads, const float* in) {
+  const int iters = 400;
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  mfma_f32_lds_kernel<AHEAD, NCHAIN><<<256, threads>>>(g_out, in, iters);
+  CK(hipEventRecord(e0));
+  mfma_f32_lds_kernel<AHEAD, NCHAIN><<<256, threads>>>(g_out, in, iters);
+  CK(hipEventRecord(e1));
+  CK(hipEventSynchronize(e1));
+  float ms;
+  CK(hipEventElapsedTime(&ms, e0, e1));
+  const double per_simd = (double)iters * 64 * (threads / 256);
+  std::printf("Q  f32 MFMA, A from LDS: %d reads in flight, %d chain(s), %d wave(s)/SIMD: %5.1f ns per MFMA per SIMD "
+              "(64 clocks at 2.4 GHz = 26.7), %6.1f TFLOP/s\n",
+              AHEAD, NCHAIN, threads / 256, ms * 1e6 / per_simd, 1024.0 * per_simd * 4096 / (ms * 1e-3) * 1e-12);
+  CK(hipEventDestroy(e0));
+  CK(hipEventDestroy(e1));
+}
+
+static void run_mfma_f32_lds() {
+  float* in;
+  CK(hipMalloc(&in, 4096));
+  float h[1024];
+  for (int i = 0; i < 1024; ++i) h[i] = 0.001f * ((i * 37) % 101 - 50);
+  CK(hipMemcpy(in, h, 4096, hipMemcpyHostToDevice));
+  for (int rep = 0; rep < 2; ++rep) {  // the first round also brings the clocks up
+    run_mfma_f32_lds_one<1, 4>(256, in);
+    run_mfma_f32_lds_one<2, 4>(256, in);
+    run_mfma_f32_lds_one<8, 4>(256, in);
+    run_mfma_f32_lds_one<2, 1>(256, in);
+    run_mfma_f32_lds_one<1, 4>(512, in);
+    run_mfma_f32_lds_one<2, 4>(512, in);
+    run_mfma_f32_lds_one<8, 4>(512, in);
+    run_mfma_f32_lds_one<2, 1>(512, in);
+  }
+  CK(hipFree(in));
+}
+
 int main() {
   CK(hipMalloc(&g_out, 1024 * 1024 * sizeof(float)));
   CK(hipMalloc(&g_clk, 256 * 16 * sizeof(long long)));
   if (getenv("MICROBENCH_ONLY_P")) {
     run_mfma_data();
     run_mfma_f32_data();
+    return 0;
+  }
+  if (getenv("MICROBENCH_ONLY_Q")) {
+    run_mfma_f32_lds();
     return 0;
   }
   if (getenv("MICROBENCH_ONLY_F")) {
@@ -811,5 +887,6 @@ int main() {
   run_chunk<8>("exp, mul, cvt_pk, ds_read_b128");
   run_reuse<1, false>(); run_reuse<2, false>(); run_reuse<1, true>(); run_reuse<2, true>();
   run_chain<1>(); run_chain<2>(); run_chain<4>();
+  run_mfma_f32_lds();
   return 0;
 }
