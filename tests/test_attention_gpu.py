@@ -116,6 +116,16 @@ def test_peaked_rows_and_consistent_scores():
     check_case(x, 5e-3, "peaked rows B5 H15 T914 D32", heads=[0, 4])
 
 
+def test_first_key_rows_stay_inside_the_contract():
+    """The rows of dK with the longest sums: the first key of a head takes a term from every query.
+    Found by a random sweep as the case closest to the bar (dK of key 0 of one head 4.99e-3 off at
+    a value of -2.95: 640 products of f16-rounded dS and scaled queries).  The kernels are
+    bit-reproducible, so this reads the same on every device: a guard against a change that
+    rounds once more on the way to dK."""
+    x = synth.attention_inputs("stress-58", 4, 8, 640, 32, np.float16, base_seed=158)
+    check_case(x, 5e-3, "first-key rows B4 H8 T640 D32", heads=[0])
+
+
 def test_config1_f32_full():
     """B=4 H=6 T=256 D=32 f32: the reference's own CPU-runnable case."""
     x = synth.attention_inputs("c1", 4, 6, 256, 32, np.float32, base_seed=0)
