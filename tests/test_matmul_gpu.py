@@ -189,6 +189,44 @@ def test_matmul_add_writes_product_plus_addend_elsewhere(dtype, tol, batch, m, n
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float16, None), (np.float32, 1e-4)])
+def test_matmul_add_takes_transposed_and_broadcast_operands(dtype, tol):
+    """The gradient products that carry an addend read views: out_grad @ w^T with w^T the
+    transposed view of a weight (MatMul::backward, src/ops.rs:1089-1101), x^T @ out_grad with x^T
+    a transposed view, and a batch of left operands against one broadcast right operand
+    (batch stride 0).  Same operand rules as deers_rocm_matmul."""
+    rng = np.random.default_rng(99)
+    m, n, k, batch = 96, 40, 64, 3
+    # b^T: the weight is stored [n, k]; the product reads it as [k, n] through strides (1, k)
+    a = rng.standard_normal((1, m, k)).astype(dtype)
+    w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(dtype)
+    c0 = rng.standard_normal((1, m, n)).astype(dtype)
+    da, dw, dadd = (rocm.DeviceBuffer.from_numpy(x) for x in (a, w, c0))
+    dc = rocm.DeviceBuffer((1, m, n), dtype)
+    rocm.matmul_add_raw(dtype, da.ptr, (k, 1, 0), dw.ptr, (1, k, 0), dadd.ptr, dc.ptr, 1, m, n, k)
+    want = oracle.matmul(a.astype(np.float32), w.T[None].astype(np.float32)) + c0.astype(np.float32)
+    assert _close(dc.numpy(), want, dtype, None if tol is None else tol * max(1.0, float(np.abs(want).max())))
+    # a^T: x stored [m, k] read as [k, m]; x^T @ g + addend, a weight gradient onto a held one
+    g = (rng.standard_normal((1, m, n)) / np.sqrt(m)).astype(dtype)
+    acc = rng.standard_normal((1, k, n)).astype(dtype)
+    dg, dacc = rocm.DeviceBuffer.from_numpy(g), rocm.DeviceBuffer.from_numpy(acc)
+    dout = rocm.DeviceBuffer((1, k, n), dtype)
+    rocm.matmul_add_raw(dtype, da.ptr, (1, k, 0), dg.ptr, (n, 1, 0), dacc.ptr, dout.ptr, 1, k, n, m)
+    want = oracle.matmul(a[0].T[None].astype(np.float32), g.astype(np.float32)) + acc.astype(np.float32)
+    assert _close(dout.numpy(), want, dtype, None if tol is None else tol * max(1.0, float(np.abs(want).max())))
+    assert np.array_equal(dacc.numpy(), acc)
+    # a batch of left operands against one right operand (batch stride 0)
+    ab = rng.standard_normal((batch, m, k)).astype(dtype)
+    b1 = (rng.standard_normal((1, k, n)) / np.sqrt(k)).astype(dtype)
+    cb = rng.standard_normal((batch, m, n)).astype(dtype)
+    dab, db1, dcb = (rocm.DeviceBuffer.from_numpy(x) for x in (ab, b1, cb))
+    dob = rocm.DeviceBuffer((batch, m, n), dtype)
+    rocm.matmul_add_raw(dtype, dab.ptr, (k, 1, m * k), db1.ptr, (n, 1, 0), dcb.ptr, dob.ptr, batch, m, n, k)
+    want = oracle.matmul(ab.astype(np.float32), np.broadcast_to(b1, (batch, k, n)).astype(np.float32)) + cb.astype(np.float32)
+    assert _close(dob.numpy(), want, dtype, None if tol is None else tol * max(1.0, float(np.abs(want).max())))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("m,n,k", [(32, 768, 768), (32, 3072, 768), (32, 768, 3072), (7, 2304, 768),
                                    (1, 768, 256), (32, 776, 512), (5, 8, 256), (31, 40, 1024)])
 def test_few_rows_against_a_weight_matrix_take_the_streaming_kernel(m, n, k):
