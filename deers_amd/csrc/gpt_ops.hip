@@ -365,11 +365,24 @@ __device__ __forceinline__ void merge_ms(float& m, float& s, float m2, float s2)
   m = mn;
 }
 
+// MODE 0: the forward.  MODE 1 and 2 also write dlogits[r, c] = (exp(x - lse) - [c == target]) *
+// inv_n, the gradient of the mean loss for an upstream gradient of one: same expression, same
+// bits as cross_entropy_bwd_kernel's.  In MODE 2 the workgroup keeps the whole row in registers
+// between the reduction and the gradient (rows of up to kCeThreads * ce_keep<T>() 16-byte chunks:
+// 57344 floats or 65536 halves), so the logits are read once; MODE 1 walks longer rows a second
+// time.  The reduction takes the chunks in the same groups and order in every mode: same lse,
+// same loss.
 template <typename T>
+constexpr int ce_keep() {  // chunks per thread MODE 2 holds (a multiple of kCeInFlight)
+  return sizeof(T) == 2 ? 16 : 28;
+}
+
+template <typename T, int MODE>
 __global__ __launch_bounds__(kCeThreads) void cross_entropy_fwd_kernel(
-    const T* logits, const int64_t* targets, float* row_lse, float* row_loss, int width,
-    int* error_flag) {
+    const T* logits, const int64_t* targets, float* row_lse, float* row_loss, T* dlogits, float inv_n,
+    int width, int* error_flag) {
   __shared__ float red_m[kCeThreads / 64], red_s[kCeThreads / 64];
+  __shared__ float lse_all;
   constexpr int kEpc = 16 / sizeof(T);
   const int tid = threadIdx.x;
   const int64_t r = blockIdx.x;
@@ -377,15 +390,11 @@ __global__ __launch_bounds__(kCeThreads) void cross_entropy_fwd_kernel(
   const int head = (int)((uintptr_t)row & 15) / (int)sizeof(T);
   const T* base = row - head;  // 16-byte aligned
   const int n_chunks = (head + width + kEpc - 1) / kEpc;
+  constexpr int kCeKeep = ce_keep<T>();
+  static_assert(kCeKeep % kCeInFlight == 0, "whole groups");
   float m = -INFINITY, s = 0.f;
-  for (int c0 = tid; c0 < n_chunks; c0 += kCeThreads * kCeInFlight) {
-    Vec16<T> v[kCeInFlight];
-#pragma unroll
-    for (int u = 0; u < kCeInFlight; ++u) {
-      const int c = c0 + u * kCeThreads;
-      v[u] = Vec16<T>{};
-      if (c < n_chunks) v[u] = load16_stream(base + c * kEpc);
-    }
+  // one group of kCeInFlight chunks: the running maximum and sum take them in
+  auto take_group = [&](int c0, const Vec16<T>* v) {
     float f[kCeInFlight][kEpc];
     float mx = -INFINITY;
 #pragma unroll
@@ -408,6 +417,31 @@ __global__ __launch_bounds__(kCeThreads) void cross_entropy_fwd_kernel(
 #pragma unroll
         for (int e = 0; e < kEpc; ++e) s += __expf(f[u][e] - m);
     }
+  };
+  Vec16<T> keep[MODE == 2 ? kCeKeep : 1];
+  if constexpr (MODE == 2) {
+#pragma unroll
+    for (int i = 0; i < kCeKeep; ++i) {  // every load of the row is in flight at once
+      const int c = tid + i * kCeThreads;
+      keep[i] = Vec16<T>{};
+      if (c < n_chunks) keep[i] = load16_stream(base + c * kEpc);
+    }
+#pragma unroll
+    for (int gq = 0; gq < kCeKeep / kCeInFlight; ++gq) {
+      const int c0 = tid + gq * kCeInFlight * kCeThreads;
+      if (c0 < n_chunks) take_group(c0, keep + gq * kCeInFlight);
+    }
+  } else {
+    for (int c0 = tid; c0 < n_chunks; c0 += kCeThreads * kCeInFlight) {
+      Vec16<T> v[kCeInFlight];
+#pragma unroll
+      for (int u = 0; u < kCeInFlight; ++u) {
+        const int c = c0 + u * kCeThreads;
+        v[u] = Vec16<T>{};
+        if (c < n_chunks) v[u] = MODE == 1 ? load16(base + c * kEpc) : load16_stream(base + c * kEpc);
+      }
+      take_group(c0, v);
+    }
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -429,7 +463,51 @@ __global__ __launch_bounds__(kCeThreads) void cross_entropy_fwd_kernel(
     if (!ok) atomicOr(error_flag, 1);
     row_lse[r] = lse;
     row_loss[r] = ok ? lse - (float)row[t] : 0.f;
+    if (MODE != 0) lse_all = lse;
   }
+  if constexpr (MODE != 0) {
+    __syncthreads();
+    const float lse = lse_all;
+    const int64_t t = targets[r];
+    T* obase = dlogits + r * width - head;  // the chunk grid of the input row
+    // 16-byte stores need the output row at the input row's offset from a 16-byte boundary
+    const bool same_phase = (((uintptr_t)(dlogits + r * width)) & 15) == ((uintptr_t)row & 15);
+    auto write_chunk = [&](int c, const Vec16<T>& v) {
+      const int lo = c * kEpc - head;  // row position of element 0
+      Vec16<T> o;
+#pragma unroll
+      for (int e = 0; e < kEpc; ++e) {
+        const float pr = __expf((float)v.e[e] - lse);
+        o.e[e] = (T)((pr - (t == lo + e ? 1.0f : 0.0f)) * inv_n);
+      }
+      if (same_phase && lo >= 0 && lo + kEpc <= width) {
+        store16_stream(o, obase + c * kEpc);
+      } else {  // an edge chunk shares its 16 bytes with the neighbouring row
+#pragma unroll
+        for (int e = 0; e < kEpc; ++e)
+          if (lo + e >= 0 && lo + e < width) obase[c * kEpc + e] = o.e[e];
+      }
+    };
+    if constexpr (MODE == 2) {
+#pragma unroll
+      for (int i = 0; i < kCeKeep; ++i) {
+        const int c = tid + i * kCeThreads;
+        if (c < n_chunks) write_chunk(c, keep[i]);
+      }
+    } else {
+      for (int c = tid; c < n_chunks; c += kCeThreads) write_chunk(c, load16(base + c * kEpc));
+    }
+  }
+}
+
+// x *= *factor, skipped where the factor is one (the gradient of a loss that is the root of
+// the graph): every block reads the factor and leaves.
+template <typename T>
+__global__ __launch_bounds__(256) void scale_by_device_scalar_kernel(T* x, int64_t n, const float* factor) {
+  const float f = *factor;
+  if (f == 1.0f) return;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    x[i] = (T)((float)x[i] * f);
 }
 
 // loss = scale * sum(row_loss), additions in a fixed order
@@ -707,17 +785,41 @@ void launch_argmax_rows(int dtype_f16, const void* x, int64_t* out, int64_t oute
 }
 
 void launch_cross_entropy_fwd(int dtype_f16, const void* logits, const int64_t* targets, float* row_lse,
-                              float* row_loss, float* loss, int64_t n_rows, int width, int* flag,
-                              hipStream_t stream) {
-  LaunchScope scope("cross_entropy_fwd", stream);
-  if (dtype_f16)
-    hipLaunchKernelGGL(cross_entropy_fwd_kernel<half_t>, dim3((unsigned)n_rows), dim3(kCeThreads), 0,
-                       stream, (const half_t*)logits, targets, row_lse, row_loss, width, flag);
-  else
-    hipLaunchKernelGGL(cross_entropy_fwd_kernel<float>, dim3((unsigned)n_rows), dim3(kCeThreads), 0,
-                       stream, (const float*)logits, targets, row_lse, row_loss, width, flag);
+                              float* row_loss, float* loss, void* dlogits, int64_t n_rows, int width,
+                              int* flag, hipStream_t stream) {
+  LaunchScope scope(dlogits ? "cross_entropy_fwd_grad" : "cross_entropy_fwd", stream);
+  const float inv_n = (float)(1.0 / (double)n_rows);
+  const dim3 grid((unsigned)n_rows), block(kCeThreads);
+  // a row and its possible lead-in fit the registers of a workgroup?
+  const bool resident = (int64_t)width + 16 <= (int64_t)kCeThreads * (dtype_f16 ? ce_keep<half_t>() * 8 : ce_keep<float>() * 4);
+  auto go = [&](auto kernel, auto* x, auto* dx) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, x, targets, row_lse, row_loss, dx, inv_n, width, flag);
+  };
+  if (dtype_f16) {
+    const half_t* x = (const half_t*)logits;
+    half_t* dx = (half_t*)dlogits;
+    if (!dlogits) go(cross_entropy_fwd_kernel<half_t, 0>, x, dx);
+    else if (resident) go(cross_entropy_fwd_kernel<half_t, 2>, x, dx);
+    else go(cross_entropy_fwd_kernel<half_t, 1>, x, dx);
+  } else {
+    const float* x = (const float*)logits;
+    float* dx = (float*)dlogits;
+    if (!dlogits) go(cross_entropy_fwd_kernel<float, 0>, x, dx);
+    else if (resident) go(cross_entropy_fwd_kernel<float, 2>, x, dx);
+    else go(cross_entropy_fwd_kernel<float, 1>, x, dx);
+  }
   hipLaunchKernelGGL(mean_rows_kernel, dim3(1), dim3(256), 0, stream, row_loss, n_rows,
                      (float)(1.0 / (double)n_rows), loss);
+}
+
+void launch_scale_by_device_scalar(int dtype_f16, void* x, int64_t n, const float* factor, hipStream_t stream) {
+  LaunchScope scope("scale_by_scalar", stream);
+  if (dtype_f16)
+    hipLaunchKernelGGL(scale_by_device_scalar_kernel<half_t>, dim3(stream_grid(n)), dim3(256), 0, stream,
+                       (half_t*)x, n, factor);
+  else
+    hipLaunchKernelGGL(scale_by_device_scalar_kernel<float>, dim3(stream_grid(n)), dim3(256), 0, stream,
+                       (float*)x, n, factor);
 }
 
 void launch_cross_entropy_bwd(int dtype_f16, const void* logits, const int64_t* targets,

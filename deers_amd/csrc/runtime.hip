@@ -65,9 +65,10 @@ void launch_relu_sq(int dtype_f16, const void* x, const void* dy, void* out, int
                     hipStream_t stream);
 void launch_argmax_rows(int dtype_f16, const void* x, int64_t* out, int64_t outer, int width,
                         hipStream_t stream);
+void launch_scale_by_device_scalar(int dtype_f16, void* x, int64_t n, const float* factor, hipStream_t stream);
 void launch_cross_entropy_fwd(int dtype_f16, const void* logits, const int64_t* targets, float* row_lse,
-                              float* row_loss, float* loss, int64_t n_rows, int width, int* flag,
-                              hipStream_t stream);
+                              float* row_loss, float* loss, void* dlogits, int64_t n_rows, int width,
+                              int* flag, hipStream_t stream);
 void launch_cross_entropy_bwd(int dtype_f16, const void* logits, const int64_t* targets,
                               const float* row_lse, const float* upstream, void* dlogits,
                               int64_t n_rows, int width, hipStream_t stream);
@@ -1091,20 +1092,47 @@ int deers_rocm_argmax_rows(int dtype, const void* x, int64_t* out, int64_t outer
   return DEERS_ROCM_OK;
 }
 
-int deers_rocm_cross_entropy_fwd(int dtype, const void* logits, const int64_t* targets,
-                                 float* row_lse, float* loss, int64_t n_rows, int64_t n_classes) {
-  std::lock_guard<std::mutex> lock(g_mu);
+// the forward, and with dlogits also the gradient for an upstream gradient of one; the caller holds g_mu
+static int cross_entropy_fwd_locked(const char* what, int dtype, const void* logits, const int64_t* targets,
+                                    float* row_lse, float* loss, void* dlogits, int64_t n_rows,
+                                    int64_t n_classes) {
   NEED_INIT();
-  if (int rc = rows_check("cross_entropy_fwd", dtype, n_rows, n_classes)) return rc;
-  if (n_rows < 1) return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_fwd: needs at least one row");
-  if (!logits || !targets || !row_lse || !loss)
-    return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_fwd: null pointer");
+  if (int rc = rows_check(what, dtype, n_rows, n_classes)) return rc;
+  if (n_rows < 1) return fail(DEERS_ROCM_ERR_ARG, "%s: needs at least one row", what);
+  if (!logits || !targets || !row_lse || !loss) return fail(DEERS_ROCM_ERR_ARG, "%s: null pointer", what);
   void* ws = nullptr;  // per-row losses
   if (int rc = workspace((size_t)n_rows * sizeof(float), &ws)) return rc;
   int* flag = nullptr;
   if (int rc = index_flag(&flag)) return rc;
-  deers::launch_cross_entropy_fwd(dtype == DEERS_ROCM_F16, logits, targets, row_lse, (float*)ws, loss,
+  deers::launch_cross_entropy_fwd(dtype == DEERS_ROCM_F16, logits, targets, row_lse, (float*)ws, loss, dlogits,
                                   n_rows, (int)n_classes, flag, g_rt.stream);
+  HIP_TRY(hipGetLastError());
+  return DEERS_ROCM_OK;
+}
+
+int deers_rocm_cross_entropy_fwd(int dtype, const void* logits, const int64_t* targets,
+                                 float* row_lse, float* loss, int64_t n_rows, int64_t n_classes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return cross_entropy_fwd_locked("cross_entropy_fwd", dtype, logits, targets, row_lse, loss, nullptr, n_rows,
+                                  n_classes);
+}
+
+int deers_rocm_cross_entropy_fwd_grad(int dtype, const void* logits, const int64_t* targets, float* row_lse,
+                                      float* loss, void* dlogits, int64_t n_rows, int64_t n_classes) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!dlogits) return fail(DEERS_ROCM_ERR_ARG, "cross_entropy_fwd_grad: null pointer");
+  return cross_entropy_fwd_locked("cross_entropy_fwd_grad", dtype, logits, targets, row_lse, loss, dlogits,
+                                  n_rows, n_classes);
+}
+
+int deers_rocm_scale_by_scalar(int dtype, void* x, int64_t n, const float* factor) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  NEED_INIT();
+  if (int rc = check_dtype(dtype)) return rc;
+  if (n < 0) return fail(DEERS_ROCM_ERR_ARG, "scale_by_scalar: negative element count");
+  if (n == 0) return DEERS_ROCM_OK;
+  if (!x || !factor) return fail(DEERS_ROCM_ERR_ARG, "scale_by_scalar: null pointer");
+  deers::launch_scale_by_device_scalar(dtype == DEERS_ROCM_F16, x, n, factor, g_rt.stream);
   HIP_TRY(hipGetLastError());
   return DEERS_ROCM_OK;
 }

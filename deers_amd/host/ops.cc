@@ -402,9 +402,18 @@ Tensor CrossEntropy::forward(std::unique_ptr<CrossEntropy> self) {
   const int64_t n = x.shape()[0], v = x.shape()[1];
   Tensor loss = empty({1}, DType::F32, backed(x));
   self->row_lse_ = empty({n}, DType::F32, backed(x));
-  if (backed(x))
+  if (backed(x) && x.requires_grad()) {
+    // A loss that will be differentiated: the forward also writes the gradient for an upstream
+    // gradient of one (what Tensor::backward seeds, src/backprop.rs:52-66) while each row is
+    // still in the caches; the backward then only applies the upstream factor.
+    self->grad_for_one_ = empty(x.shape(), x.dtype(), true);
+    check(deers_rocm_cross_entropy_fwd_grad((int)x.dtype(), x.data(), (const int64_t*)self->targets_.data(),
+                                            (float*)self->row_lse_.data(), (float*)loss.data(),
+                                            self->grad_for_one_.data(), n, v));
+  } else if (backed(x)) {
     check(deers_rocm_cross_entropy_fwd((int)x.dtype(), x.data(), (const int64_t*)self->targets_.data(),
                                        (float*)self->row_lse_.data(), (float*)loss.data(), n, v));
+  }
   return Tensor(loss.storage(), loss.layout(), false, std::move(self));
 }
 void CrossEntropy::backward(GradientStore& grads, const Tensor& out_grad) const {
@@ -413,6 +422,16 @@ void CrossEntropy::backward(GradientStore& grads, const Tensor& out_grad) const 
     throw std::logic_error("cross_entropy: the upstream gradient is one f32 value");
   const Tensor up = out_grad.compact();
   const Tensor& x = logits_;
+  if (grad_for_one_.defined()) {
+    // the first backward takes the gradient the forward wrote; a second one (the graph kept and
+    // differentiated again) recomputes, since the first may have scaled the buffer
+    Tensor dx = std::move(grad_for_one_);
+    grad_for_one_ = Tensor();
+    check(deers_rocm_scale_by_scalar((int)x.dtype(), const_cast<void*>(dx.data()), (int64_t)dx.layout().size(),
+                                     (const float*)up.data()));
+    grads.accumulate(logits_, dx);
+    return;
+  }
   Tensor dx = empty(x.shape(), x.dtype(), backed(x));
   if (backed(x))
     check(deers_rocm_cross_entropy_bwd((int)x.dtype(), x.data(), (const int64_t*)targets_.data(),

@@ -222,6 +222,9 @@ class CrossEntropy : public TensorOp {
  private:
   Tensor logits_, targets_;
   Tensor row_lse_;  // [N] f32, set by forward
+  // d loss / d logits for an upstream gradient of one, written by a forward whose logits carry
+  // a gradient; handed over (and released here) by the first backward
+  mutable Tensor grad_for_one_;
 };
 Tensor cross_entropy(const Tensor& logits, const Tensor& targets);
 

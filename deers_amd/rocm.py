@@ -312,6 +312,16 @@ def cross_entropy_fwd_raw(dtype, logits, targets, row_lse, loss, n_rows, n_class
                                                loss, ctypes.c_int64(n_rows), ctypes.c_int64(n_classes)))
 
 
+def cross_entropy_fwd_grad_raw(dtype, logits, targets, row_lse, loss, dlogits, n_rows, n_classes):
+    _check(load().deers_rocm_cross_entropy_fwd_grad(ctypes.c_int(dtype_code(dtype)), logits, targets, row_lse,
+                                                    loss, dlogits, ctypes.c_int64(n_rows),
+                                                    ctypes.c_int64(n_classes)))
+
+
+def scale_by_scalar_raw(dtype, x, n, factor):
+    _check(load().deers_rocm_scale_by_scalar(ctypes.c_int(dtype_code(dtype)), x, ctypes.c_int64(n), factor))
+
+
 def cross_entropy_bwd_raw(dtype, logits, targets, row_lse, upstream, dlogits, n_rows, n_classes):
     _check(load().deers_rocm_cross_entropy_bwd(ctypes.c_int(dtype_code(dtype)), logits, targets, row_lse,
                                                upstream, dlogits, ctypes.c_int64(n_rows),

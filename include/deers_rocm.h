@@ -410,6 +410,18 @@ int deers_rocm_cross_entropy_fwd(int dtype, const void* logits, const int64_t* t
 int deers_rocm_cross_entropy_bwd(int dtype, const void* logits, const int64_t* targets,
                                  const float* row_lse, const float* upstream, void* dlogits,
                                  int64_t n_rows, int64_t n_classes);
+/* deers_rocm_cross_entropy_fwd that also writes dlogits = (softmax(logits) - onehot(targets)) / n_rows,
+ * what deers_rocm_cross_entropy_bwd gives for an upstream gradient of one (same bits), while the
+ * row it has just reduced is still in the caches: one pass over the logits less than the two
+ * calls.  For the loss of a training step, whose gradient is the seed of the reverse sweep
+ * (src/backprop.rs:52-66, Tensor::backward seeds ones); another upstream gradient is applied
+ * afterwards with deers_rocm_scale_by_scalar. */
+int deers_rocm_cross_entropy_fwd_grad(int dtype, const void* logits, const int64_t* targets, float* row_lse,
+                                      float* loss, void* dlogits, int64_t n_rows, int64_t n_classes);
+/* x[i] *= *factor, with the factor in device memory (a scalar tensor such as the gradient of a
+ * loss); a launch that finds the factor equal to one leaves x untouched and costs a few
+ * microseconds.  ScalarMul by a tensor-valued scalar (src/ops.rs:638-643) without a host read. */
+int deers_rocm_scale_by_scalar(int dtype, void* x, int64_t n, const float* factor);
 
 /* ---- optimizer step ---------------------------------------------------------------
  * One AdamW update of one parameter tensor in place, the body of the loop in

@@ -149,7 +149,8 @@ def test_relu_sq_is_bit_exact(dtype, n, skew):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("n,v", [(2, 3), (6, 8), (7, 33), (5, 2049), (64, 256), (3, 8200), (16, 50257)])
+@pytest.mark.parametrize("n,v", [(2, 3), (6, 8), (7, 33), (5, 2049), (64, 256), (3, 8200), (16, 50257),
+                                 (2, 70001)])  # the last one is longer than a workgroup's registers hold
 def test_cross_entropy_fwd_bwd(dtype, n, v):
     x = synth.normal((n, v), synth.tensor_seed(74, "ce", "x"), 3.0).astype(dtype)
     t = _tokens(n, v, 74, repeats=False)
@@ -176,6 +177,24 @@ def test_cross_entropy_fwd_bwd(dtype, n, v):
     assert np.abs(d.numpy().astype(np.float32) - oracle.cross_entropy_bwd(x32, t)).max() <= tol
     if dtype == np.float32:
         assert np.abs(d.numpy().astype(np.float64).sum(axis=1)).max() < 1e-6
+    # the forward that also writes the gradient for an upstream gradient of one: the forward's
+    # loss and row statistics, the backward's bits
+    lse2, loss2 = rocm.DeviceBuffer((n,), np.float32), rocm.DeviceBuffer((1,), np.float32)
+    d2 = _dev(np.full((n, v), 9.0, dtype=dtype))
+    rocm.cross_entropy_fwd_grad_raw(dtype, bx.ptr, bt.ptr, lse2.ptr, loss2.ptr, d2.ptr, n, v)
+    assert np.array_equal(lse2.numpy(), lse.numpy()) and np.array_equal(loss2.numpy(), loss.numpy())
+    assert np.array_equal(d2.numpy(), d.numpy())
+    # the upstream factor afterwards: one leaves the bits, another multiplies and rounds once
+    one, f07 = _dev(np.float32([1.0])), _dev(np.float32([0.7]))
+    rocm.scale_by_scalar_raw(dtype, d2.ptr, n * v, one.ptr)
+    assert np.array_equal(d2.numpy(), d.numpy())
+    rocm.scale_by_scalar_raw(dtype, d2.ptr, n * v, f07.ptr)
+    # (the f16 product may be rounded from the exact value or from its f32 rounding: the two differ
+    # only on ties)
+    got = d2.numpy()
+    once = (d.numpy().astype(np.float64) * np.float64(np.float32(0.7))).astype(dtype)
+    twice = (d.numpy().astype(np.float32) * np.float32(0.7)).astype(dtype)
+    assert np.all((got == once) | (got == twice))
 
 
 @pytest.mark.gpu
@@ -199,6 +218,11 @@ def test_cross_entropy_views_and_bad_target():
         got = d.numpy()
         assert np.abs(got[skew_out:skew_out + n * v].reshape(n, v) - want).max() < 1e-6
         assert (got[:skew_out] == 9).all() and (got[skew_out + n * v:] == 9).all()
+        # the gradient-writing forward on the same views: same bits, nothing outside them
+        d2 = _dev(np.full(n * v + 16, 9.0, dtype=np.float32))
+        lse2, loss2 = rocm.DeviceBuffer((n,), np.float32), rocm.DeviceBuffer((1,), np.float32)
+        rocm.cross_entropy_fwd_grad_raw(np.float32, at(bx, 3), bt.ptr, lse2.ptr, loss2.ptr, at(d2, skew_out), n, v)
+        assert np.array_equal(d2.numpy(), got) and np.array_equal(lse2.numpy(), lse.numpy())
     # a target out of range is reported at the next sync and contributes zero loss
     rocm.sync()
     t_bad = t.copy()
